@@ -1,0 +1,124 @@
+"""Engine configuration: model, cache and scheduler sections, YAML and key=value overrides.
+
+Same sections and field names as the reference (clockwork/config.py:17-87); the
+reference's ``attention_backend`` is gone (there is one backend: the HIP kernels)
+and the scheduler gains the chunked-prefill knobs.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field, fields
+from pathlib import Path
+
+import yaml
+
+_DTYPES = ("float32", "bfloat16")
+
+
+@dataclass
+class ModelConfig:
+    """Which model folder to serve and how (clockwork/config.py:17-31)."""
+
+    model: str
+    dtype: str = "float32"
+    device: str = "cuda"
+    max_model_len: int = 4096
+    seed: int = 0
+    trust_remote_code: bool = False
+
+    def torch_dtype(self):
+        import torch
+
+        if self.dtype == "float16":
+            raise ValueError(
+                "dtype 'float16' is not built in this engine; use 'bfloat16' or 'float32'"
+            )
+        if self.dtype not in _DTYPES:
+            raise ValueError(f"unknown dtype {self.dtype!r}, expected one of {_DTYPES}")
+        return getattr(torch, self.dtype)
+
+
+@dataclass
+class CacheConfig:
+    """Paged cache sizing (clockwork/config.py:34-39). ``num_blocks`` is pages per layer group."""
+
+    block_size: int = 16
+    num_blocks: int = 512
+    enable_prefix_cache: bool = True
+    watermark: float = 0.01
+
+
+@dataclass
+class SchedulerConfig:
+    """Batching limits (clockwork/config.py:42-47) plus chunked prefill.
+
+    ``max_prefill_chunk`` caps the tokens one request contributes to a step;
+    0 means "as many as the token budget allows". With
+    ``enable_chunked_prefill`` off a prompt is admitted only whole, as in the
+    reference (clockwork/scheduler/scheduler.py:120-146).
+    """
+
+    max_num_seqs: int = 64
+    max_num_batched_tokens: int = 2048
+    max_model_len: int = 4096
+    preemption_mode: str = "recompute"
+    enable_chunked_prefill: bool = True
+    max_prefill_chunk: int = 0
+
+
+_SECTIONS = ("model", "cache", "scheduler")
+
+
+@dataclass
+class EngineConfig:
+    model: ModelConfig
+    cache: CacheConfig = field(default_factory=CacheConfig)
+    scheduler: SchedulerConfig = field(default_factory=SchedulerConfig)
+
+    @classmethod
+    def from_yaml(cls, path: str | Path) -> "EngineConfig":
+        """Read sections ``model:``, ``cache:``, ``scheduler:`` (clockwork/config.py:57-68)."""
+        data = yaml.safe_load(Path(path).read_text(encoding="utf-8")) or {}
+        model = data.get("model")
+        if not isinstance(model, dict) or "model" not in model:
+            raise ValueError(f"{path}: expected a top-level 'model' section naming the model")
+        unknown = sorted(set(data) - set(_SECTIONS) - {"attention_backend"})
+        if unknown:
+            raise ValueError(f"{path}: unknown top-level sections {unknown}")
+        return cls(
+            model=ModelConfig(**model),
+            cache=CacheConfig(**(data.get("cache") or {})),
+            scheduler=SchedulerConfig(**(data.get("scheduler") or {})),
+        )
+
+    @classmethod
+    def defaults(cls, model: str, **overrides) -> "EngineConfig":
+        """Defaults plus keyword overrides routed by field name (clockwork/config.py:70-87)."""
+        cfg = cls(model=ModelConfig(model=model))
+        for key, value in overrides.items():
+            cfg.set(key, value)
+        return cfg
+
+    def set(self, key: str, value) -> None:
+        """Set ``key`` on every section that has such a field; unknown keys are an error.
+
+        ``max_model_len`` lives on both the model and the scheduler section and
+        is set on both, as in the reference (clockwork/config.py:76-86).
+        """
+        targets = [
+            sub
+            for sub in (self.model, self.cache, self.scheduler)
+            if key in {f.name for f in fields(sub)}
+        ]
+        if not targets:
+            raise ValueError(f"unknown config override {key!r}")
+        for sub in targets:
+            setattr(sub, key, value)
+
+    def apply_overrides(self, pairs: list[str]) -> None:
+        """``KEY=VALUE`` strings, the value read as YAML (scripts/serve.py:13-30)."""
+        for pair in pairs:
+            if "=" not in pair:
+                raise ValueError(f"override {pair!r} is not KEY=VALUE")
+            key, raw = pair.split("=", 1)
+            self.set(key, yaml.safe_load(raw))

@@ -1,0 +1,138 @@
+"""Architecture-neutral description of a decoder: what the parts and the cache are built from.
+
+An architecture module (``clockwork_amd.models.*``) reads its own ``config.json``
+keys into a typed configuration and turns that into a :class:`ModelSpec`. Nothing
+below this line knows a model's name: parts see only their own spec, the cache
+manager sees only :class:`KVPagesSpec` / :class:`StateSpec`, and the order in which
+layers run is the ``run`` list.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Optional, Sequence
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One tensor a part owns.
+
+    ``precision``:
+      * ``"compute"`` - cast to the engine's dtype (bfloat16 or float32);
+      * ``"stored"``  - like ``"compute"``, but a tensor the checkpoint holds in
+        float32 stays float32 (small vectors: norm weights, biases);
+      * ``"float32"`` / ``"int32"`` - always that type.
+    ``init`` names the random-weights distribution: ``("normal", std)``,
+    ``("one_plus_uniform", half_width)`` or ``("zeros",)``.
+    """
+
+    shape: tuple[int, ...]
+    precision: str = "compute"
+    init: tuple = ("normal", 0.02)
+
+
+@dataclass(frozen=True)
+class KVPagesSpec:
+    """A mixer that keeps keys and values of earlier tokens in pages.
+
+    ``window`` None: every earlier token is read, pages live as long as the
+    request. ``window`` W: a token reads itself and the W-1 tokens before it;
+    pages wholly behind the window are given back while the request runs.
+    Mixers whose (kv_heads, head_dim, window) agree share a layer group and
+    therefore a block table.
+    """
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+    def group_key(self) -> tuple:
+        return ("kv", self.num_kv_heads, self.head_dim, self.window)
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """A mixer that keeps a fixed-size state per request (a recurrence, a convolution tail).
+
+    One slot of ``shape``/``dtype`` per live request and per run entry; zeroed
+    when a request's first token arrives.
+    """
+
+    shape: tuple[int, ...]
+    dtype: str = "float32"
+
+    def group_key(self) -> tuple:
+        return ("state", self.shape, self.dtype)
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    """One block: which parts it is made of and how they are wired.
+
+    ``arrangement`` names an entry of the arrangement registry ("prenorm":
+    x + mixer(norm(x)), then x + ffn(norm(x))). ``mixer``, ``feed_forward`` and
+    the norms are specs of registered part kinds; different layers of one model
+    may hold different kinds.
+    """
+
+    arrangement: str
+    mixer: Any
+    feed_forward: Any
+    mixer_norm: Any
+    ffn_norm: Any
+
+
+@dataclass(frozen=True)
+class RunEntry:
+    """One step of the forward pass: run ``layer`` (an index into ``ModelSpec.layers``).
+
+    A layer may appear in several entries (its weights are then shared; each
+    entry still has a cache of its own). ``cache_from`` names an *earlier entry*
+    whose cache this entry reads instead of writing its own.
+    """
+
+    layer: int
+    cache_from: Optional[int] = None
+
+
+@dataclass
+class ModelSpec:
+    architecture: str
+    vocab_size: int
+    hidden_size: int
+    layers: Sequence[LayerSpec]
+    run: Sequence[RunEntry]
+    final_norm: Any
+    tie_embeddings: bool = False
+    eos_token_ids: tuple[int, ...] = ()
+    # free-form facts for reporting (bench config lines and the like), never read by parts
+    info: dict = field(default_factory=dict)
+
+    def validate(self) -> None:
+        if not self.layers:
+            raise ValueError("a model needs at least one layer")
+        if not self.run:
+            raise ValueError("the run list is empty")
+        for i, entry in enumerate(self.run):
+            if not 0 <= entry.layer < len(self.layers):
+                raise ValueError(f"run[{i}] names layer {entry.layer}, model has {len(self.layers)}")
+            if entry.cache_from is not None:
+                if not 0 <= entry.cache_from < i:
+                    raise ValueError(f"run[{i}].cache_from={entry.cache_from} must name an earlier entry")
+                if self.run[entry.cache_from].cache_from is not None:
+                    raise ValueError(f"run[{i}].cache_from names an entry that itself borrows a cache")
+
+
+@dataclass(frozen=True)
+class WeightTarget:
+    """How one parameter of the model is filled from checkpoint tensors.
+
+    ``sources`` are tensor names in the checkpoint with their expected shapes;
+    several sources are concatenated along dim 0 (fused projections).
+    ``optional`` sources may be absent (a tied output head).
+    """
+
+    param: str
+    sources: tuple[str, ...]
+    source_shapes: tuple[tuple[int, ...], ...]
+    optional: bool = False

@@ -1,0 +1,55 @@
+// Shared definitions for the gfx950 kernels: element types, error codes, small device helpers.
+// Every entry point is extern "C", takes raw device pointers and a hipStream_t, launches
+// asynchronously on that stream and returns 0, or a negative code without launching anything.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#define CW_OK 0
+#define CW_ERR_ARG -1      // a size or pointer the kernel does not take
+#define CW_ERR_DTYPE -2    // unknown element type code
+#define CW_ERR_LAUNCH -3   // the HIP runtime refused the launch
+#define CW_ERR_SIZE -4     // beyond a stated maximum
+
+#define CW_F32 0
+#define CW_BF16 1
+
+#define CW_EXPORT extern "C" __attribute__((visibility("default")))
+
+typedef __hip_bfloat16 bf16_t;
+
+__device__ __forceinline__ float cw_to_float(float x) { return x; }
+__device__ __forceinline__ float cw_to_float(bf16_t x) { return __bfloat162float(x); }
+
+template <typename T> __device__ __forceinline__ T cw_from_float(float x);
+template <> __device__ __forceinline__ float cw_from_float<float>(float x) { return x; }
+template <> __device__ __forceinline__ bf16_t cw_from_float<bf16_t>(float x) { return __float2bfloat16(x); }
+
+// bfloat16 bits <-> float without going through the class type (for packed 16-byte loads)
+__device__ __forceinline__ float cw_bf16_bits_to_float(uint16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+__device__ __forceinline__ uint16_t cw_float_to_bf16_bits(float f) {
+  // round to nearest even; NaN stays NaN
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float cw_wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float cw_wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+static inline int cw_launch_status() {
+  return hipGetLastError() == hipSuccess ? CW_OK : CW_ERR_LAUNCH;
+}

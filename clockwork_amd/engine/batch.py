@@ -1,0 +1,195 @@
+"""One step's batch: which request contributes which tokens, laid out for the kernels.
+
+A step holds R requests; request r contributes q_len[r] >= 1 consecutive tokens
+starting at position start[r]: a portion of a prompt, a whole prompt, or one decoded
+token. All index arrays are packed into one pinned int32 buffer and go to the GPU
+in a single copy; the kernels read device views of that buffer.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    """Next tokens of one request. ``want``: indices into ``tokens`` whose logits are asked for."""
+
+    seq_id: str
+    start: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class AttentionPlan:
+    """Work items of the attention kernels for one head geometry (see csrc/attention.hip).
+
+    Requests with one token go to the 16-row kernel, cut over their keys into
+    ``single_splits`` parts; longer portions are cut into tiles of the 64-row kernel."""
+
+    wide_items: Optional[torch.Tensor] = None
+    n_wide: int = 0
+    gh_wide: int = 1
+    single_items: Optional[torch.Tensor] = None
+    n_single: int = 0
+    gh_single: int = 1
+    chunks_single: int = 1
+    single_splits: int = 1
+
+
+class _Packer:
+    def __init__(self) -> None:
+        self.parts: list[np.ndarray] = []
+        self.offsets: list[tuple[int, int]] = []
+        self.size = 0
+
+    def add(self, values) -> int:
+        a = np.asarray(values, dtype=np.int32).reshape(-1)
+        pad = (-self.size) % 4  # keep every array 16-byte aligned
+        if pad:
+            self.parts.append(np.zeros(pad, dtype=np.int32))
+            self.size += pad
+        self.offsets.append((self.size, a.size))
+        self.parts.append(a)
+        self.size += a.size
+        return len(self.offsets) - 1
+
+    def upload(self, device) -> list[torch.Tensor]:
+        host = torch.empty(max(self.size, 1), dtype=torch.int32, pin_memory=True)
+        if self.size:
+            host.numpy()[: self.size] = np.concatenate(self.parts)
+        dev = host.to(device, non_blocking=True)
+        self._host = host  # keep the pinned buffer alive until the copy has run
+        return [dev[o : o + n] for o, n in self.offsets]
+
+
+class StepContext:
+    """Everything a part may ask about the step. Built by :func:`build_context`."""
+
+    def __init__(self) -> None:
+        self.num_tokens = 0
+        self.num_requests = 0
+        self.num_logit_rows = 0
+        self.device = None
+        self.block_size = 0
+        # device int32 tensors
+        self.token_ids = None
+        self.positions = None
+        self.cu_q = None          # [R + 1]
+        self.ctx_lens = None      # [R]  keys of each request once this step's tokens are cached
+        self.starts = None        # [R]  position of each request's first token in this step
+        self.state_slots = None   # [R]
+        self.logit_rows = None    # [num_logit_rows] rows of the flat batch
+        self.slots: list[torch.Tensor] = []         # per kv group [T]
+        self.block_tables: list[torch.Tensor] = []  # per kv group [R, max_blocks]
+        # host copies for planning
+        self.h_q_lens: list[int] = []
+        self.h_ctx_lens: list[int] = []
+        self.h_starts: list[int] = []
+        self.seq_ids: list[str] = []
+        self._plans: dict = {}
+        self.num_compute_units = 256
+
+    def attention_plan(self, nh: int, nkv: int) -> AttentionPlan:
+        key = (nh, nkv)
+        plan = self._plans.get(key)
+        if plan is None:
+            plan = self._plans[key] = self._make_plan(nh, nkv)
+        return plan
+
+    def _make_plan(self, nh: int, nkv: int) -> AttentionPlan:
+        group = nh // nkv
+        gh_wide = min(group, 64)
+        tokens_per_tile = 64 // gh_wide
+        gh_single = min(group, 16)
+        wide: list[int] = []
+        single: list[int] = []
+        longest_single = 0
+        for r, q_len in enumerate(self.h_q_lens):
+            if q_len == 1:
+                single += [r, 0, 1, 0]
+                longest_single = max(longest_single, self.h_ctx_lens[r])
+            else:
+                for tok0 in range(0, q_len, tokens_per_tile):
+                    wide += [r, tok0, min(tokens_per_tile, q_len - tok0), 0]
+        plan = AttentionPlan(gh_wide=gh_wide, gh_single=gh_single)
+        plan.n_wide, plan.n_single = len(wide) // 4, len(single) // 4
+        plan.chunks_single = -(-group // gh_single)
+        if plan.n_single:
+            groups_running = plan.n_single * nkv * plan.chunks_single
+            by_occupancy = -(-4 * self.num_compute_units // groups_running)
+            by_length = max(1, longest_single // 256)
+            plan.single_splits = max(1, min(by_occupancy, by_length, 64))
+        packer = _Packer()
+        packer.add(wide)
+        packer.add(single)
+        plan.wide_items, plan.single_items = packer.upload(self.device)
+        self._keep = getattr(self, "_keep", []) + [packer]
+        return plan
+
+
+def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int) -> StepContext:
+    """Lay out ``entries`` (pages already reserved through ``manager``) as one batch."""
+    ctx = StepContext()
+    ctx.device = device
+    ctx.block_size = manager.block_size
+    tokens: list[int] = []
+    positions: list[int] = []
+    cu = [0]
+    logit_rows: list[int] = []
+    state_slots: list[int] = []
+    for e in entries:
+        n = len(e.tokens)
+        if n < 1:
+            raise ValueError(f"request {e.seq_id}: a step entry needs at least one token")
+        for t in e.tokens:
+            if not 0 <= int(t) < vocab_size:
+                raise ValueError(f"request {e.seq_id}: token id {t} outside the vocabulary [0, {vocab_size})")
+        for w in e.want:
+            if not 0 <= int(w) < n:
+                raise ValueError(f"request {e.seq_id}: wanted index {w} outside its {n} tokens")
+            logit_rows.append(cu[-1] + int(w))
+        tokens += [int(t) for t in e.tokens]
+        positions += range(e.start, e.start + n)
+        cu.append(cu[-1] + n)
+        ctx.h_q_lens.append(n)
+        ctx.h_starts.append(e.start)
+        ctx.h_ctx_lens.append(e.start + n)
+        ctx.seq_ids.append(e.seq_id)
+        state_slots.append(manager.state_slot(e.seq_id))
+    ctx.num_tokens = cu[-1]
+    ctx.num_requests = len(entries)
+    ctx.num_logit_rows = len(logit_rows)
+
+    packer = _Packer()
+    i_tok = packer.add(tokens)
+    i_pos = packer.add(positions)
+    i_cu = packer.add(cu)
+    i_ctx = packer.add(ctx.h_ctx_lens)
+    i_start = packer.add(ctx.h_starts)
+    i_state = packer.add(state_slots)
+    i_rows = packer.add(logit_rows)
+    group_idx = []
+    for g in range(len(manager.kv_groups)):
+        slots: list[int] = []
+        width = max(1, max(-(-c // manager.block_size) for c in ctx.h_ctx_lens))
+        table = np.full((len(entries), width), -1, dtype=np.int32)
+        for r, e in enumerate(entries):
+            slots += manager.slot_mapping(e.seq_id, e.start, e.start + len(e.tokens), g)
+            row = manager.block_table(e.seq_id, g)[:width]
+            table[r, : len(row)] = row
+        group_idx.append((packer.add(slots), packer.add(table), width))
+    views = packer.upload(device)
+    ctx._packer = packer
+    ctx.token_ids, ctx.positions, ctx.cu_q = views[i_tok], views[i_pos], views[i_cu]
+    ctx.ctx_lens, ctx.starts = views[i_ctx], views[i_start]
+    ctx.state_slots, ctx.logit_rows = views[i_state], views[i_rows]
+    for i_slots, i_table, width in group_idx:
+        ctx.slots.append(views[i_slots])
+        ctx.block_tables.append(views[i_table].view(len(entries), width))
+    return ctx

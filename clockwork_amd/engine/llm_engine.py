@@ -1,0 +1,251 @@
+"""The engine loop and the Python entry point.
+
+Same surface as the reference's ``LLMEngine`` (clockwork/engine/llm_engine.py:35-242):
+``add_request``, ``step``, ``generate``, ``abort_request``, ``has_unfinished_requests``,
+``stats``. A tokenizer is optional here: token ids in, token ids out is the primary
+mode; text (prompts, stop strings, ``RequestOutput.text``) needs a tokenizer with
+``encode``/``decode``.
+"""
+
+from __future__ import annotations
+
+import itertools
+from dataclasses import dataclass
+from typing import Optional
+
+from clockwork_amd.cache.prefix import PrefixCache
+from clockwork_amd.config.engine import EngineConfig
+from clockwork_amd.engine.batch import StepEntry
+from clockwork_amd.engine.model_runner import ModelRunner
+from clockwork_amd.engine.scheduler import Scheduler
+from clockwork_amd.engine.sequence import RequestOutput, SamplingParams, Sequence, SequenceStatus
+from clockwork_amd.sampling.sampler import Sampler
+
+
+@dataclass
+class _TextState:
+    prefix_offset: int = 0
+    read_offset: int = 0
+    text: str = ""
+
+
+class LLMEngine:
+    def __init__(self, cfg: EngineConfig, tokenizer=None, runner: Optional[ModelRunner] = None,
+                 weight_source=None, config_dict: Optional[dict] = None) -> None:
+        self.cfg = cfg
+        self.runner = runner if runner is not None else ModelRunner(
+            cfg, weight_source=weight_source, config_dict=config_dict
+        )
+        self.tokenizer = tokenizer
+        self.manager = self.runner.manager
+        self.prefix_cache = PrefixCache(
+            cfg.cache.block_size,
+            share=self.manager.share_handle,
+            drop=self.manager.drop_handle,
+            enabled=cfg.cache.enable_prefix_cache and self.manager.supports_prefix_sharing,
+        )
+        self.scheduler = Scheduler(cfg.scheduler, self.manager, self.prefix_cache)
+        self.sampler = Sampler(self.runner.device, cfg.model.seed)
+        self._eos_ids = self._resolve_eos()
+        self._seqs: dict[str, Sequence] = {}
+        self._text: dict[str, _TextState] = {}
+        # arrival "times" are a counter, so order never depends on the clock (llm_engine.py:57-59)
+        self._arrivals = itertools.count()
+        self._generate_ids = itertools.count()
+
+    @classmethod
+    def from_config(cls, cfg: EngineConfig) -> "LLMEngine":
+        return cls(cfg)
+
+    def _resolve_eos(self) -> frozenset:
+        """llm_engine.py:24-32: the tokenizer's eos id, else the model config's (int or list)."""
+        eos = getattr(self.tokenizer, "eos_token_id", None)
+        if eos is None:
+            return frozenset(self.runner.spec.eos_token_ids)
+        return frozenset({eos}) if isinstance(eos, int) else frozenset(eos)
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, request_id: str, prompt: Optional[str] = None,
+                    sampling_params: Optional[SamplingParams] = None,
+                    prompt_token_ids: Optional[list[int]] = None) -> None:
+        """Queue one request; exactly one of ``prompt`` and ``prompt_token_ids`` (llm_engine.py:67-97)."""
+        if (prompt is None) == (prompt_token_ids is None):
+            raise ValueError("provide exactly one of prompt or prompt_token_ids")
+        if request_id in self._seqs:
+            raise ValueError(f"request id {request_id!r} is already active")
+        if prompt_token_ids is None:
+            if self.tokenizer is None:
+                raise ValueError("a text prompt needs a tokenizer; pass prompt_token_ids instead")
+            prompt_token_ids = self.tokenizer.encode(prompt)
+        prompt_token_ids = [int(t) for t in prompt_token_ids]
+        if not prompt_token_ids:
+            raise ValueError("prompt must contain at least one token")
+        vocab = self.runner.spec.vocab_size
+        bad = [t for t in prompt_token_ids if not 0 <= t < vocab]
+        if bad:
+            raise ValueError(f"token ids {bad[:5]} lie outside the vocabulary [0, {vocab})")
+        if len(prompt_token_ids) >= self.cfg.model.max_model_len:
+            raise ValueError(
+                f"prompt of {len(prompt_token_ids)} tokens leaves no room to generate "
+                f"within max_model_len {self.cfg.model.max_model_len}"
+            )
+        params = sampling_params if sampling_params is not None else SamplingParams()
+        if params.stop and self.tokenizer is None:
+            raise ValueError("stop strings need a tokenizer; use stop_token_ids instead")
+        seq = Sequence(request_id, prompt_token_ids, params, arrival_time=float(next(self._arrivals)))
+        self._seqs[request_id] = seq
+        self._text[request_id] = _TextState()
+        self.scheduler.add_seq(seq)
+
+    def abort_request(self, request_id: str) -> None:
+        self.scheduler.abort(request_id)
+        self._forget(request_id)
+
+    def has_unfinished_requests(self) -> bool:
+        return self.scheduler.has_unfinished()
+
+    def _forget(self, request_id: str) -> None:
+        self._seqs.pop(request_id, None)
+        self._text.pop(request_id, None)
+
+    # ------------------------------------------------------------------ one iteration
+    def step(self) -> list[RequestOutput]:
+        """Schedule, run one batch, sample, finish; an output per request that got a token
+        (llm_engine.py:99-125)."""
+        out = self.scheduler.schedule()
+        if not out.portions:
+            if out.preempted or not self.scheduler.has_unfinished():
+                return []
+            # nothing runs and the head does not fit: give it everything the prefix cache
+            # holds idle, once, before calling the request unschedulable (llm_engine.py:102-113)
+            if self.prefix_cache.evict(self.manager.num_blocks) > 0:
+                out = self.scheduler.schedule()
+            if not out.portions:
+                raise RuntimeError("waiting request cannot be admitted even with an empty prefix cache")
+        self.runner.apply_copies(out.copies)
+        entries = [
+            StepEntry(
+                p.seq.seq_id,
+                p.start,
+                p.seq.token_ids()[p.start : p.start + p.num_tokens],
+                [p.num_tokens - 1] if p.samples else [],
+            )
+            for p in out.portions
+        ]
+        logits = self.runner.step(entries)
+        sampling = [p.seq for p in out.portions if p.samples]
+        tokens = self.sampler.sample(logits, sampling) if sampling else []
+        outputs: list[RequestOutput] = []
+        drawn = iter(tokens)
+        for p in out.portions:
+            seq = p.seq
+            seq.num_computed_tokens = p.start + p.num_tokens
+            prompt_done = p.start < len(seq.prompt_token_ids) <= seq.num_computed_tokens
+            if prompt_done and self.prefix_cache.enabled:
+                # the trie takes a hold only on blocks it adopts, so inserting while the
+                # request still holds its pages is safe (llm_engine.py:115-119)
+                n_full = len(seq.prompt_token_ids) // self.cfg.cache.block_size
+                self.prefix_cache.insert(seq.prompt_token_ids, self.manager.handles(seq.seq_id, n_full))
+            if p.samples:
+                seq.append_token(next(drawn))
+                outputs.append(self._process(seq))
+        self.scheduler.free_finished()
+        for output in outputs:
+            if output.finished:
+                self._forget(output.request_id)
+        return outputs
+
+    def generate(self, prompts, sampling_params: Optional[SamplingParams] = None) -> list[RequestOutput]:
+        """Run prompts (strings or lists of token ids) to completion; final outputs in prompt order
+        (llm_engine.py:135-159)."""
+        ids = []
+        for prompt in prompts:
+            request_id = f"generate-{next(self._generate_ids)}"
+            ids.append(request_id)
+            if isinstance(prompt, str):
+                self.add_request(request_id, prompt=prompt, sampling_params=sampling_params)
+            else:
+                self.add_request(request_id, prompt_token_ids=prompt, sampling_params=sampling_params)
+        finals: dict[str, RequestOutput] = {}
+        pending = set(ids)
+        while pending:
+            outputs = self.step()
+            for output in outputs:
+                if output.finished and output.request_id in pending:
+                    finals[output.request_id] = output
+                    pending.discard(output.request_id)
+            if not outputs and not self.scheduler.has_unfinished() and pending:
+                raise RuntimeError(f"engine drained with unfinished requests: {sorted(pending)}")
+        return [finals[i] for i in ids]
+
+    def stats(self) -> dict:
+        sched, cache = self.scheduler.stats, self.prefix_cache.stats
+        return {
+            "num_waiting": sched.num_waiting,
+            "num_running": sched.num_running,
+            "num_preempted_total": sched.num_preempted_total,
+            "num_scheduled_batches": sched.num_scheduled_batches,
+            "total_prompt_tokens": sched.total_prompt_tokens,
+            "total_cached_tokens": sched.total_cached_tokens,
+            "prefix_cache_queries": cache.queries,
+            "prefix_cache_hit_tokens": cache.hit_tokens,
+            "prefix_cache_prompt_tokens": cache.prompt_tokens,
+            "prefix_cache_hit_rate": cache.hit_rate,
+            "num_free_blocks": self.manager.min_free_blocks(),
+        }
+
+    # ------------------------------------------------------------------ text and finishing
+    def _decode(self, ids: list[int]) -> str:
+        return self.tokenizer.decode(ids, skip_special_tokens=True)
+
+    def _text_step(self, seq: Sequence, state: _TextState) -> str:
+        """Incremental detokenisation; text that ends in U+FFFD is an unfinished multi-token
+        character and is held back (llm_engine.py:187-198)."""
+        ids = seq.output_token_ids
+        new_text = self._decode(ids[state.prefix_offset:])
+        if new_text.endswith("\ufffd"):
+            return ""
+        prefix_text = self._decode(ids[state.prefix_offset:state.read_offset])
+        state.prefix_offset, state.read_offset = state.read_offset, len(ids)
+        return new_text[len(prefix_text):]
+
+    def _process(self, seq: Sequence) -> RequestOutput:
+        """Finish rules (llm_engine.py:200-242): a stop token (EOS unless ignore_eos, or one of
+        stop_token_ids) stays in the ids and adds no text; a stop string cuts the text; then
+        max_tokens and max_model_len give "length"."""
+        params = seq.sampling_params
+        state = self._text[seq.seq_id]
+        token = seq.output_token_ids[-1]
+        reason = None
+        delta = ""
+        if (not params.ignore_eos and token in self._eos_ids) or token in params.stop_token_ids:
+            reason = "stop"
+        elif self.tokenizer is not None:
+            delta = self._text_step(seq, state)
+            candidate = state.text + delta
+            hits = [pos for pos in (candidate.find(s) for s in params.stop) if pos >= 0]
+            if hits:
+                candidate = candidate[: min(hits)]
+                delta = candidate[len(state.text):] if len(candidate) > len(state.text) else ""
+                reason = "stop"
+            state.text = candidate
+        if reason is None and (
+            len(seq.output_token_ids) >= params.max_tokens or len(seq) >= self.cfg.model.max_model_len
+        ):
+            reason = "length"
+        if reason == "stop":
+            seq.status = SequenceStatus.FINISHED_STOPPED
+        elif reason == "length":
+            seq.status = SequenceStatus.FINISHED_LENGTH
+        return RequestOutput(
+            request_id=seq.seq_id,
+            prompt_token_ids=list(seq.prompt_token_ids),
+            token_ids=list(seq.output_token_ids),
+            text=state.text,
+            finished=seq.is_finished(),
+            finish_reason=reason,
+            num_cached_tokens=seq.num_cached_tokens,
+            num_prompt_tokens=len(seq.prompt_token_ids),
+            num_generated_tokens=len(seq.output_token_ids),
+            delta_text=delta,
+        )

@@ -1,0 +1,245 @@
+"""Continuous batching: decode first, first-come-first-served admission, chunked prefill,
+preemption by recompute.
+
+The reference's decisions are kept (clockwork/scheduler/scheduler.py:34-204):
+
+* running requests are served before anything is admitted, in order of arrival;
+* when a running request cannot get the page it needs, the latest-arrived request
+  that has not yet been served this step is preempted (the request itself if none is
+  left): its pages go back, its progress is reset to zero, and it re-enters the
+  waiting queue in front of every request that was never admitted;
+* admission is strictly in queue order: a head that does not fit blocks the rest;
+* admitting a request must leave the cache's watermark of pages free.
+
+New here: a prompt no longer has to fit the token budget whole. A request
+contributes ``min(remaining, budget left, max_prefill_chunk)`` tokens per step, so
+running requests are either *prefilling* (more than one token still to run) or
+*decoding* (exactly one). With ``enable_chunked_prefill`` off the reference's
+behaviour returns: a prompt is admitted only whole.
+
+When pages run out: before a request is refused admission and before a running
+request is preempted, idle blocks of the prefix cache are evicted, oldest first.
+What then still does not fit waits (admission) or is preempted (running). A waiting
+head that cannot be admitted although nothing runs and nothing can be evicted is an
+error raised by the engine.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Optional
+
+from clockwork_amd.cache.manager import CacheManager
+from clockwork_amd.cache.prefix import PrefixCache, PrefixMatch
+from clockwork_amd.config.engine import SchedulerConfig
+from clockwork_amd.engine.sequence import Sequence, SequenceStatus
+
+
+@dataclass
+class ScheduledPortion:
+    """``num_tokens`` tokens of ``seq`` starting at position ``start`` run in this step;
+    ``samples`` is True when the portion reaches the sequence's end (a token is then drawn)."""
+
+    seq: Sequence
+    start: int
+    num_tokens: int
+    samples: bool
+
+
+@dataclass
+class SchedulerOutput:
+    portions: list[ScheduledPortion] = field(default_factory=list)
+    prefill_seqs: list[Sequence] = field(default_factory=list)  # sequences running more than one token
+    decode_seqs: list[Sequence] = field(default_factory=list)   # sequences running exactly one
+    preempted: list[Sequence] = field(default_factory=list)
+    copies: list[tuple[int, int, int]] = field(default_factory=list)  # (group, src, dst) page copies
+    num_batched_tokens: int = 0
+
+    def is_empty(self) -> bool:
+        return not (self.portions or self.preempted)
+
+
+@dataclass
+class SchedulerStats:
+    num_waiting: int = 0
+    num_running: int = 0
+    num_preempted_total: int = 0
+    num_scheduled_batches: int = 0
+    total_prompt_tokens: int = 0
+    total_cached_tokens: int = 0
+
+
+class Scheduler:
+    def __init__(self, cfg: SchedulerConfig, manager: CacheManager,
+                 prefix_cache: Optional[PrefixCache] = None) -> None:
+        self.cfg = cfg
+        self.manager = manager
+        self.prefix_cache = prefix_cache if (prefix_cache is not None and manager.supports_prefix_sharing) else None
+        self.waiting: list[Sequence] = []
+        self.running: list[Sequence] = []
+        self.stats = SchedulerStats()
+        self._matches: dict[str, PrefixMatch] = {}
+        self._order: dict[str, int] = {}
+        self._counter = 0
+
+    # ------------------------------------------------------------------ queue
+    def _priority(self, seq: Sequence) -> tuple[float, int]:
+        return (seq.arrival_time, self._order.get(seq.seq_id, 0))
+
+    def add_seq(self, seq: Sequence) -> None:
+        self._order[seq.seq_id] = self._counter
+        self._counter += 1
+        seq.status = SequenceStatus.WAITING
+        self.waiting.append(seq)
+        self._refresh()
+
+    def has_unfinished(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def _refresh(self) -> None:
+        self.stats.num_waiting = len(self.waiting)
+        self.stats.num_running = len(self.running)
+
+    # ------------------------------------------------------------------ giving back
+    def _release(self, seq: Sequence) -> None:
+        match = self._matches.pop(seq.seq_id, None)
+        if match is not None and self.prefix_cache is not None:
+            self.prefix_cache.release(match)  # the lock; the holds go with the pages below
+        self.manager.free(seq.seq_id)
+
+    def _preempt(self, seq: Sequence) -> None:
+        self._release(seq)
+        seq.reset_for_recompute()
+        seq.num_cached_tokens = 0
+        seq.status = SequenceStatus.PREEMPTED
+        key = self._priority(seq)
+        i = 0
+        while (i < len(self.waiting) and self.waiting[i].status is SequenceStatus.PREEMPTED
+               and self._priority(self.waiting[i]) < key):
+            i += 1
+        self.waiting.insert(i, seq)
+        self.stats.num_preempted_total += 1
+
+    def _evict_for(self, pages: int) -> bool:
+        """Try to free ``pages`` pages from idle prefix-cache blocks; True if any went."""
+        if self.prefix_cache is None or pages <= 0:
+            return False
+        return self.prefix_cache.evict(pages) > 0
+
+    # ------------------------------------------------------------------ one step
+    def _chunk(self, remaining: int, budget_left: int) -> int:
+        n = min(remaining, budget_left)
+        if self.cfg.max_prefill_chunk > 0:
+            n = min(n, self.cfg.max_prefill_chunk)
+        return n
+
+    def _serve_running(self, out: SchedulerOutput) -> None:
+        ordered = sorted(self.running, key=self._priority)
+        budget = self.cfg.max_num_batched_tokens
+        served: list[Sequence] = []
+        while ordered:
+            seq = ordered.pop(0)
+            remaining = seq.num_uncomputed_tokens()
+            if remaining == 1:
+                n = 1  # decoding requests are always served (scheduler.py:98-118)
+            else:
+                n = self._chunk(remaining, budget - out.num_batched_tokens)
+                if not self.cfg.enable_chunked_prefill and n < remaining:
+                    n = 0
+                if n <= 0:
+                    served.append(seq)  # stays running, contributes nothing this step
+                    continue
+            start = seq.num_computed_tokens
+            while not self.manager.can_extend(seq.seq_id, start, start + n):
+                if self._evict_for(1):
+                    continue
+                victim = ordered.pop() if ordered else seq
+                self._preempt(victim)
+                out.preempted.append(victim)
+                if victim is seq:
+                    break
+            if seq.status is SequenceStatus.PREEMPTED:
+                continue
+            out.copies += self.manager.extend(seq.seq_id, start, start + n)
+            served.append(seq)
+            self._emit(out, seq, start, n)
+        self.running = served
+
+    def _emit(self, out: SchedulerOutput, seq: Sequence, start: int, n: int, admitted: bool = False) -> None:
+        samples = start + n == len(seq)
+        out.portions.append(ScheduledPortion(seq, start, n, samples))
+        decoding = seq.num_uncomputed_tokens() == 1 and not admitted
+        (out.decode_seqs if decoding else out.prefill_seqs).append(seq)
+        out.num_batched_tokens += n
+
+    def _try_admit(self, seq: Sequence, out: SchedulerOutput) -> bool:
+        match = PrefixMatch()
+        if self.prefix_cache is not None:
+            match = self.prefix_cache.match(seq.token_ids())
+        cached = match.num_tokens
+        remaining = len(seq) - cached
+        budget_left = self.cfg.max_num_batched_tokens - out.num_batched_tokens
+        n = self._chunk(remaining, budget_left)
+        if not self.cfg.enable_chunked_prefill and n < remaining:
+            n = 0
+        fits = n > 0
+        if fits:
+            prefix_blocks = len(match.handles)
+            if not self.manager.can_admit(len(seq), cached + n, prefix_blocks):
+                # idle cached blocks are worth less than a waiting request
+                need = -(-len(seq) // self.manager.block_size) - prefix_blocks
+                short = need + self.manager.watermark_blocks - self.manager.min_free_blocks()
+                self._evict_for(short)
+                fits = self.manager.can_admit(len(seq), cached + n, prefix_blocks)
+        if not fits:
+            if self.prefix_cache is not None:
+                self.prefix_cache.release(match, drop_holds=True)  # scheduler.py:132-140
+            return False
+        self.manager.admit(seq.seq_id, len(seq), cached + n, prefix=match.handles)
+        if match.node is not None:
+            self._matches[seq.seq_id] = match
+        seq.num_cached_tokens = cached
+        seq.num_computed_tokens = cached
+        seq.status = SequenceStatus.RUNNING
+        self.stats.total_prompt_tokens += len(seq)
+        self.stats.total_cached_tokens += cached
+        out.copies += self.manager.extend(seq.seq_id, cached, cached + n)
+        self._emit(out, seq, cached, n, admitted=True)
+        return True
+
+    def schedule(self) -> SchedulerOutput:
+        out = SchedulerOutput()
+        self._serve_running(out)
+        while self.waiting and len(self.running) < self.cfg.max_num_seqs:
+            seq = self.waiting[0]
+            if not self._try_admit(seq, out):
+                break
+            self.waiting.pop(0)
+            self.running.append(seq)
+        if not out.is_empty():
+            self.stats.num_scheduled_batches += 1
+        self._refresh()
+        return out
+
+    # ------------------------------------------------------------------ finishing
+    def free_finished(self) -> None:
+        for seq in self.running:
+            if seq.is_finished():
+                self._release(seq)
+                self._order.pop(seq.seq_id, None)
+        self.running = [seq for seq in self.running if not seq.is_finished()]
+        self._refresh()
+
+    def abort(self, seq_id: str) -> None:
+        """Waiting and preempted requests hold nothing; a running one gives its pages back.
+        An unknown id is ignored (scheduler.py:180-197)."""
+        for queue, holds in ((self.waiting, False), (self.running, True)):
+            for i, seq in enumerate(queue):
+                if seq.seq_id == seq_id:
+                    if holds:
+                        self._release(seq)
+                    queue.pop(i)
+                    seq.status = SequenceStatus.FINISHED_ABORTED
+                    self._order.pop(seq_id, None)
+                    self._refresh()
+                    return

@@ -1,0 +1,318 @@
+"""Python face of the HIP libraries: shape and type checks on the host, then one C call.
+
+Every function takes torch tensors that live on the GPU, checks what the kernel
+and its grid assume (so a wrong shape is an exception here, never an
+out-of-bounds access there) and launches on torch's current stream. There is no
+other implementation behind these functions: if a library cannot be built or
+loaded the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_int64, c_void_p
+
+import torch
+
+from clockwork_amd.csrc import build
+
+F32, BF16 = 0, 1
+_ERRORS = {
+    -1: "an argument the kernel does not take",
+    -2: "an element type the kernel is not built for",
+    -3: "the HIP runtime refused the launch",
+    -4: "a size beyond the kernel's stated maximum",
+}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _check(code: int, what: str) -> None:
+    if code != 0:
+        raise KernelError(f"{what}: {_ERRORS.get(code, f'error {code}')}")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"the kernels take float32 and bfloat16 tensors, not {dtype}")
+
+
+_libs: dict = {}
+
+
+def _load(name: str, head_dim: int | None = None) -> ctypes.CDLL:
+    key = (name, head_dim)
+    lib = _libs.get(key)
+    if lib is None:
+        path = build.ensure_built(name, head_dim)
+        try:
+            lib = ctypes.CDLL(str(path))
+        except OSError as e:
+            raise KernelError(f"cannot load the HIP library {path}: {e}") from e
+        _declare(name, lib)
+        _libs[key] = lib
+    return lib
+
+
+def preload(head_dims) -> None:
+    """Build (side by side, if several are missing) and load what a model with these head sizes runs."""
+    jobs = [("core", None), ("gemm", None), ("sampling", None)]
+    jobs += [("attention", int(hd)) for hd in sorted(set(head_dims))]
+    build.ensure_many(jobs)
+    for name, hd in jobs:
+        _load(name, hd)
+
+
+def loaded_libraries() -> list[str]:
+    return sorted(str(lib._name) for lib in _libs.values())
+
+
+def _declare(name: str, lib: ctypes.CDLL) -> None:
+    P, I, L, F = c_void_p, c_int, c_int64, c_float
+    sigs = {
+        "core": {
+            "cw_embedding": [P, I, P, P, I, I, I, P],
+            "cw_add_rmsnorm": [P, P, P, I, F, P, I, P, I, I, P],
+            "cw_rope_kv_write": [P, I, P, I, P, P, P, I, I, I, I, I, P, P, L, P],
+            "cw_silu_mul": [P, P, I, I, I, P],
+            "cw_copy_pages": [P, I, L, L, P, I, P],
+            "cw_bf16_to_f32": [P, P, L, P],
+        },
+        "gemm": {
+            "cw_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
+        },
+        "sampling": {
+            "cw_argmax_chunks": [I],
+            "cw_argmax": [P, L, I, I, P, P, L, P],
+            "cw_sample": [P, L, I, I, P, P, P, P, P, P, P],
+        },
+        "attention": {
+            "cw_attention_head_dim": [],
+            "cw_attention_workspace_floats": [I, I, I, I, I],
+            "cw_attention": [I, I, P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P, L, P],
+        },
+    }[name]
+    for fn, argtypes in sigs.items():
+        f = getattr(lib, fn)
+        f.argtypes = argtypes
+        f.restype = c_int64 if fn == "cw_attention_workspace_floats" else c_int
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel arguments must live on the GPU")
+            _need(t.is_contiguous(), "kernel arguments must be contiguous")
+
+
+def _i32(t, n: int | None, what: str) -> None:
+    _need(t.dtype == torch.int32 and t.dim() == 1, f"{what} must be a 1-d int32 tensor")
+    if n is not None:
+        _need(t.numel() >= n, f"{what} holds {t.numel()} entries, {n} needed")
+
+
+# ---------------------------------------------------------------------------------------------
+def embedding(table: torch.Tensor, ids: torch.Tensor, out_resid: torch.Tensor) -> torch.Tensor:
+    """out_resid[t] = float32(table[ids[t]]); out_resid is [T, H] float32."""
+    _gpu(table, ids, out_resid)
+    T = ids.numel()
+    V, H = table.shape
+    _i32(ids, T, "ids")
+    _need(out_resid.dtype == torch.float32 and tuple(out_resid.shape) == (T, H), "residual must be [T, H] float32")
+    _check(
+        _load("core").cw_embedding(_ptr(table), dtype_code(table.dtype), _ptr(ids), _ptr(out_resid), T, H, V, _stream()),
+        "embedding",
+    )
+    return out_resid
+
+
+def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None) -> torch.Tensor:
+    """resid += delta (when given), out = rmsnorm(resid) * weight; with ``rows`` only those rows
+    are normed into out[i] and resid is left alone. resid float32 [T, H]; delta/out in the
+    activation type."""
+    _gpu(resid, delta, weight, out, rows)
+    T, H = resid.shape
+    _need(resid.dtype == torch.float32, "the residual stream is float32")
+    n = T if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, n, "rows")
+    _need(tuple(out.shape) == (n, H), f"out must be [{n}, {H}]")
+    _need(weight.numel() == H, "norm weight has the wrong size")
+    if delta is not None:
+        _need(tuple(delta.shape) == (T, H) and delta.dtype == out.dtype, "delta must be [T, H] in the activation type")
+    _check(
+        _load("core").cw_add_rmsnorm(
+            _ptr(resid), _ptr(delta), _ptr(weight), dtype_code(weight.dtype), float(eps), _ptr(out),
+            dtype_code(out.dtype), _ptr(rows), n, H, _stream()),
+        "add_rmsnorm",
+    )
+    return out
+
+
+def rope_kv_write(qkv, bias, positions, slots, inv_freq, rotary_dim: int, nh: int, nkv: int, hd: int,
+                  k_cache, v_cache) -> None:
+    """Add the bias, rotate q (in place) and k, write k and v rows to the cache at ``slots``.
+
+    qkv [T, (nh + 2 nkv) hd]; k_cache/v_cache [rows, nkv, hd] flat over pages; slots int32 [T]
+    (None: nothing is cached, for a mixer that reads another's cache: then nkv must be 0)."""
+    _gpu(qkv, bias, positions, slots, inv_freq, k_cache, v_cache)
+    T = qkv.shape[0]
+    width = (nh + 2 * nkv) * hd
+    _need(qkv.dim() == 2 and qkv.shape[1] == width, f"qkv must be [T, {width}]")
+    _i32(positions, T, "positions")
+    cache_rows = 0
+    if slots is not None:
+        _i32(slots, T, "slots")
+        _need(k_cache is not None and v_cache is not None, "slots without a cache")
+        _need(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype, "cache and activations differ in type")
+        _need(tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape, "cache must be [..., nkv, hd]")
+        cache_rows = k_cache.numel() // (nkv * hd)
+    else:
+        _need(nkv == 0, "keys and values need slots to be written to")
+    if bias is not None:
+        _need(bias.numel() == width, "qkv bias has the wrong size")
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == rotary_dim // 2, "inv_freq must be float32 [rotary_dim / 2]")
+    else:
+        rotary_dim = 0
+    _check(
+        _load("core").cw_rope_kv_write(
+            _ptr(qkv), dtype_code(qkv.dtype), _ptr(bias), dtype_code(bias.dtype) if bias is not None else 0,
+            _ptr(positions), _ptr(slots), _ptr(inv_freq), int(rotary_dim), T, nh, nkv, hd,
+            _ptr(k_cache), _ptr(v_cache), cache_rows, _stream()),
+        "rope_kv_write",
+    )
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+    _gpu(gate_up, out)
+    T, two_i = gate_up.shape
+    _need(two_i % 2 == 0 and tuple(out.shape) == (T, two_i // 2) and out.dtype == gate_up.dtype, "silu_mul shapes")
+    _check(_load("core").cw_silu_mul(_ptr(gate_up), _ptr(out), dtype_code(out.dtype), T, two_i // 2, _stream()), "silu_mul")
+    return out
+
+
+def copy_pages(pool: torch.Tensor, pairs: torch.Tensor) -> None:
+    """pool [planes, num_blocks, ...]: for each (src, dst) row of ``pairs`` copy page src to dst in every plane."""
+    _gpu(pool, pairs)
+    planes, num_blocks = pool.shape[0], pool.shape[1]
+    block_bytes = pool[0, 0].numel() * pool.element_size()
+    _need(pairs.dtype == torch.int32 and pairs.dim() == 2 and pairs.shape[1] == 2, "pairs must be int32 [n, 2]")
+    _check(_load("core").cw_copy_pages(_ptr(pool), planes, num_blocks, block_bytes, _ptr(pairs), pairs.shape[0], _stream()), "copy_pages")
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None) -> torch.Tensor:
+    """y = x @ weight.T (+ bias). float32: the true-float32 HIP product; bfloat16: the library
+    product (as the reference's engine uses one), float32 accumulation."""
+    _gpu(x, weight, bias)
+    M, K = x.shape
+    N = weight.shape[0]
+    _need(weight.shape[1] == K, f"weight is {tuple(weight.shape)}, input has {K} columns")
+    if x.dtype == torch.float32:
+        _need(weight.dtype == torch.float32, "a float32 product needs float32 weights")
+        out = torch.empty((M, N), dtype=torch.float32, device=x.device)
+        if bias is not None:
+            _need(bias.dtype == torch.float32 and bias.numel() == N, "bias must be float32 [N]")
+        _check(_load("gemm").cw_gemm_f32(_ptr(x), K, _ptr(weight), _ptr(bias), _ptr(out), N, M, N, K, _stream()), "gemm_f32")
+        return out
+    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "a bfloat16 product needs bfloat16 operands")
+    y = torch.mm(x, weight.t()) if bias is None else torch.addmm(bias, x, weight.t())
+    if out_dtype == torch.float32:
+        out = torch.empty((M, N), dtype=torch.float32, device=x.device)
+        _check(_load("core").cw_bf16_to_f32(_ptr(y), _ptr(out), M * N, _stream()), "bf16_to_f32")
+        return out
+    return y
+
+
+def attention(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
+              rows: int, nh: int, nkv: int, hd: int, block_size: int, gh: int, n_splits: int, window: int,
+              scale: float, n_tokens: int, n_requests: int, workspace=None) -> None:
+    """Paged causal attention for ``n_items`` work items (see csrc/attention.hip).
+
+    q: any tensor whose token rows are ``q_stride`` elements apart with head h at column h * hd;
+    out [n_tokens, nh * hd]; caches [num_blocks * block_size, nkv, hd]; block_tables int32
+    [n_requests, max_blocks]; items int32 [n_items, 4] = (request, first token, tokens, 0)."""
+    _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, workspace)
+    _need(q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype, "attention operands differ in type or device")
+    _need(out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd, "attention output must be [T, nh * hd]")
+    _need(q_stride >= nh * hd, "query rows overlap")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= n_requests, "block_tables must be int32 [R, max_blocks]")
+    _i32(ctx_lens, n_requests, "ctx_lens")
+    _i32(cu_q, n_requests + 1, "cu_q")
+    _need(items.dtype == torch.int32 and items.numel() >= 4 * n_items, "items must be int32 [n_items, 4]")
+    _need(tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape, "cache must be [..., nkv, hd]")
+    lib = _load("attention", hd)
+    group = nh // nkv
+    n_chunks = -(-group // gh)
+    need = lib.cw_attention_workspace_floats(rows, n_items, nkv, n_chunks, n_splits)
+    ws_floats = 0
+    if need > 0:
+        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need,
+              f"attention needs a float32 workspace of {need} elements")
+        ws_floats = workspace.numel()
+    _check(
+        lib.cw_attention(
+            rows, dtype_code(out.dtype), q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache),
+            _ptr(block_tables), block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, nh, nkv,
+            block_size, gh, n_splits, window, float(scale), _ptr(workspace), ws_floats, _stream()),
+        "attention",
+    )
+
+
+def attention_workspace_floats(hd: int, rows: int, n_items: int, nkv: int, n_chunks: int, n_splits: int) -> int:
+    return int(_load("attention", hd).cw_attention_workspace_floats(rows, n_items, nkv, n_chunks, n_splits))
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """First index of the maximum of every row of float32 ``logits`` [n, V] -> int32 [n]."""
+    _gpu(logits, out)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be float32 [n, V]")
+    n, V = logits.shape
+    lib = _load("sampling")
+    chunks = lib.cw_argmax_chunks(V)
+    ws = torch.empty(max(1, n * chunks * 2), dtype=torch.int32, device=logits.device)
+    if out is None:
+        out = torch.empty(n, dtype=torch.int32, device=logits.device)
+    _i32(out, n, "out")
+    _check(lib.cw_argmax(_ptr(logits), V, n, V, _ptr(out), _ptr(ws), ws.numel() * 4, _stream()), "argmax")
+    return out
+
+
+def sample(logits, temperature, top_k, top_p, seeds, draws, out=None) -> torch.Tensor:
+    """One token per row: rows with temperature 0 take the arg-max, the others are drawn."""
+    _gpu(logits, temperature, top_k, top_p, seeds, draws, out)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be float32 [n, V]")
+    n, V = logits.shape
+    _need(temperature.dtype == torch.float32 and temperature.numel() == n, "temperature must be float32 [n]")
+    _need(top_p.dtype == torch.float32 and top_p.numel() == n, "top_p must be float32 [n]")
+    _i32(top_k, n, "top_k")
+    _need(seeds.dtype == torch.int64 and seeds.numel() == n, "seeds must be int64 [n]")
+    _need(draws.dtype == torch.int64 and draws.numel() == n, "draws must be int64 [n]")
+    if out is None:
+        out = torch.empty(n, dtype=torch.int32, device=logits.device)
+    _i32(out, n, "out")
+    _check(
+        _load("sampling").cw_sample(_ptr(logits), V, n, V, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds),
+                                    _ptr(draws), _ptr(out), _stream()),
+        "sample",
+    )
+    return out

@@ -1,0 +1,66 @@
+"""Interfaces of the parts a layer is put together from.
+
+A part is built from its spec alone (sizes and constants are parameters; no part
+knows which model it is in) and goes through three stages:
+
+1. ``param_specs()`` - the tensors it owns: ``{local name: ParamSpec}``. Needs no GPU.
+2. ``bind(params, device, dtype)`` - receives ``{local name: device tensor}`` and
+   prepares whatever else it needs on the device (tables, constants).
+3. its run method, called by the block arrangement during a step.
+
+Roles and their run methods:
+
+* norm:          ``forward(resid, delta, rows=None) -> normed`` - ``resid`` is the
+                 float32 residual stream [T, H]; ``delta`` (activation type, or None)
+                 is added to it in place first; returns the normed rows in the
+                 activation type. With ``rows`` only those rows are produced and
+                 ``resid`` is left untouched.
+* mixer:         ``forward(x, ctx, cache) -> y`` with x, y [T, H] in the activation
+                 type; ``cache_need()`` returns a KVPagesSpec, a StateSpec or None.
+                 ``cache`` is the run entry's :class:`EntryCache`.
+* feed-forward:  ``forward(x, ctx) -> y``.
+* position enc.: used by a mixer, not by the block; the attention mixer expects
+                 ``rotate_and_store(qkv, bias, positions, slots, nh, nkv, hd, k, v)``.
+* arrangement:   ``forward(resid, delta, ctx, cache) -> delta`` - wires norms,
+                 mixer and feed-forward around the residual stream; the returned
+                 ``delta`` is the last branch output, not yet added.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Optional
+
+from clockwork_amd.config.spec import ParamSpec
+
+
+class Part:
+    """Convenience base: no parameters, nothing to prepare."""
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {}
+
+    def bind(self, params: dict, device, dtype) -> None:
+        self.params = params
+
+    def cache_need(self) -> Optional[Any]:
+        return None
+
+
+@dataclass
+class EntryCache:
+    """The cache of one run entry as its mixer sees it.
+
+    Key/value kind: ``k`` and ``v`` are flat [num_blocks * block_size, kv_heads, head_dim]
+    views of the entry's pages, ``group`` indexes the step context's per-group block
+    tables and slot mappings, ``writes`` is False when the entry reads another entry's
+    cache. State kind: ``state`` is [max_num_seqs, *shape]; the request's row is
+    ``ctx.state_slots[r]``.
+    """
+
+    group: int = -1
+    k: Any = None
+    v: Any = None
+    state: Any = None
+    writes: bool = True
+    block_size: int = 0

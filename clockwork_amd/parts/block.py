@@ -1,0 +1,32 @@
+"""Block arrangements: how norms, mixer and feed-forward sit around the residual stream."""
+
+from __future__ import annotations
+
+
+class PreNormBlock:
+    """x = x + mixer(norm(x)); x = x + ffn(norm(x)) (clockwork/engine/model.py:139-154).
+
+    The residual stream is float32 and is only ever touched by the norms' fused add, so
+    each branch output is added exactly once, in float32. ``forward`` takes the previous
+    block's pending output ``delta`` and returns its own.
+    """
+
+    def __init__(self, mixer, feed_forward, mixer_norm, ffn_norm) -> None:
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.ffn_norm = ffn_norm
+
+    def parts(self) -> dict:
+        return {
+            "mixer": self.mixer,
+            "feed_forward": self.feed_forward,
+            "mixer_norm": self.mixer_norm,
+            "ffn_norm": self.ffn_norm,
+        }
+
+    def forward(self, resid, delta, ctx, cache):
+        x = self.mixer_norm.forward(resid, delta)
+        a = self.mixer.forward(x, ctx, cache)
+        x = self.ffn_norm.forward(resid, a)
+        return self.feed_forward.forward(x, ctx)

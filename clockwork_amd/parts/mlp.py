@@ -1,0 +1,32 @@
+"""Dense SwiGLU feed-forward: down(silu(gate(x)) * up(x)) (clockwork/engine/model.py:52-63).
+
+gate and up are one product over a fused [2 I, H] weight; the gate multiply is one kernel.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from clockwork_amd import ops
+from clockwork_amd.config.spec import ParamSpec
+from clockwork_amd.parts.base import Part
+from clockwork_amd.parts.specs import SwiGLUSpec
+
+
+class SwiGLU(Part):
+    def __init__(self, spec: SwiGLUSpec) -> None:
+        self.spec = spec
+
+    def param_specs(self):
+        H, I = self.spec.hidden_size, self.spec.intermediate_size
+        return {"gate_up_weight": ParamSpec((2 * I, H)), "down_weight": ParamSpec((H, I))}
+
+    def bind(self, params, device, dtype) -> None:
+        self.gate_up = params["gate_up_weight"]
+        self.down = params["down_weight"]
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        gu = ops.linear(x, self.gate_up)
+        act = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
+        ops.silu_mul(gu, act)
+        return ops.linear(act, self.down)

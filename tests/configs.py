@@ -1,0 +1,26 @@
+"""The tiny configurations the tests run: they differ in every size and option.
+
+A and B are the benchmark description's tiny models; C makes num_heads * head_dim
+differ from hidden_size (an explicit head_dim key) and uses sizes that are no powers
+of two, which neither A nor B pins.
+"""
+
+TINY_A = dict(
+    model_type="qwen2", architectures=["Qwen2ForCausalLM"], vocab_size=512, hidden_size=64,
+    num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, intermediate_size=176,
+    rms_norm_eps=1e-6, rope_theta=10000.0, tie_word_embeddings=True, hidden_act="silu",
+    use_sliding_window=False, max_position_embeddings=256,
+)
+TINY_B = dict(
+    model_type="qwen2", architectures=["Qwen2ForCausalLM"], vocab_size=1000, hidden_size=192,
+    num_hidden_layers=3, num_attention_heads=6, num_key_value_heads=1, intermediate_size=384,
+    rms_norm_eps=1e-5, rope_theta=1000000.0, tie_word_embeddings=False, hidden_act="silu",
+    use_sliding_window=False, max_position_embeddings=512,
+)
+TINY_C = dict(
+    model_type="qwen2", vocab_size=777, hidden_size=80, head_dim=48,
+    num_hidden_layers=2, num_attention_heads=3, num_key_value_heads=3, intermediate_size=100,
+    rms_norm_eps=3e-6, rope_theta=50000.0, tie_word_embeddings=False,
+)
+# name -> (config, weight seed, cache block size)
+TINY_CONFIGS = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8), "C": (TINY_C, 5, 16)}

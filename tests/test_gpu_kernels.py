@@ -1,0 +1,439 @@
+"""Each HIP kernel alone against a plain float32 formula, at sizes other than the engine's."""
+
+import math
+
+import pytest
+import torch
+
+from tests.plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+@pytest.fixture(autouse=True)
+def _seed():
+    torch.manual_seed(1234)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("V,H,T", [(777, 100, 13), (32, 1536, 1)])
+def test_embedding(dtype, V, H, T):
+    from clockwork_amd import ops
+
+    table = torch.randn(V, H, device=DEV).to(dtype)
+    ids = torch.randint(0, V, (T,), device=DEV, dtype=torch.int32)
+    ids[0] = V - 1
+    out = torch.full((T, H), 7.0, device=DEV)
+    ops.embedding(table, ids, out)
+    torch.testing.assert_close(out, plain.embedding(table.float().cpu(), ids.long().cpu()).to(DEV), rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype,wdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("T,H,eps", [(5, 100, 1e-5), (3, 1536, 1e-6), (2, 7, 3e-6), (1, 4100, 1e-6)])
+def test_add_rmsnorm(dtype, wdtype, T, H, eps):
+    from clockwork_amd import ops
+
+    resid = torch.randn(T, H, device=DEV) * 3
+    delta = torch.randn(T, H, device=DEV).to(dtype)
+    weight = (1 + 0.1 * torch.randn(H, device=DEV)).to(wdtype)
+    want_resid = resid + delta.float()
+    want = plain.rmsnorm(want_resid.cpu(), weight.float().cpu(), eps).to(DEV)
+    r = resid.clone()
+    out = torch.empty(T, H, device=DEV, dtype=dtype)
+    ops.add_rmsnorm(r, delta, weight, eps, out)
+    torch.testing.assert_close(r, want_resid, rtol=0, atol=0)
+    torch.testing.assert_close(out.float(), want, **tol(dtype))
+    # without a delta the stream is left as it is
+    r2 = resid.clone()
+    ops.add_rmsnorm(r2, None, weight, eps, out)
+    torch.testing.assert_close(r2, resid, rtol=0, atol=0)
+    torch.testing.assert_close(out.float(), plain.rmsnorm(resid.cpu(), weight.float().cpu(), eps).to(DEV), **tol(dtype))
+    # selected rows: normed into a compact output, the stream untouched
+    rows = torch.tensor([T - 1, 0], dtype=torch.int32, device=DEV)
+    r3 = resid.clone()
+    out2 = torch.empty(2, H, device=DEV, dtype=dtype)
+    ops.add_rmsnorm(r3, delta, weight, eps, out2, rows)
+    torch.testing.assert_close(r3, resid, rtol=0, atol=0)
+    torch.testing.assert_close(out2.float(), want[rows.long()], **tol(dtype))
+
+
+def test_rmsnorm_zero_row_and_scale_invariance():
+    from clockwork_amd import ops
+
+    H = 96
+    x = torch.randn(2, H, device=DEV)
+    x[1] = 0
+    w = torch.ones(H, device=DEV)
+    out = torch.empty(2, H, device=DEV)
+    ops.add_rmsnorm(x.clone(), None, w, 1e-6, out)
+    assert torch.all(out[1] == 0)
+    assert abs(float(out[0].pow(2).mean().sqrt()) - 1.0) < 1e-4
+    out2 = torch.empty(2, H, device=DEV)
+    ops.add_rmsnorm((x * 37.0).clone(), None, w, 1e-6, out2)
+    torch.testing.assert_close(out2[0], out[0], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,rotary,theta", [(4, 2, 16, 16, 1e4), (6, 1, 32, 32, 1e6), (3, 3, 48, 48, 5e4), (5, 1, 64, 32, 1e4)])
+def test_rope_kv_write(dtype, nh, nkv, hd, rotary, theta):
+    from clockwork_amd import ops
+
+    T, rows = 9, 40
+    width = (nh + 2 * nkv) * hd
+    qkv = torch.randn(T, width, device=DEV).to(dtype)
+    bias = (0.5 * torch.randn(width, device=DEV)).to(dtype)
+    positions = torch.tensor([0, 1, 2, 3, 4000, 4001, 17, 255, 256], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([5, 39, 0, 17, 3, -1, 8, 21, 30], dtype=torch.int32, device=DEV)
+    kc = torch.full((rows, nkv, hd), 100.0, device=DEV, dtype=dtype)
+    vc = torch.full((rows, nkv, hd), 100.0, device=DEV, dtype=dtype)
+    inv_freq = plain.inv_frequencies(rotary, theta).to(DEV)
+
+    x = (qkv.float() + bias.float()).cpu()
+    q = x[:, : nh * hd].view(T, nh, hd)
+    k = x[:, nh * hd : (nh + nkv) * hd].view(T, nkv, hd)
+    v = x[:, (nh + nkv) * hd :].view(T, nkv, hd)
+    cos, sin = plain.rope_tables(positions.cpu(), rotary, theta)
+    q_ref, k_ref = q.clone(), k.clone()
+    q_ref[..., :rotary] = plain.apply_rope(q[..., :rotary], cos, sin)
+    k_ref[..., :rotary] = plain.apply_rope(k[..., :rotary], cos, sin)
+
+    work = qkv.clone()
+    ops.rope_kv_write(work, bias, positions, slots, inv_freq, rotary, nh, nkv, hd, kc, vc)
+    t = dict(rtol=1e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(work[:, : nh * hd].float().cpu().view(T, nh, hd), q_ref, **t)
+    written = set()
+    for i, s in enumerate(slots.tolist()):
+        if s < 0:
+            continue
+        written.add(s)
+        torch.testing.assert_close(kc[s].float().cpu(), k_ref[i], **t)
+        torch.testing.assert_close(vc[s].float().cpu(), v[i], **t)
+    for s in range(rows):
+        if s not in written:
+            assert torch.all(kc[s] == 100.0) and torch.all(vc[s] == 100.0)
+
+
+def test_rope_is_relative_and_identity_at_zero():
+    """<R_m q, R_n k> depends on m - n only; position 0 rotates nothing; values pass through."""
+    from clockwork_amd import ops
+
+    nh, nkv, hd = 1, 1, 32
+    inv_freq = plain.inv_frequencies(hd, 1e4).to(DEV)
+    base = torch.randn(1, 3 * hd, device=DEV)
+
+    def rotated(pos_q, pos_k):
+        out = []
+        for pos in (pos_q, pos_k):
+            qkv = base.clone()
+            kc = torch.zeros(1, 1, hd, device=DEV)
+            vc = torch.zeros(1, 1, hd, device=DEV)
+            ops.rope_kv_write(qkv, None, torch.tensor([pos], dtype=torch.int32, device=DEV),
+                              torch.tensor([0], dtype=torch.int32, device=DEV), inv_freq, hd, nh, nkv, hd, kc, vc)
+            out.append((qkv[0, :hd].clone(), kc[0, 0].clone(), vc[0, 0].clone()))
+        return out
+
+    (q0, k0, v0), _ = rotated(0, 0)
+    torch.testing.assert_close(q0, base[0, :hd], rtol=0, atol=0)
+    torch.testing.assert_close(k0, base[0, hd : 2 * hd], rtol=0, atol=0)
+    torch.testing.assert_close(v0, base[0, 2 * hd :], rtol=0, atol=0)
+    (qa, _, _), (_, kb, _) = rotated(7, 3)
+    (qc, _, _), (_, kd, _) = rotated(107, 103)
+    assert abs(float(qa @ kb) - float(qc @ kd)) < 1e-4
+    assert abs(float(qa @ kb) - float(q0 @ k0)) > 1e-3  # and it does depend on the distance
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 100, 176), (7, 64, 33), (64, 130, 64), (130, 17, 1000), (3, 1000, 192)])
+def test_gemm_f32(M, N, K):
+    from clockwork_amd import ops
+
+    x = torch.randn(M, K, device=DEV)
+    w = torch.randn(N, K, device=DEV)
+    b = torch.randn(N, device=DEV)
+    want = (x.double() @ w.double().t() + b.double()).float()
+    got = ops.linear(x, w, b)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5 * math.sqrt(K))
+    got = ops.linear(x, w)
+    torch.testing.assert_close(got, (x.double() @ w.double().t()).float(), rtol=1e-5, atol=1e-5 * math.sqrt(K))
+
+
+def test_gemm_f32_rows_do_not_depend_on_batch():
+    from clockwork_amd import ops
+
+    x = torch.randn(70, 200, device=DEV)
+    w = torch.randn(90, 200, device=DEV)
+    whole = ops.linear(x, w)
+    for i in (0, 33, 69):
+        assert torch.equal(ops.linear(x[i : i + 1].contiguous(), w)[0], whole[i])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_linear_library_path_and_float32_logits(dtype):
+    from clockwork_amd import ops
+
+    x = torch.randn(5, 96, device=DEV).to(dtype)
+    w = torch.randn(50, 96, device=DEV).to(dtype)
+    got = ops.linear(x, w, out_dtype=torch.float32)
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got, x.float() @ w.float().t(), **(dict(rtol=1e-5, atol=1e-4) if dtype == torch.float32 else dict(rtol=2e-2, atol=1e-1)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I", [(3, 176), (1, 100), (17, 384)])
+def test_silu_mul(dtype, T, I):
+    from clockwork_amd import ops
+
+    gu = (2 * torch.randn(T, 2 * I, device=DEV)).to(dtype)
+    gu[0, 0] = 0.0
+    out = torch.empty(T, I, device=DEV, dtype=dtype)
+    ops.silu_mul(gu, out)
+    want = torch.nn.functional.silu(gu[:, :I].float()) * gu[:, I:].float()
+    torch.testing.assert_close(out.float(), want, **tol(dtype))
+    assert float(out[0, 0]) == 0.0
+
+
+def test_copy_pages():
+    from clockwork_amd import ops
+
+    pool = torch.randn(6, 10, 4, 2, 8, device=DEV)
+    before = pool.clone()
+    ops.copy_pages(pool.view(6, 10, -1), torch.tensor([[3, 7], [0, 9]], dtype=torch.int32, device=DEV))
+    want = before.clone()
+    want[:, 7] = before[:, 3]
+    want[:, 9] = before[:, 0]
+    assert torch.equal(pool, want)
+
+
+# ---------------------------------------------------------------------------------- attention
+def _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens, poison=100.0):
+    """Random keys/values per request laid into scrambled pages; unowned slots hold ``poison``."""
+    kc = torch.full((num_blocks * bs, nkv, hd), poison, dtype=dtype, device=DEV)
+    vc = torch.full((num_blocks * bs, nkv, hd), poison, dtype=dtype, device=DEV)
+    ks, vs = [], []
+    for table, ctx in zip(tables, ctx_lens):
+        k = torch.randn(ctx, nkv, hd, device=DEV).to(dtype)
+        v = torch.randn(ctx, nkv, hd, device=DEV).to(dtype)
+        for p in range(ctx):
+            slot = table[p // bs] * bs + p % bs
+            kc[slot], vc[slot] = k[p], v[p]
+        ks.append(k)
+        vs.append(v)
+    return kc, vc, ks, vs
+
+
+def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs, window=0, splits=None, scale=None):
+    from clockwork_amd import ops
+    from clockwork_amd.engine.batch import StepContext
+
+    ctx = StepContext()
+    ctx.device = torch.device(DEV)
+    ctx.h_q_lens, ctx.h_ctx_lens = list(q_lens), list(ctx_lens)
+    plan = ctx.attention_plan(nh, nkv)
+    if splits is not None:
+        plan.single_splits = splits
+    R = len(q_lens)
+    width = max(len(t) for t in tables)
+    bt = torch.full((R, width), -1, dtype=torch.int32, device=DEV)
+    for r, t in enumerate(tables):
+        bt[r, : len(t)] = torch.tensor(t, dtype=torch.int32)
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32, device=DEV)
+    cl = torch.tensor(ctx_lens, dtype=torch.int32, device=DEV)
+    T = sum(q_lens)
+    # queries sit inside a wider row, as they do in the fused qkv buffer
+    pad = 24
+    qbuf = torch.full((T, nh * hd + pad), 55.0, dtype=dtype, device=DEV)
+    qbuf[:, : nh * hd] = torch.cat(qs).reshape(T, nh * hd)
+    out = torch.full((T, nh * hd), -77.0, dtype=dtype, device=DEV)
+    scale = scale if scale is not None else hd ** -0.5
+    common = dict(q=qbuf, q_stride=qbuf.shape[1], out=out, k_cache=kc, v_cache=vc, block_tables=bt, ctx_lens=cl,
+                  cu_q=cu, nh=nh, nkv=nkv, hd=hd, block_size=bs, window=window, scale=scale, n_tokens=T, n_requests=R)
+    if plan.n_wide:
+        ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide, n_splits=1, **common)
+    if plan.n_single:
+        ws = None
+        if plan.single_splits > 1:
+            ws = torch.empty(ops.attention_workspace_floats(hd, 16, plan.n_single, nkv, plan.chunks_single, plan.single_splits),
+                             dtype=torch.float32, device=DEV)
+        ops.attention(items=plan.single_items, n_items=plan.n_single, rows=16, gh=plan.gh_single,
+                      n_splits=plan.single_splits, workspace=ws, **common)
+    return out.view(T, nh, hd)
+
+
+# the reference's decode cases (tests/test_triton_kernel.py:14-20) plus sizes of our own
+DECODE_CASES = [
+    (4, 4, 16, 4, [5, 12, 9]),
+    (8, 2, 32, 4, [1, 7, 16, 3]),
+    (6, 3, 64, 8, [23, 8, 31]),
+    (12, 2, 128, 16, [17, 64, 49, 2]),
+    (6, 1, 48, 16, [300, 33]),
+    (40, 2, 16, 8, [70]),  # a group of 20 heads: more than one head chunk
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,bs,ctx_lens", DECODE_CASES)
+@pytest.mark.parametrize("splits", [1, 3])
+def test_attention_single_tokens(dtype, nh, nkv, hd, bs, ctx_lens, splits):
+    num_blocks = sum(-(-c // bs) for c in ctx_lens) + 5
+    perm = torch.randperm(num_blocks).tolist()
+    tables, at = [], 0
+    for c in ctx_lens:
+        n = -(-c // bs)
+        tables.append(perm[at : at + n])
+        at += n
+    kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens)
+    qs = [torch.randn(1, nh, hd, device=DEV).to(dtype) for _ in ctx_lens]
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, [1] * len(ctx_lens), kc, vc, qs, splits=splits)
+    assert not torch.isnan(out.float()).any()
+    for r in range(len(ctx_lens)):
+        want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5)
+        torch.testing.assert_close(out[r : r + 1].float().cpu(), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,bs", [(4, 2, 16, 4), (6, 1, 32, 8), (3, 3, 48, 16), (12, 2, 128, 16), (2, 1, 256, 16)])
+def test_attention_portions_and_mixed_batches(dtype, nh, nkv, hd, bs):
+    """Portions (cached prefix + new tokens, end-aligned mask: clockwork/kernels/attention.py:45-65,
+    tests/test_attention_kernels.py:49-62) next to single tokens, scrambled pages, poisoned free slots."""
+    ctx_lens = [21, 150, 2, 77, 1, 64]
+    q_lens = [6, 150, 2, 1, 1, 33]
+    num_blocks = sum(-(-c // bs) for c in ctx_lens) + 3
+    perm = torch.randperm(num_blocks).tolist()
+    tables, at = [], 0
+    for c in ctx_lens:
+        n = -(-c // bs)
+        tables.append(perm[at : at + n])
+        at += n
+    kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens)
+    qs = [torch.randn(q, nh, hd, device=DEV).to(dtype) for q in q_lens]
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs)
+    at = 0
+    for r, q_len in enumerate(q_lens):
+        want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5)
+        torch.testing.assert_close(out[at : at + q_len].float().cpu(), want, **tol(dtype))
+        at += q_len
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 5, 16, 40])
+def test_attention_window(dtype, window):
+    """A token reads itself and the window-1 tokens before it; pages behind the window may be gone
+    (table entry -1) and are never dereferenced."""
+    nh, nkv, hd, bs = 4, 2, 32, 8
+    ctx_lens, q_lens = [90, 50, 70], [30, 1, 2]
+    num_blocks = 40
+    tables = [list(range(0, 12)), list(range(12, 19)), list(range(19, 28))]
+    kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens)
+    tables_dev = [list(t) for t in tables]
+    for r, (c, q) in enumerate(zip(ctx_lens, q_lens)):
+        first_needed = max(0, (c - q) - window + 1) // bs
+        for b in range(first_needed):
+            tables_dev[r][b] = -1
+    qs = [torch.randn(q, nh, hd, device=DEV).to(dtype) for q in q_lens]
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables_dev, ctx_lens, q_lens, kc, vc, qs, window=window)
+    at = 0
+    for r, q_len in enumerate(q_lens):
+        want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5, window=window)
+        torch.testing.assert_close(out[at : at + q_len].float().cpu(), want, **tol(dtype))
+        at += q_len
+
+
+def test_attention_far_key_stands_out():
+    """One key among hundreds, scaled so that its score dominates: the output must be its value,
+    wherever in the context (first page, page edge, last position) it sits."""
+    nh, nkv, hd, bs = 2, 1, 64, 16
+    ctx = 700
+    for where in (0, 15, 16, 511, 512, 698, 699):
+        tables = [list(range(44))]
+        kc, vc, ks, vs = _paged_setup(torch.float32, nkv, hd, bs, 50, tables, [ctx])
+        q = torch.randn(1, nh, hd, device=DEV)
+        slot = tables[0][where // bs] * bs + where % bs
+        kc[slot, 0] = 40.0 * q[0, 0] / q[0, 0].norm()
+        out = _run_attention(torch.float32, nh, nkv, hd, bs, tables, [ctx], [1], kc, vc, [q], splits=4)
+        torch.testing.assert_close(out[0, 0], vc[slot, 0], rtol=1e-3, atol=1e-3)
+
+
+def test_attention_reduces_to_library_routine():
+    """One head group, no rotation: equals F.scaled_dot_product_attention(is_causal=True)
+    (tests/test_attention_kernels.py:137-145)."""
+    nh, hd, bs, T = 4, 32, 8, 45
+    tables = [list(range(6))]
+    kc, vc, ks, vs = _paged_setup(torch.float32, nh, hd, bs, 8, tables, [T])
+    q = torch.randn(T, nh, hd, device=DEV)
+    out = _run_attention(torch.float32, nh, nh, hd, bs, tables, [T], [T], kc, vc, [q], scale=0.3)
+    want = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], ks[0].transpose(0, 1)[None], vs[0].transpose(0, 1)[None], is_causal=True, scale=0.3
+    )[0].transpose(0, 1)
+    torch.testing.assert_close(out, want, rtol=1e-5, atol=1e-5)
+
+
+def test_attention_refuses_wrong_shapes():
+    from clockwork_amd import ops
+    from clockwork_amd.ops import KernelError
+
+    with pytest.raises(ValueError):
+        ops._load("attention", 24)
+    kc = torch.zeros(64, 2, 32, device=DEV)
+    with pytest.raises(KernelError):
+        _run_attention(torch.float32, 4, 2, 32, 8, [[0]], [4], [1], kc[:, :1], kc, [torch.zeros(1, 4, 32, device=DEV)])
+
+
+# ---------------------------------------------------------------------------------- sampling
+@pytest.mark.parametrize("n,V", [(1, 1000), (5, 151936), (3, 17)])
+def test_argmax_first_index_wins(n, V):
+    from clockwork_amd import ops
+
+    logits = torch.randn(n, V, device=DEV)
+    logits[0, V // 2] = 50.0
+    logits[0, V - 1] = 50.0
+    got = ops.argmax(logits)
+    assert got.tolist() == logits.argmax(-1).tolist()
+    assert got[0] == V // 2
+
+
+def test_sampling_matches_plain_definition():
+    from clockwork_amd import ops
+
+    V, n = 1000, 24
+    logits = 3 * torch.randn(n, V, device=DEV)
+    temps = torch.tensor([0.0, 0.8, 1.5, 1.0] * 6, device=DEV)
+    top_k = torch.tensor(([-1] * 4 + [5] * 4 + [1] * 4 + [-1] * 4 + [50] * 4 + [V] * 4), dtype=torch.int32, device=DEV)
+    top_p = torch.tensor(([1.0] * 12 + [0.9] * 4 + [0.5] * 4 + [0.05] * 4), device=DEV)
+    seeds = torch.arange(n, dtype=torch.int64, device=DEV) * 7 + 1
+    draws = torch.arange(n, dtype=torch.int64, device=DEV) % 5
+    got = ops.sample(logits, temps, top_k, top_p, seeds, draws).tolist()
+    for i in range(n):
+        if temps[i] == 0:
+            assert got[i] == int(logits[i].argmax())
+            continue
+        probs = plain.sampling_probs(logits[i].cpu(), float(temps[i]), int(top_k[i]), float(top_p[i]))
+        u = plain.uniform01(int(seeds[i]), int(draws[i]))
+        want, margin = plain.draw(probs, u)
+        assert probs[got[i]] > 0, f"row {i}: a token outside the kept set was drawn"
+        assert got[i] == want or margin < 1e-4, f"row {i}: got {got[i]}, plain draws {want} (margin {margin})"
+        if int(top_k[i]) == 1:
+            assert got[i] == int(logits[i].argmax())  # tests/test_server.py:323
+
+
+def test_sampling_is_reproducible_and_follows_the_distribution():
+    from clockwork_amd import ops
+
+    V, n = 8, 4000
+    row = torch.tensor([2.0, 1.0, 0.0, -1.0, 0.5, -3.0, 1.5, 0.2], device=DEV)
+    logits = row.repeat(n, 1)
+    args = (torch.ones(n, device=DEV), torch.full((n,), -1, dtype=torch.int32, device=DEV), torch.ones(n, device=DEV))
+    seeds = torch.full((n,), 42, dtype=torch.int64, device=DEV)
+    draws = torch.arange(n, dtype=torch.int64, device=DEV)
+    a = ops.sample(logits, *args, seeds, draws)
+    b = ops.sample(logits, *args, seeds, draws)
+    assert torch.equal(a, b)
+    c = ops.sample(logits, *args, seeds + 1, draws)
+    assert not torch.equal(a, c)
+    freq = torch.bincount(a.long(), minlength=V).float() / n
+    torch.testing.assert_close(freq.cpu(), torch.softmax(row, -1).cpu(), rtol=0, atol=0.03)

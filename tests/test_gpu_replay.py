@@ -1,0 +1,126 @@
+"""The engine's step function, cache and kernels against the plain implementation: the same
+requests whole, with the last 32 tokens decoded one by one, in portions of changing size, and
+mixed with other requests on so few pages that pages are used again; float32 and bfloat16."""
+
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from tests import replay
+from tests.configs import TINY_CONFIGS
+from tests.plain.qwen2_plain import PlainQwen2
+
+pytestmark = pytest.mark.gpu
+REPO = Path(__file__).resolve().parents[1]
+
+# float32 must agree to 1e-5 (the reference's own bar, tests/test_hf_equivalence.py:15-16);
+# bfloat16 rounds every activation to 8 bits: logits here are O(1), errors stay under 0.03
+TOL = {"float32": dict(rtol=1e-5, atol=1e-5), "bfloat16": dict(rtol=3e-2, atol=3e-2)}
+LENGTHS = {"A": [5, 17, 33, 100, 64, 131, 47], "B": [1, 9, 40, 64, 100, 150, 77], "C": [3, 70, 129, 16, 48]}
+
+
+def _requests(name):
+    cfg = TINY_CONFIGS[name][0]
+    gen = torch.Generator().manual_seed(len(name) + cfg["vocab_size"])
+    return {
+        f"r{i}": torch.randint(0, cfg["vocab_size"], (n,), generator=gen).tolist()
+        for i, n in enumerate(LENGTHS[name])
+    }
+
+
+_plain_cache = {}
+
+
+def _plain(name, model_dirs):
+    if name not in _plain_cache:
+        model = PlainQwen2(model_dirs[name])
+        _plain_cache[name] = {rid: model.logits(toks) for rid, toks in _requests(name).items()}
+    return _plain_cache[name]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("mode", ["whole", "prefill_then_decode", "portions", "mixed"])
+def test_replay_matches_plain(model_dirs, name, dtype, mode):
+    requests = _requests(name)
+    block_size = TINY_CONFIGS[name][2]
+    live = 4 if mode == "mixed" else 1
+    runner = replay.make_runner(model_dirs[name], dtype, block_size, replay.pages_needed(requests, live, block_size))
+    steps = getattr(replay, mode)(requests)
+    got = replay.run_trace(runner, steps)
+    assert len(got) == sum(len(t) for t in requests.values())
+    worst = replay.compare(got, _plain(name, model_dirs), **TOL[dtype])
+    print(f"{name} {dtype} {mode}: largest error {worst:.3e}")
+    assert not runner.manager.live_requests()
+    assert runner.manager.min_free_blocks() == runner.manager.num_blocks
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_and_long_decoding(model_dirs, dtype):
+    """The first tokens of a sequence (one-token prompt, then decoding from position 1) and a
+    long run of single tokens across many page edges."""
+    name = "B"
+    cfg, _, block_size = TINY_CONFIGS[name]
+    toks = torch.randint(0, cfg["vocab_size"], (200,), generator=torch.Generator().manual_seed(7)).tolist()
+    runner = replay.make_runner(model_dirs[name], dtype, block_size, -(-200 // block_size))
+    steps = [{"entries": [{"id": "x", "tokens": [t], "want": [0]}], "end": []} for t in toks]
+    got = replay.run_trace(runner, steps)
+    ref = {"x": PlainQwen2(model_dirs[name]).logits(toks)}
+    replay.compare(got, ref, **TOL[dtype])
+
+
+def test_negative_control_a_small_weight_change_breaks_the_match(model_dirs, tmp_path):
+    """tests/test_hf_equivalence.py:141-153: the 1e-5 bar must bite. One q_proj row of layer 1
+    moved by 2^-7 is far more than the bar allows."""
+    from safetensors.torch import load_file, save_file
+
+    name = "A"
+    src = model_dirs[name]
+    tensors = load_file(str(src / "model.safetensors"))
+    tensors["model.layers.1.self_attn.q_proj.weight"] = tensors["model.layers.1.self_attn.q_proj.weight"].clone()
+    tensors["model.layers.1.self_attn.q_proj.weight"][:8] += 2.0 ** -7
+    dst = tmp_path / "perturbed"
+    dst.mkdir()
+    (dst / "config.json").write_text((src / "config.json").read_text())
+    save_file(tensors, str(dst / "model.safetensors"))
+    requests = {"r0": _requests(name)["r3"]}
+    runner = replay.make_runner(dst, "float32", 16, 8)
+    got = replay.run_trace(runner, replay.whole(requests))
+    with pytest.raises(AssertionError):
+        replay.compare(got, {"r0": _plain(name, model_dirs)["r3"]}, **TOL["float32"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model_dirs, tmp_path, dtype):
+    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and 'done <step>' out."""
+    name = "A"
+    requests = {k: v for k, v in list(_requests(name).items())[:5]}
+    steps = replay.mixed(requests)
+    lines = [json.dumps({"step": i, **s}) for i, s in enumerate(steps)]
+    max_tokens = 4 * 64 * -(-max(len(t) for t in requests.values()) // 64)
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, str(REPO / "bin" / "trace_run"), "--model", str(model_dirs[name]), "--dtype", dtype,
+         "--out", str(out), "--max-tokens", str(max_tokens)],
+        input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(len(steps))]
+    vocab = TINY_CONFIGS[name][0]["vocab_size"]
+    ref = _plain(name, model_dirs)
+    at = {rid: 0 for rid in requests}
+    for i, s in enumerate(steps):
+        rows = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, vocab)
+        r = 0
+        for e in s["entries"]:
+            for w in e["want"]:
+                want = ref[e["id"]][at[e["id"]] + w]
+                torch.testing.assert_close(torch.from_numpy(rows[r]), want, **TOL[dtype])
+                r += 1
+            at[e["id"]] += len(e["tokens"])
+        assert r == rows.shape[0]
