@@ -1,0 +1,211 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16]
+
+Default workload: the layer sizes of Qwen2.5-1.5B with random weights (seed 2), bfloat16,
+8 requests that each hold a 2048-token prompt, context limit 4096, pages of 16 tokens. A
+"step" is one decode step of the whole batch through the engine's own loop (scheduler, step
+function, sampling kernels; greedy). Prints one JSON line: ``value`` is decoded tokens a second
+at the default batch; ``prefill`` is one 2048-token prompt; ``roofline`` prices the decode step
+against HBM bandwidth; ``points`` holds decode at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+QWEN25_1P5B = dict(
+    model_type="qwen2", architectures=["Qwen2ForCausalLM"], vocab_size=151936, hidden_size=1536,
+    num_hidden_layers=28, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960,
+    rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True, hidden_act="silu",
+    use_sliding_window=False, max_position_embeddings=32768,
+)
+FULL_LAYERS = QWEN25_1P5B["num_hidden_layers"]
+PROMPT_LEN = 2048
+CONTEXT = 4096
+BLOCK = 16
+
+
+def _sync():
+    import torch
+
+    torch.cuda.synchronize()
+
+
+def build_runner(args):
+    from clockwork_amd.config.engine import EngineConfig
+    from clockwork_amd.engine.model_runner import ModelRunner
+    from clockwork_amd.parts.model import model_param_specs
+    from clockwork_amd.registry import resolve_architecture
+    from clockwork_amd.weights.random_init import RandomSource
+
+    config = dict(QWEN25_1P5B, num_hidden_layers=args.layers)
+    arch = resolve_architecture(config)
+    mcfg = arch.parse_config(config)
+    spec = arch.build_spec(mcfg)
+    source = RandomSource(arch.weight_plan(mcfg, spec), model_param_specs(spec), seed=2, device="cuda")
+    max_batch = max(args.batch, 64)
+    cfg = EngineConfig.defaults(
+        "random:qwen2.5-1.5b", dtype=args.dtype, max_model_len=CONTEXT, block_size=BLOCK,
+        num_blocks=max_batch * CONTEXT // BLOCK, enable_prefix_cache=False, watermark=0.0,
+        max_num_seqs=max_batch, max_num_batched_tokens=max(PROMPT_LEN, max_batch),
+    )
+    return cfg, ModelRunner(cfg, weight_source=source, config_dict=config)
+
+
+def time_decode(cfg, runner, batch: int, steps: int, warmup: int):
+    """Prefill ``batch`` prompts of PROMPT_LEN tokens, then time ``steps`` decode steps."""
+    import torch
+
+    from clockwork_amd.engine.llm_engine import LLMEngine
+    from clockwork_amd.engine.sequence import SamplingParams
+
+    engine = LLMEngine(cfg, runner=runner)
+    gen = torch.Generator().manual_seed(batch)
+    vocab = runner.spec.vocab_size
+    params = SamplingParams(max_tokens=warmup + steps + batch + 2, temperature=0.0, ignore_eos=True)
+    for i in range(batch):
+        engine.add_request(f"b{batch}-{i}", prompt_token_ids=torch.randint(0, vocab, (PROMPT_LEN,), generator=gen).tolist(),
+                           sampling_params=params)
+    while any(s.is_prefilling() or s.num_computed_tokens == 0 for s in engine.scheduler.running + engine.scheduler.waiting):
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    _sync()
+    seqs = list(engine.scheduler.running)
+    assert len(seqs) == batch and all(s.num_uncomputed_tokens() == 1 for s in seqs)
+    ctx_begin = sum(len(s) for s in seqs) / batch
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        outs = engine.step()
+        assert len(outs) == batch
+    _sync()
+    elapsed = time.perf_counter() - t0
+    for i in range(batch):
+        engine.abort_request(f"b{batch}-{i}")
+    mean_ctx = ctx_begin + (steps - 1) / 2.0  # keys a request reads in the middle step
+    return elapsed, mean_ctx
+
+
+def time_prefill(cfg, runner, repeats: int = 3):
+    import torch
+
+    from clockwork_amd.engine.batch import StepEntry
+
+    vocab = runner.spec.vocab_size
+    tokens = torch.randint(0, vocab, (PROMPT_LEN,), generator=torch.Generator().manual_seed(99)).tolist()
+    best = None
+    for i in range(repeats + 1):
+        runner.reserve("prefill", 0, PROMPT_LEN)
+        _sync()
+        t0 = time.perf_counter()
+        logits = runner.step([StepEntry("prefill", 0, tokens, [PROMPT_LEN - 1])])
+        _sync()
+        dt = time.perf_counter() - t0
+        runner.release("prefill")
+        if i > 0:  # the first run pays for library heuristics and allocations
+            best = dt if best is None else min(best, dt)
+    assert logits.shape == (1, vocab)
+    return best
+
+
+def prefill_flops(spec, model, T: int) -> float:
+    """2 * T * (matrix parameters of the layers) + causal attention + one row of the output head."""
+    layer_params = 0
+    for name, t in model.params.items():
+        if name.startswith("layers.") and t.dim() == 2:
+            layer_params += t.numel()
+    info = spec.info
+    attn = 4.0 * info["head_dim"] * info["heads"] * (T * (T + 1) / 2.0) * info["layers"]
+    head = 2.0 * info["hidden"] * info["vocab"]
+    return 2.0 * T * layer_params + attn + head
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
+        return 2
+
+    import torch
+
+    cfg, runner = build_runner(args)
+    elapsed, mean_ctx = time_decode(cfg, runner, args.batch, args.steps, args.warmup)
+    value = args.batch * args.steps / elapsed
+    ms = 1e3 * elapsed / args.steps
+    step_bytes = runner.model.weight_bytes_per_step() + args.batch * mean_ctx * runner.pools.kv_bytes_per_token()
+    achieved = step_bytes / (elapsed / args.steps) / 1e9
+
+    record = {
+        "metric": "decode tok/s, Qwen2.5-1.5B shape, batch 8, 2048-token prompts",
+        "value": round(value, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: uniform random token ids, random weights (seed 2)",
+        "config": {
+            "model": "Qwen2.5-1.5B shape (random weights)",
+            "layers": args.layers,
+            "layers_of_full_model": FULL_LAYERS,
+            "hidden": runner.spec.info["hidden"],
+            "heads": runner.spec.info["heads"],
+            "kv_heads": runner.spec.info["kv_heads"],
+            "head_dim": runner.spec.info["head_dim"],
+            "intermediate": runner.spec.info["intermediate"],
+            "vocab": runner.spec.info["vocab"],
+            "tied_embeddings": runner.spec.info["tied"],
+            "global_batch": args.batch,
+            "prompt_len": PROMPT_LEN,
+            "seq_len": CONTEXT,
+            "block_size": BLOCK,
+            "sampling": "greedy",
+            "parallelism": "single GPU",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": PEAK_HBM_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / PEAK_HBM_GBS, 4),
+        },
+    }
+    if not args.no_points:
+        t = time_prefill(cfg, runner)
+        flops = prefill_flops(runner.spec, runner.model, PROMPT_LEN)
+        record["prefill"] = {
+            "value": round(PROMPT_LEN / t, 1),
+            "tokens": PROMPT_LEN,
+            "ms": round(1e3 * t, 3),
+            "frac": round(flops / t / PEAK_FLOPS[args.dtype], 4),
+        }
+        points = {}
+        for b in (1, 64):
+            e, _ = time_decode(cfg, runner, b, args.steps, args.warmup)
+            points[f"decode_b{b}"] = round(b * args.steps / e, 1)
+        record["points"] = points
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
