@@ -91,6 +91,7 @@ class StepContext:
         self.h_q_lens: list[int] = []
         self.h_ctx_lens: list[int] = []
         self.h_starts: list[int] = []
+        self.h_state_slots: list[int] = []
         self.seq_ids: list[str] = []
         self._plans: dict = {}
         self.num_compute_units = 256
@@ -173,6 +174,7 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int
     i_ctx = packer.add(ctx.h_ctx_lens)
     i_start = packer.add(ctx.h_starts)
     i_state = packer.add(state_slots)
+    ctx.h_state_slots = state_slots
     i_rows = packer.add(logit_rows)
     group_idx = []
     for g in range(len(manager.kv_groups)):

@@ -1,0 +1,231 @@
+"""Generation through the entry point: scheduler, step function, sampling, prefix cache and
+preemption together, against the plain implementation and against each request run alone."""
+
+import pytest
+import torch
+
+from clockwork_amd.config.engine import EngineConfig
+from clockwork_amd.engine.sequence import SamplingParams
+from tests.configs import TINY_CONFIGS
+from tests.plain.qwen2_plain import PlainQwen2
+
+pytestmark = pytest.mark.gpu
+
+
+def engine(model_dir, **overrides):
+    from clockwork_amd.engine.llm_engine import LLMEngine
+
+    defaults = dict(dtype="float32", block_size=4, num_blocks=128, watermark=0.0)
+    defaults.update(overrides)
+    return LLMEngine(EngineConfig.defaults(str(model_dir), **defaults))
+
+
+def prompts_for(name, lengths, seed=0):
+    vocab = TINY_CONFIGS[name][0]["vocab_size"]
+    gen = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, vocab, (n,), generator=gen).tolist() for n in lengths]
+
+
+def greedy(n):
+    return SamplingParams(max_tokens=n, temperature=0.0, ignore_eos=True)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_greedy_generation_equals_the_plain_implementation(model_dirs, name):
+    # prompt lengths 1, 3, 9, 17 and 24 greedy tokens: tests/test_hf_equivalence.py:14,17,108-113
+    prompts = prompts_for(name, [1, 3, 9, 17])
+    plain = PlainQwen2(model_dirs[name])
+    outs = engine(model_dirs[name]).generate(prompts, greedy(24))
+    for prompt, out in zip(prompts, outs):
+        assert out.token_ids == plain.greedy(prompt, 24)
+        assert out.finished and out.finish_reason == "length" and out.num_generated_tokens == 24
+        assert out.prompt_token_ids == prompt
+
+
+def test_bfloat16_generation_follows_the_plain_implementation(model_dirs):
+    name = "B"
+    prompts = prompts_for(name, [5, 40])
+    plain = PlainQwen2(model_dirs[name])
+    outs = engine(model_dirs[name], dtype="bfloat16").generate(prompts, greedy(8))
+    for prompt, out in zip(prompts, outs):
+        want = plain.greedy(prompt, 8)
+        # bfloat16 may flip a near-tie; up to the first flip the tokens agree, and a flip must be a near-tie
+        for i, (a, b) in enumerate(zip(out.token_ids, want)):
+            if a != b:
+                row = plain.logits(prompt + want[:i])[-1]
+                assert float(row[b] - row[a]) < 0.05
+                break
+
+
+def test_eight_staggered_requests_equal_each_alone(model_dirs):
+    # tests/test_llm_engine.py:94-131: a budget of 32 tokens forces portions and mixed steps
+    name = "A"
+    prompts = prompts_for(name, [12, 30, 7, 45, 3, 19, 26, 50], seed=3)
+    alone = [engine(model_dirs[name]).generate([p], greedy(10))[0].token_ids for p in prompts[:3]]
+    plain = PlainQwen2(model_dirs[name])
+    e = engine(model_dirs[name], max_num_batched_tokens=32, enable_prefix_cache=False)
+    finals = {}
+    pending = list(enumerate(prompts))
+    for step in range(400):
+        if pending and step % 2 == 0:
+            i, p = pending.pop(0)
+            e.add_request(f"r{i}", prompt_token_ids=p, sampling_params=greedy(10))
+        for out in e.step():
+            if out.finished:
+                finals[out.request_id] = out.token_ids
+        if not pending and not e.has_unfinished_requests():
+            break
+    assert len(finals) == 8
+    for i, p in enumerate(prompts):
+        assert finals[f"r{i}"] == plain.greedy(p, 10), f"request {i}"
+    assert [finals[f"r{i}"] for i in range(3)] == alone
+    assert e.manager.min_free_blocks() == 128
+
+
+def test_prefix_cache_second_pass_is_identical_and_counts_cached_tokens(model_dirs):
+    # tests/test_llm_engine.py:134-165: lengths [12, 10, 15, 8], pages of 4 -> cached [8, 8, 12, 4]
+    name = "A"
+    prompts = prompts_for(name, [12, 10, 15, 8], seed=5)
+    e = engine(model_dirs[name])
+    first = e.generate(prompts, greedy(6))
+    assert [o.num_cached_tokens for o in first] == [0, 0, 0, 0]
+    second = e.generate(prompts, greedy(6))
+    assert [o.num_cached_tokens for o in second] == [8, 8, 12, 4]
+    assert [o.token_ids for o in second] == [o.token_ids for o in first]
+    off = engine(model_dirs[name], enable_prefix_cache=False).generate(prompts, greedy(6))
+    assert [o.token_ids for o in off] == [o.token_ids for o in first]
+    assert e.stats()["prefix_cache_hit_tokens"] == 32
+
+
+def test_shared_prefix_accounting(model_dirs):
+    # tests/test_llm_engine.py:168-200: four 19-token prompts sharing 16 tokens, one at a time
+    name = "A"
+    shared = prompts_for(name, [16], seed=9)[0]
+    prompts = [shared + [i + 1, i + 2, i + 3] for i in range(4)]
+    e = engine(model_dirs[name])
+    plain = PlainQwen2(model_dirs[name])
+    for p in prompts:
+        out = e.generate([p], greedy(4))[0]
+        assert out.token_ids == plain.greedy(p, 4)
+    s = e.stats()
+    assert (s["prefix_cache_queries"], s["prefix_cache_prompt_tokens"], s["prefix_cache_hit_tokens"]) == (4, 76, 48)
+    assert s["prefix_cache_hit_rate"] == 48 / 76
+
+
+def test_preemption_leaves_outputs_unchanged(model_dirs):
+    # tests/test_llm_engine.py:203-219: 8 pages of 4, three requests of 8 + 8 tokens
+    name = "A"
+    prompts = prompts_for(name, [8, 8, 8], seed=11)
+    plain = PlainQwen2(model_dirs[name])
+    e = engine(model_dirs[name], num_blocks=8, enable_prefix_cache=False)
+    outs = e.generate(prompts, greedy(8))
+    assert e.stats()["num_preempted_total"] > 0
+    for p, o in zip(prompts, outs):
+        assert o.token_ids == plain.greedy(p, 8)
+    assert e.manager.min_free_blocks() == 8
+
+
+def test_a_request_that_can_never_fit_is_an_error(model_dirs):
+    e = engine(model_dirs["A"], num_blocks=2, enable_prefix_cache=False)
+    e.add_request("big", prompt_token_ids=list(range(12)))
+    with pytest.raises(RuntimeError, match="cannot be admitted"):
+        e.step()
+
+
+def test_seeded_sampling_is_reproducible_and_seeds_differ(model_dirs):
+    # tests/test_llm_engine.py:222-236
+    name = "B"
+    prompt = prompts_for(name, [9], seed=2)
+
+    def run(seed, **kw):
+        params = SamplingParams(max_tokens=12, temperature=1.5, seed=seed, ignore_eos=True, **kw)
+        return engine(model_dirs[name]).generate(prompt, params)[0].token_ids
+
+    assert run(1) == run(1)
+    assert run(1) != run(2)
+    assert run(1, top_k=1) == PlainQwen2(model_dirs[name]).greedy(prompt[0], 12)  # tests/test_server.py:323
+    # a request samples the same tokens alone and in a crowd
+    e = engine(model_dirs[name], max_num_batched_tokens=16)
+    crowd = prompts_for(name, [20, 5, 33], seed=4)
+    e.add_request("x", prompt_token_ids=prompt[0], sampling_params=SamplingParams(max_tokens=12, temperature=1.5, seed=1, ignore_eos=True))
+    for i, p in enumerate(crowd):
+        e.add_request(f"c{i}", prompt_token_ids=p, sampling_params=SamplingParams(max_tokens=9, temperature=0.7, seed=i, ignore_eos=True))
+    got = None
+    while e.has_unfinished_requests():
+        for out in e.step():
+            if out.finished and out.request_id == "x":
+                got = out.token_ids
+    assert got == run(1)
+
+
+def test_finish_rules(model_dirs):
+    # tests/test_llm_engine.py:239-296
+    name = "A"
+    prompt = prompts_for(name, [10], seed=6)[0]
+    free = engine(model_dirs[name]).generate([prompt], greedy(8))[0].token_ids
+    stop_at = free[3]
+    first = free.index(stop_at)
+    out = engine(model_dirs[name]).generate([prompt], SamplingParams(max_tokens=8, stop_token_ids=[stop_at]))[0]
+    assert out.finish_reason == "stop" and out.token_ids == free[: first + 1]  # the stop token stays in the ids
+    cfg_eos = dict(TINY_CONFIGS[name][0], eos_token_id=stop_at)
+    from clockwork_amd.engine.llm_engine import LLMEngine
+
+    e = LLMEngine(EngineConfig.defaults(str(model_dirs[name]), block_size=4, num_blocks=64), config_dict=cfg_eos)
+    assert e.generate([prompt], SamplingParams(max_tokens=8))[0].token_ids == free[: first + 1]
+    e = LLMEngine(EngineConfig.defaults(str(model_dirs[name]), block_size=4, num_blocks=64), config_dict=cfg_eos)
+    assert e.generate([prompt], SamplingParams(max_tokens=8, ignore_eos=True))[0].token_ids == free
+    # max_model_len 16 with a 10-token prompt: 6 tokens, "length"
+    out = engine(model_dirs[name], max_model_len=16).generate([prompt], greedy(50))[0]
+    assert out.num_generated_tokens == 6 and out.finish_reason == "length"
+    with pytest.raises(ValueError, match="leaves no room"):
+        engine(model_dirs[name], max_model_len=10).add_request("x", prompt_token_ids=prompt)
+
+
+class IntTokenizer:
+    """Token i is the text "<i>" (tests/test_llm_engine.py:17-27 uses a fake of this kind)."""
+
+    eos_token_id = None
+
+    def encode(self, text):
+        return [int(t) for t in text.replace(">", "").split("<") if t]
+
+    def decode(self, ids, skip_special_tokens=True):
+        return "".join(f"<{i}>" for i in ids)
+
+
+def test_text_prompts_and_stop_strings_need_and_use_a_tokenizer(model_dirs):
+    from clockwork_amd.engine.llm_engine import LLMEngine
+
+    name = "A"
+    prompt = prompts_for(name, [6], seed=8)[0]
+    cfg = EngineConfig.defaults(str(model_dirs[name]), block_size=4, num_blocks=64)
+    free = LLMEngine(cfg).generate([prompt], greedy(6))[0].token_ids
+    e = LLMEngine(cfg, tokenizer=IntTokenizer())
+    text_prompt = "".join(f"<{t}>" for t in prompt)
+    out = e.generate([text_prompt], SamplingParams(max_tokens=6, stop=[f"<{free[2]}>"], ignore_eos=True))[0]
+    cut = free.index(free[2])
+    assert out.finish_reason == "stop" and out.text == "".join(f"<{t}>" for t in free[:cut])
+    with pytest.raises(ValueError, match="tokenizer"):
+        LLMEngine(cfg).add_request("t", prompt="<1><2>")
+    with pytest.raises(ValueError, match="exactly one"):
+        e.add_request("t")
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        e.add_request("t", prompt_token_ids=[999999])
+
+
+def test_command_line(model_dirs, tmp_path, capsys):
+    from clockwork_amd import cli
+
+    name = "A"
+    prompt = prompts_for(name, [7], seed=10)[0]
+    yaml_path = tmp_path / "engine.yaml"
+    yaml_path.write_text(f"model:\n  model: {model_dirs[name]}\ncache:\n  block_size: 4\n  num_blocks: 64\n")
+    rc = cli.main(["--config", str(yaml_path), "--set", "dtype=float32", "--prompt-ids", ",".join(map(str, prompt)),
+                   "--max-tokens", "5", "--ignore-eos"])
+    assert rc == 0
+    import json
+
+    line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert line["token_ids"] == PlainQwen2(model_dirs[name]).greedy(prompt, 5)
+    with pytest.raises(SystemExit):
+        cli.main(["--config", str(yaml_path), "--set", "nonsense=1", "--prompt-ids", "1"])

@@ -1,0 +1,287 @@
+"""Each part alone against the plain formulas, and the framework's openness: toy parts and a toy
+architecture defined here are registered, built from a model folder and stepped without any
+change to the framework's files (a mixer with state of its own, windowed attention in a group
+of its own, a layer that runs twice, a layer that reads another layer's cache)."""
+
+import json
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+from clockwork_amd.config.spec import LayerSpec, ModelSpec, ParamSpec, RunEntry, StateSpec, WeightTarget
+from clockwork_amd.parts.specs import AttentionSpec, RMSNormSpec, RopeNeoxSpec, SwiGLUSpec
+from clockwork_amd.registry import Architecture, build_part, register_architecture, register_part
+from tests import replay
+from tests.plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _bind(part, dtype, scale=0.1, seed=0):
+    gen = torch.Generator().manual_seed(seed)
+    params = {}
+    for name, spec in part.param_specs().items():
+        t = torch.randn(spec.shape, generator=gen) * scale
+        if spec.init[0] == "one_plus_uniform":
+            t = 1 + t
+        params[name] = t.to(dtype).to(DEV)
+    part.bind(params, torch.device(DEV), dtype)
+    return {k: v.float().cpu() for k, v in params.items()}
+
+
+TOL = {torch.float32: dict(rtol=1e-5, atol=1e-5), torch.bfloat16: dict(rtol=3e-2, atol=3e-2)}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    part = build_part(RMSNormSpec(size=100, eps=2e-6))
+    w = _bind(part, dtype)
+    resid = torch.randn(6, 100, device=DEV)
+    delta = torch.randn(6, 100, device=DEV).to(dtype)
+    before = resid.clone()
+    out = part.forward(resid, delta)
+    torch.testing.assert_close(resid, before + delta.float())
+    torch.testing.assert_close(out.float().cpu(), plain.rmsnorm(resid.cpu(), w["weight"], 2e-6), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    part = build_part(SwiGLUSpec(hidden_size=80, intermediate_size=100))
+    w = _bind(part, dtype)
+    x = torch.randn(5, 80, device=DEV).to(dtype)
+    got = part.forward(x, None)
+    gu = w["gate_up_weight"]
+    want = plain.swiglu(x.float().cpu(), gu[:100], gu[100:], w["down_weight"])
+    torch.testing.assert_close(got.float().cpu(), want, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [None, 7])
+def test_attention_part_whole_and_in_portions(dtype, window):
+    """The mixer alone, through the real cache manager and pools: a sequence run whole, then the
+    same sequence in portions and single tokens, against the plain formulas."""
+    from clockwork_amd.cache import CacheManager, plan_groups
+    from clockwork_amd.cache.pools import CachePools
+    from clockwork_amd.engine.batch import StepEntry, build_context
+
+    spec = AttentionSpec(hidden_size=72, num_heads=6, num_kv_heads=2, head_dim=48, qkv_bias=True, out_bias=True,
+                         scale=0.2, window=window, position=RopeNeoxSpec(rotary_dim=48, theta=5000.0))
+    part = build_part(spec)
+    # the expected values are computed in float64, so all of the allowed error is the engine's
+    w = {k: v.double() for k, v in _bind(part, dtype, scale=0.12).items()}
+    T = 41
+    x = torch.randn(T, 72).to(dtype)
+    xf = x.double()
+    qkv = plain.linear(xf, w["qkv_weight"], w["qkv_bias"])
+    q, k, v = qkv[:, :288].view(T, 6, 48), qkv[:, 288:384].view(T, 2, 48), qkv[:, 384:].view(T, 2, 48)
+    cos, sin = plain.rope_tables(torch.arange(T), 48, 5000.0, torch.float64)
+    a = plain.attention_dense(plain.apply_rope(q, cos, sin), plain.apply_rope(k, cos, sin), v, 0.2, window=window)
+    want = plain.linear(a.reshape(T, 288), w["out_weight"], w["out_bias"]).float()
+
+    for cuts in ([T], [5, 1, 1, 17, 2, 1, 14]):
+        groups = plan_groups([part.cache_need()])
+        manager = CacheManager(groups, 8, 12)
+        pools = CachePools(groups, 8, 12, 4, dtype, torch.device(DEV), fill=float("nan"))
+        cache = pools.entry_cache(0)
+        got, at = [], 0
+        for n in cuts:
+            if at == 0:
+                manager.admit("s", n)
+            manager.extend("s", at, at + n)
+            ctx = build_context([StepEntry("s", at, [0] * n)], manager, torch.device(DEV), 10)
+            got.append(part.forward(x[at : at + n].to(DEV), ctx, cache))
+            at += n
+            manager.release_behind_window("s", at)
+        torch.testing.assert_close(torch.cat(got).float().cpu(), want, **TOL[dtype])
+
+
+# ---------------------------------------------------------------------------------- toy parts
+@dataclass(frozen=True)
+class EmaMixerSpec:
+    """y_t = s_t with s_t = decay * s_{t-1} + (1 - decay) * (x_t W): a recurrence whose only cache
+    is a fixed-size state per request."""
+
+    hidden_size: int
+    decay: float
+
+
+class EmaMixer:
+    def __init__(self, spec):
+        self.spec = spec
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.spec.hidden_size, self.spec.hidden_size))}
+
+    def cache_need(self):
+        return StateSpec((self.spec.hidden_size,), "float32")
+
+    def bind(self, params, device, dtype):
+        self.weight = params["weight"]
+
+    def forward(self, x, ctx, cache):
+        u = (x.float() @ self.weight.float().t())
+        out = torch.empty_like(u)
+        at = 0
+        for r, n in enumerate(ctx.h_q_lens):
+            slot = ctx.h_state_slots[r]
+            s = cache.state[slot]
+            for t in range(at, at + n):
+                s = self.spec.decay * s + (1 - self.spec.decay) * u[t]
+                out[t] = s
+            cache.state[slot] = s
+            at += n
+        return out.to(x.dtype)
+
+
+@dataclass(frozen=True)
+class ToyConfig:
+    vocab: int
+    hidden: int
+    kinds: tuple
+    window: int
+    eps: float
+
+
+def _toy_spec(cfg: ToyConfig) -> ModelSpec:
+    norm = RMSNormSpec(cfg.hidden, cfg.eps)
+    ffn = SwiGLUSpec(cfg.hidden, 2 * cfg.hidden)
+    rope = RopeNeoxSpec(rotary_dim=16, theta=1000.0)
+
+    def attn(window):
+        return AttentionSpec(cfg.hidden, 4, 2, 16, True, False, 0.25, window=window, position=rope)
+
+    layers, run = [], []
+    for kind in cfg.kinds:
+        if kind == "again":       # the previous layer's weights once more, with a cache of its own
+            run.append(RunEntry(layer=len(layers) - 1))
+            continue
+        if kind == "borrow":      # a layer that makes queries only and reads the first entry's keys
+            layers.append(LayerSpec("prenorm", attn(None), ffn, norm, norm))
+            run.append(RunEntry(layer=len(layers) - 1, cache_from=0))
+            continue
+        mixer = {"full": attn(None), "window": attn(cfg.window), "ema": EmaMixerSpec(cfg.hidden, 0.75)}[kind]
+        layers.append(LayerSpec("prenorm", mixer, ffn, norm, norm))
+        run.append(RunEntry(layer=len(layers) - 1))
+    return ModelSpec("ToyForCausalLM", cfg.vocab, cfg.hidden, layers, run, norm, tie_embeddings=True)
+
+
+def _toy_plan(cfg: ToyConfig, spec: ModelSpec):
+    """The toy's checkpoint simply uses the model's own parameter names."""
+    from clockwork_amd.parts.model import model_param_specs
+
+    plan = []
+    for name, p in model_param_specs(spec).items():
+        plan.append(WeightTarget(name, (name,), (tuple(p.shape),), optional=(name == "lm_head.weight")))
+    return plan
+
+
+@pytest.fixture(scope="module")
+def toy_dir(tmp_path_factory):
+    from clockwork_amd.weights.random_init import write_random_model
+
+    register_part(EmaMixerSpec, EmaMixer)
+    register_architecture(
+        ["ToyForCausalLM"],
+        Architecture(
+            "ToyForCausalLM",
+            parse_config=lambda d: ToyConfig(d["vocab"], d["hidden"], tuple(d["kinds"]), d["window"], d["eps"]),
+            build_spec=_toy_spec,
+            weight_plan=_toy_plan,
+        ),
+    )
+    config = {"architectures": ["ToyForCausalLM"], "vocab": 300, "hidden": 64, "window": 6, "eps": 1e-5,
+              "kinds": ["full", "window", "again", "ema", "borrow"]}
+    return write_random_model(tmp_path_factory.mktemp("toy") / "toy", config, seed=3)
+
+
+def _toy_plain_logits(model_dir, tokens):
+    """The toy model from the plain formulas, whole sequence, no cache."""
+    from safetensors.torch import load_file
+
+    cfg = json.loads((model_dir / "config.json").read_text())
+    w = {k: v.float() for k, v in load_file(str(model_dir / "model.safetensors")).items()}
+    T, H = len(tokens), cfg["hidden"]
+    h = plain.embedding(w["embed.weight"], torch.tensor(tokens))
+    cos, sin = plain.rope_tables(torch.arange(T), 16, 1000.0)
+    layer_of, kv_of, run = [], {}, []
+    n_layers = 0
+    for kind in cfg["kinds"]:
+        if kind == "again":
+            run.append((n_layers - 1, run[-1][1], None))
+            continue
+        run.append((n_layers, kind, 0 if kind == "borrow" else None))
+        n_layers += 1
+    for i, (layer, kind, borrow) in enumerate(run):
+        p = f"layers.{layer}."
+        x = plain.rmsnorm(h, w[p + "mixer_norm.weight"], cfg["eps"])
+        if kind == "ema":
+            u = x @ w[p + "mixer.weight"].t()
+            s = torch.zeros(H)
+            rows = []
+            for t in range(T):
+                s = 0.75 * s + 0.25 * u[t]
+                rows.append(s)
+            a = torch.stack(rows)
+        else:
+            qkv = plain.linear(x, w[p + "mixer.qkv_weight"], w[p + "mixer.qkv_bias"])
+            q = plain.apply_rope(qkv[:, :64].view(T, 4, 16), cos, sin)
+            if borrow is None:
+                k = plain.apply_rope(qkv[:, 64:96].view(T, 2, 16), cos, sin)
+                v = qkv[:, 96:].view(T, 2, 16)
+                kv_of[i] = (k, v)
+            else:
+                k, v = kv_of[borrow]
+            window = cfg["window"] if kind == "window" else None
+            a = plain.linear(plain.attention_dense(q, k, v, 0.25, window=window).reshape(T, 64), w[p + "mixer.out_weight"])
+        h = h + a
+        x = plain.rmsnorm(h, w[p + "ffn_norm.weight"], cfg["eps"])
+        gu = w[p + "feed_forward.gate_up_weight"]
+        h = h + plain.swiglu(x, gu[: 2 * H], gu[2 * H :], w[p + "feed_forward.down_weight"])
+    return plain.linear(plain.rmsnorm(h, w["final_norm.weight"], cfg["eps"]), w["embed.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["whole", "prefill_then_decode", "portions", "mixed"])
+def test_a_toy_architecture_registers_builds_and_steps(toy_dir, dtype, mode):
+    gen = torch.Generator().manual_seed(5)
+    requests = {f"t{i}": torch.randint(0, 300, (n,), generator=gen).tolist() for i, n in enumerate([50, 9, 77, 30, 64])}
+    runner = replay.make_runner(toy_dir, dtype, 8, 64)
+    # three groups: all keys (two entries + a borrower), a window (two entries: the layer and its rerun), a state
+    assert [(g.is_kv, g.window, g.entries) for g in runner.manager.groups] == [(True, None, (0,)), (True, 6, (1, 2)), (False, None, (3,))]
+    assert not runner.manager.supports_prefix_sharing
+    got = replay.run_trace(runner, getattr(replay, mode)(requests))
+    ref = {rid: _toy_plain_logits(toy_dir, toks) for rid, toks in requests.items()}
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == "float32" else dict(rtol=3e-2, atol=3e-2)
+    replay.compare(got, ref, **tol)
+    assert not runner.manager.live_requests()
+    assert [p.num_free for p in runner.manager.pools] == [64, 64]
+
+
+def test_windowed_group_uses_few_pages_for_a_long_request(toy_dir):
+    runner = replay.make_runner(toy_dir, "float32", 8, 64)
+    toks = torch.randint(0, 300, (200,), generator=torch.Generator().manual_seed(6)).tolist()
+    runner.reserve("x", 0, 100)
+    from clockwork_amd.engine.batch import StepEntry
+
+    runner.step([StepEntry("x", 0, toks[:100], [])])
+    for p in range(100, 200):
+        runner.reserve("x", p, 1)
+        runner.step([StepEntry("x", p, toks[p : p + 1], [])])
+        assert 64 - runner.manager.pools[1].num_free <= 2  # a window of 6 tokens spans at most two pages of 8
+    assert 64 - runner.manager.pools[0].num_free == 25
+    runner.release("x")
+
+
+def test_unknown_parts_and_architectures_are_refused():
+    @dataclass(frozen=True)
+    class Unknown:
+        x: int = 0
+
+    with pytest.raises(KeyError, match="no part is registered"):
+        build_part(Unknown())
+    from clockwork_amd.registry import resolve_architecture
+
+    with pytest.raises(ValueError, match="expected a qwen2 model"):
+        resolve_architecture({"architectures": ["NopeForCausalLM"], "model_type": "nope"})

@@ -1,0 +1,348 @@
+"""The scheduler's decisions on the CPU, with a stand-in for the step function.
+
+Vectors of the reference's scheduler tests (tests/test_scheduler.py) run with chunked prefill
+off, where our scheduler must decide exactly as the reference does; the rest covers what is
+new: portions under the token budget, and what happens when pages run out."""
+
+import pytest
+
+from clockwork_amd.cache import CacheManager, PrefixCache, plan_groups
+from clockwork_amd.config.engine import SchedulerConfig
+from clockwork_amd.config.spec import KVPagesSpec
+from clockwork_amd.engine.scheduler import Scheduler
+from clockwork_amd.engine.sequence import SamplingParams, Sequence, SequenceStatus
+
+BS = 4
+
+
+def make_env(num_blocks=64, max_num_seqs=8, budget=64, watermark=0.0, prefix=False, chunked=False, chunk=0):
+    manager = CacheManager(plan_groups([KVPagesSpec(1, 16)]), BS, num_blocks, max_num_seqs, watermark)
+    cache = PrefixCache(BS, manager.share_handle, manager.drop_handle) if prefix else None
+    cfg = SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=budget,
+                          enable_chunked_prefill=chunked, max_prefill_chunk=chunk)
+    return Scheduler(cfg, manager, cache), manager, cache
+
+
+def make_seq(seq_id, prompt, arrival, max_tokens=64):
+    return Sequence(seq_id, list(prompt), SamplingParams(max_tokens=max_tokens), arrival_time=arrival)
+
+
+def apply(sched, out):
+    """What the engine does after a step: mark the portion computed, append a token where one
+    was sampled, finish at max_tokens, give back what finished requests held."""
+    for p in out.portions:
+        p.seq.num_computed_tokens = p.start + p.num_tokens
+        if p.samples:
+            p.seq.append_token(7)
+            if len(p.seq.output_token_ids) >= p.seq.sampling_params.max_tokens:
+                p.seq.status = SequenceStatus.FINISHED_LENGTH
+    sched.free_finished()
+
+
+def engine_step(sched):
+    out = sched.schedule()
+    apply(sched, out)
+    return out
+
+
+def ids(seqs):
+    return [s.seq_id for s in seqs]
+
+
+# ------------------------------------------------------------------ the reference's vectors
+def test_token_budget_splits_a_batch():
+    # tests/test_scheduler.py:49-67
+    sched, _, _ = make_env(budget=10)
+    a, b = make_seq("a", range(6), 0.0), make_seq("b", range(6), 1.0)
+    sched.add_seq(a)
+    sched.add_seq(b)
+    out1 = sched.schedule()
+    assert ids(out1.prefill_seqs) == ["a"] and out1.decode_seqs == [] and out1.num_batched_tokens == 6
+    assert b.status is SequenceStatus.WAITING
+    apply(sched, out1)
+    out2 = sched.schedule()
+    assert ids(out2.decode_seqs) == ["a"] and ids(out2.prefill_seqs) == ["b"] and out2.num_batched_tokens == 7
+
+
+def test_max_num_seqs_cap():
+    sched, _, _ = make_env(max_num_seqs=2)
+    a, b, c = make_seq("a", range(4), 0.0, 1), make_seq("b", range(4), 1.0, 8), make_seq("c", range(4), 2.0, 8)
+    for s in (a, b, c):
+        sched.add_seq(s)
+    out1 = engine_step(sched)
+    assert ids(out1.prefill_seqs) == ["a", "b"] and c.status is SequenceStatus.WAITING and a.is_finished()
+    out2 = engine_step(sched)
+    assert ids(out2.decode_seqs) == ["b"] and ids(out2.prefill_seqs) == ["c"]
+
+
+def pressure_env(max_num_seqs=2):
+    # tests/test_scheduler.py:88-96: 6 pages; two 2-page prompts fit, decode growth runs the pool dry
+    sched, manager, _ = make_env(num_blocks=6, max_num_seqs=max_num_seqs)
+    a, b = make_seq("a", range(8), 0.0, 6), make_seq("b", range(100, 108), 1.0, 6)
+    sched.add_seq(a)
+    sched.add_seq(b)
+    return sched, manager, a, b
+
+
+def run_until_preemption(sched, limit=20):
+    for _ in range(limit):
+        out = engine_step(sched)
+        if out.preempted:
+            return out
+    raise AssertionError("no preemption occurred")
+
+
+def test_preemption_recompute_and_readmission():
+    sched, manager, a, b = pressure_env()
+    out = run_until_preemption(sched)
+    assert ids(out.preempted) == ["b"]  # the latest arrival is the victim
+    assert b.status is SequenceStatus.PREEMPTED and b.num_computed_tokens == 0 and not manager.has("b")
+    assert sched.waiting[0] is b and a in out.decode_seqs and sched.stats.num_preempted_total == 1
+    for _ in range(20):
+        if b.is_finished():
+            break
+        engine_step(sched)
+    assert b.status is SequenceStatus.FINISHED_LENGTH and len(b.output_token_ids) == 6
+    assert a.status is SequenceStatus.FINISHED_LENGTH and not sched.has_unfinished()
+    assert manager.num_free_blocks() == 6
+
+
+def test_preempted_requests_are_readmitted_before_newcomers():
+    sched, _, a, b = pressure_env()
+    c = make_seq("c", range(200, 204), 2.0, 2)
+    sched.add_seq(c)
+    run_until_preemption(sched)
+    assert ids(sched.waiting) == ["b", "c"]
+    for _ in range(20):
+        out = sched.schedule()
+        if out.prefill_seqs:
+            break
+        apply(sched, out)
+    assert out.prefill_seqs[0] is b and b.status is SequenceStatus.RUNNING
+
+
+def cached_env(budget):
+    sched, manager, cache = make_env(num_blocks=16, budget=budget, prefix=True)
+    tokens = list(range(100, 112))
+    handles = [(p,) for p in manager.pools[0].take_many(2)]
+    cache.insert(tokens[:8], handles)
+    for h in handles:
+        manager.drop_handle(h)
+    return sched, manager, cache, tokens, handles
+
+
+def test_prefix_hit_lowers_the_admission_cost():
+    # tests/test_scheduler.py:173-194
+    sched, manager, _, tokens, handles = cached_env(budget=6)
+    seq = make_seq("s", tokens, 0.0)
+    sched.add_seq(seq)
+    out = sched.schedule()
+    assert ids(out.prefill_seqs) == ["s"] and out.num_batched_tokens == 4
+    assert seq.num_cached_tokens == 8 and seq.num_computed_tokens == 8
+    assert manager.block_table("s")[:2] == [h[0] for h in handles] and len(manager.block_table("s")) == 3
+    assert sched.stats.total_cached_tokens == 8 and sched.stats.total_prompt_tokens == 12
+    cold_sched, _, _, _, _ = cached_env(budget=6)
+    cold = make_seq("cold", range(200, 212), 0.0)
+    cold_sched.add_seq(cold)
+    assert cold_sched.schedule().is_empty() and cold.status is SequenceStatus.WAITING
+
+
+def test_failed_admission_undoes_the_prefix_match():
+    # tests/test_scheduler.py:197-209
+    sched, manager, cache, tokens, handles = cached_env(budget=3)
+    seq = make_seq("s", tokens, 0.0)
+    sched.add_seq(seq)
+    assert sched.schedule().is_empty()
+    assert not manager.has("s") and seq.num_cached_tokens == 0 and seq.num_computed_tokens == 0
+    assert cache.evictable_blocks() == 2
+    assert all(manager.pools[0].refcount(h[0]) == 1 for h in handles)
+
+
+def test_abort_in_every_state():
+    sched, manager, _ = make_env()
+    a = make_seq("a", range(4), 0.0)
+    sched.add_seq(a)
+    sched.abort("a")
+    assert a.status is SequenceStatus.FINISHED_ABORTED and not sched.has_unfinished()
+    b = make_seq("b", range(6), 1.0)
+    sched.add_seq(b)
+    sched.schedule()
+    assert b.status is SequenceStatus.RUNNING
+    sched.abort("b")
+    assert b.status is SequenceStatus.FINISHED_ABORTED and sched.running == [] and manager.num_free_blocks() == 64
+    sched.abort("missing")  # a no-op
+    sched2, manager2, a2, b2 = pressure_env()
+    run_until_preemption(sched2)
+    sched2.abort("b")
+    assert b2.status is SequenceStatus.FINISHED_ABORTED and b2 not in sched2.waiting
+    for _ in range(20):
+        if not sched2.has_unfinished():
+            break
+        engine_step(sched2)
+    assert a2.is_finished() and manager2.num_free_blocks() == 6
+
+
+def test_abort_running_releases_prefix_locks():
+    sched, manager, cache, tokens, handles = cached_env(budget=64)
+    seq = make_seq("s", tokens, 0.0)
+    sched.add_seq(seq)
+    sched.schedule()
+    assert seq.num_cached_tokens == 8 and cache.evictable_blocks() == 0
+    sched.abort("s")
+    assert manager.num_free_blocks() == 14 and cache.evictable_blocks() == 2
+    assert all(manager.pools[0].refcount(h[0]) == 1 for h in handles)
+
+
+def scripted_session(chunked):
+    # tests/test_scheduler.py:270-301: 7 pages, budget 16; admission splits, preemptions, drain
+    sched, manager, _ = make_env(num_blocks=7, max_num_seqs=3, budget=16, chunked=chunked)
+    seqs = [make_seq("a", range(8), 0.0, 6), make_seq("b", range(100, 108), 1.0, 6),
+            make_seq("c", range(200, 204), 2.0, 4), make_seq("d", range(300, 312), 3.0, 3)]
+    for s in seqs:
+        sched.add_seq(s)
+    history = []
+    for _ in range(60):
+        out = engine_step(sched)
+        history.append((tuple((p.seq.seq_id, p.start, p.num_tokens) for p in out.portions),
+                        tuple(ids(out.preempted)), out.num_batched_tokens))
+        # pages are held only by running requests
+        assert set(manager.live_requests()) == {s.seq_id for s in sched.running}
+        if not sched.has_unfinished():
+            break
+    assert not sched.has_unfinished() and manager.num_free_blocks() == 7
+    assert [len(s.output_token_ids) for s in seqs] == [6, 6, 4, 3]
+    return history
+
+
+@pytest.mark.parametrize("chunked", [False, True])
+def test_a_scripted_session_is_deterministic_and_drains(chunked):
+    h = scripted_session(chunked)
+    assert h == scripted_session(chunked)
+    assert any(step[1] for step in h), "the session was meant to force a preemption"
+
+
+# ------------------------------------------------------------------ chunked prefill
+def test_a_prompt_longer_than_the_budget_runs_in_portions():
+    sched, manager, _ = make_env(budget=10, chunked=True)
+    a = make_seq("a", range(25), 0.0, 2)
+    sched.add_seq(a)
+    seen = []
+    for _ in range(6):
+        out = engine_step(sched)
+        seen.append([(p.start, p.num_tokens, p.samples) for p in out.portions])
+        if a.is_finished():
+            break
+    assert seen == [[(0, 10, False)], [(10, 10, False)], [(20, 5, True)], [(25, 1, True)]]
+    assert manager.num_free_blocks() == 64
+
+
+def test_decoding_requests_go_first_and_prefill_takes_the_rest_of_the_budget():
+    sched, _, _ = make_env(budget=8, chunked=True)
+    a, b = make_seq("a", range(3), 0.0, 10), make_seq("b", range(30), 1.0, 2)
+    sched.add_seq(a)
+    out = engine_step(sched)
+    assert [(p.seq.seq_id, p.num_tokens) for p in out.portions] == [("a", 3)]
+    sched.add_seq(b)
+    out = engine_step(sched)
+    assert [(p.seq.seq_id, p.start, p.num_tokens, p.samples) for p in out.portions] == [("a", 3, 1, True), ("b", 0, 7, False)]
+    assert ids(out.decode_seqs) == ["a"] and ids(out.prefill_seqs) == ["b"] and out.num_batched_tokens == 8
+    out = engine_step(sched)
+    assert [(p.seq.seq_id, p.start, p.num_tokens) for p in out.portions] == [("a", 4, 1), ("b", 7, 7)]
+
+
+def test_max_prefill_chunk_caps_a_portion_and_two_prompts_share_a_step():
+    sched, _, _ = make_env(budget=64, chunked=True, chunk=5)
+    a, b = make_seq("a", range(12), 0.0, 1), make_seq("b", range(7), 1.0, 1)
+    sched.add_seq(a)
+    sched.add_seq(b)
+    out = engine_step(sched)
+    assert [(p.seq.seq_id, p.start, p.num_tokens) for p in out.portions] == [("a", 0, 5), ("b", 0, 5)]
+    out = engine_step(sched)
+    assert [(p.seq.seq_id, p.start, p.num_tokens, p.samples) for p in out.portions] == [("a", 5, 5, False), ("b", 5, 2, True)]
+
+
+def test_admission_sets_pages_aside_for_the_whole_request():
+    """A half-prefilled request never has to fight for pages to finish its prompt: the second
+    request waits although its first portion alone would fit."""
+    sched, manager, _ = make_env(num_blocks=8, budget=8, chunked=True)
+    a, b = make_seq("a", range(20), 0.0, 1), make_seq("b", range(16), 1.0, 1)
+    sched.add_seq(a)
+    sched.add_seq(b)
+    out = sched.schedule()
+    assert [(p.seq.seq_id, p.num_tokens) for p in out.portions] == [("a", 8)]
+    assert len(manager.block_table("a")) == 5 and b.status is SequenceStatus.WAITING
+
+
+def test_a_half_prefilled_request_can_be_the_victim_and_starts_over():
+    # a (8-token prompt) decodes and grows; b's 16-token prompt is set aside whole (4 pages) and
+    # runs in portions of 2; a's next page edge comes while b is still in its prompt
+    sched, manager, _ = make_env(num_blocks=7, budget=3, chunked=True)
+    a = make_seq("a", range(8), 0.0, 12)
+    sched.add_seq(a)
+    for _ in range(3):
+        engine_step(sched)  # 3 + 3 + 2 tokens of the prompt, first token sampled
+    assert len(a) == 9 and a.num_uncomputed_tokens() == 1
+    b = make_seq("b", range(100, 116), 1.0, 2)
+    sched.add_seq(b)
+    before = None
+    for _ in range(10):
+        before = b.num_computed_tokens
+        out = engine_step(sched)
+        if out.preempted:
+            break
+    assert ids(out.preempted) == ["b"] and 0 < before < 16, "b was meant to be caught in its prompt"
+    assert b.num_computed_tokens == 0 and b.status is SequenceStatus.PREEMPTED and not manager.has("b")
+    assert ids(out.decode_seqs) == ["a"]
+    for _ in range(40):
+        if not sched.has_unfinished():
+            break
+        engine_step(sched)
+    assert a.is_finished() and b.is_finished() and len(b.output_token_ids) == 2
+    assert manager.num_free_blocks() == 7
+
+
+def test_idle_prefix_blocks_are_evicted_before_a_request_is_refused_or_preempted():
+    sched, manager, cache = make_env(num_blocks=6, budget=64, prefix=True, chunked=True)
+    first = make_seq("first", range(16), 0.0, 1)
+    sched.add_seq(first)
+    engine_step(sched)
+    # the engine inserts finished prompts; stand in for it here
+    handles = [(p,) for p in manager.pools[0].take_many(4)]
+    cache.insert(list(range(500, 516)), handles)
+    for h in handles:
+        manager.drop_handle(h)
+    assert manager.num_free_blocks() == 2 and cache.evictable_blocks() == 4
+    big = make_seq("big", range(300, 320), 1.0, 3)  # 5 pages, then a sixth while decoding
+    sched.add_seq(big)
+    out = engine_step(sched)
+    assert ids(out.prefill_seqs) == ["big"] and cache.num_blocks() <= 1
+    for _ in range(4):
+        out = engine_step(sched)
+        assert not out.preempted
+    assert big.is_finished()
+    cache.reset()
+    assert manager.num_free_blocks() == 6
+
+
+def test_pages_run_out_for_the_only_request():
+    """Nothing else to preempt: the request itself is preempted and waits; with a pool that can
+    never hold it the scheduler keeps returning an empty schedule (the engine raises)."""
+    sched, manager, _ = make_env(num_blocks=2, budget=64, chunked=True)
+    a = make_seq("a", range(8), 0.0, 4)
+    sched.add_seq(a)
+    engine_step(sched)
+    out = engine_step(sched)  # position 8 needs a third page
+    assert ids(out.preempted) == ["a"] and not out.portions
+    out = sched.schedule()  # 9 tokens now need 3 pages: never admissible
+    assert out.is_empty() and a.status is SequenceStatus.PREEMPTED and manager.num_free_blocks() == 2
+
+
+def test_stats_count_admissions_and_batches():
+    sched, _, _ = make_env()
+    a = make_seq("a", range(5), 0.0, 2)
+    sched.add_seq(a)
+    assert (sched.stats.num_waiting, sched.stats.num_running) == (1, 0)
+    engine_step(sched)
+    assert (sched.stats.num_waiting, sched.stats.num_running, sched.stats.total_prompt_tokens) == (0, 1, 5)
+    engine_step(sched)
+    assert sched.stats.num_scheduled_batches == 2 and sched.stats.num_running == 0
