@@ -136,6 +136,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--only-prefill", action="store_true", help="run the 2048-token prefill alone (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
@@ -144,6 +145,10 @@ def main() -> int:
     import torch
 
     cfg, runner = build_runner(args)
+    if args.only_prefill:
+        t = time_prefill(cfg, runner)
+        print(json.dumps({"prefill_ms": round(1e3 * t, 3), "tokens_per_s": round(PROMPT_LEN / t, 1)}))
+        return 0
     elapsed, mean_ctx = time_decode(cfg, runner, args.batch, args.steps, args.warmup)
     value = args.batch * args.steps / elapsed
     ms = 1e3 * elapsed / args.steps

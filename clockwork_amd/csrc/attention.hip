@@ -390,3 +390,330 @@ CW_EXPORT int cw_attention(int rows, int dtype, const void* q, int64_t q_stride,
   }
   return CW_ERR_DTYPE;
 }
+
+// =====================================================================================
+// bfloat16 decode attention: one query token per work item, keys streamed at memory speed.
+//
+// A workgroup (4 waves) takes one (request, key/value head, split of the key range); each wave
+// walks tiles of 16 keys. Scores come from one MFMA chain per tile: S^T[16 keys, 16 heads] =
+// K[16 keys, HD] * Q^T[HD, 16 heads], with K fragments loaded straight from the pages into the
+// MFMA operand layout (lane = key l%16, 8 consecutive head elements at slot l/16) and the same
+// element order used for Q, so no LDS transpose is needed. Softmax statistics are float32,
+// per head, per wave. P*V runs on the vector ALUs: the wave's probabilities go through LDS
+// so that lane (l/16, l%16) can weight the 8 value elements it loaded (key 4j + l/16, elements
+// 8*(l%16)..) for every head of the group. Waves and lane groups are merged once at the end.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+#define DEC_WAVES 4
+
+template <int HD, int GH>
+__global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnParams p) {
+  constexpr int NF = HD / 32;   // MFMA k-steps over the head dimension
+  constexpr int NC = HD / 8;    // 16-byte chunks of a key/value row
+  constexpr int VPI = 64 / NC;  // value rows one load instruction of a wave covers (hd 128: 4)
+  constexpr int VJ = 16 / VPI;  // load instructions per 16-key tile
+  static_assert(HD % 32 == 0 && NC <= 64 && 64 % NC == 0 && VPI <= 16, "head size of the decode kernel");
+  __shared__ float P_s[DEC_WAVES][16][16];
+  __shared__ float A_s[DEC_WAVES][16];
+  __shared__ float M_s[DEC_WAVES][16];
+  __shared__ float L_s[DEC_WAVES][16];
+  extern __shared__ __align__(16) float acc_s[];  // [waves][VPI][GH][HD]
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, s = lane >> 4;
+  const int item = blockIdx.x;
+  const int kvh = blockIdx.y / p.n_chunks, chunk = blockIdx.y % p.n_chunks;
+  const int split = blockIdx.z;
+  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1];
+  const int ctx = p.ctx_lens[req];
+  const int q_begin = p.cu_q[req];
+  const int qlen = p.cu_q[req + 1] - q_begin;
+  const int group = p.nh / p.nkv;
+  const int pos = ctx - qlen + tok0;
+  const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int tile0 = lo / 16;
+  const int n_tiles = pos / 16 + 1 - tile0;
+  const int tps = (n_tiles + p.n_splits - 1) / p.n_splits;
+  const int t_begin = tile0 + split * tps;
+  const int t_end = min(tile0 + n_tiles, t_begin + tps);
+  const int* table = p.block_tables + (int64_t)req * p.table_stride;
+  const bf16_t* kc = (const bf16_t*)p.k_cache;
+  const bf16_t* vc = (const bf16_t*)p.v_cache;
+  const int bs = p.block_size;
+
+  // query fragments: lane (r, s) holds head r, elements (j * 4 + s) * 8 .. + 7
+  bf16x8_t qf[NF];
+  {
+    const int hig = chunk * GH + r;
+    const bool ok = r < GH && hig < group;
+    const bf16_t* qrow = (const bf16_t*)p.q + (int64_t)(q_begin + tok0) * p.q_stride + (kvh * group + (ok ? hig : 0)) * HD;
+#pragma unroll
+    for (int j = 0; j < NF; ++j) {
+      if (ok) qf[j] = *reinterpret_cast<const bf16x8_t*>(qrow + (j * 4 + s) * 8);
+      else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[j][e] = (__bf16)0.0f;
+      }
+    }
+  }
+
+  float m_run = -INFINITY, l_run = 0.0f;  // of head r, the same in all four lane groups
+  float acc[GH][8];
+#pragma unroll
+  for (int g = 0; g < GH; ++g)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
+  // value loads: lane covers row (lane / NC) of each group of VPI rows, chunk lane % NC
+  const int vrow = lane / NC, vchunk = lane % NC;
+
+  for (int t = t_begin + wave; t < t_end; t += DEC_WAVES) {
+    const int kv0 = t * 16;
+    // ---- keys: one row per lane r, NF fragments
+    bf16x8_t kf[NF];
+    {
+      const int kp = kv0 + r;
+      const bool ok = kp >= lo && kp <= pos;
+      int page = ok ? table[kp / bs] : -1;
+      const bool have = ok && page >= 0;
+      const bf16_t* krow = kc + (((int64_t)(have ? page : 0) * bs + kp % bs) * p.nkv + kvh) * HD;
+#pragma unroll
+      for (int j = 0; j < NF; ++j) {
+        if (have) kf[j] = *reinterpret_cast<const bf16x8_t*>(krow + (j * 4 + s) * 8);
+        else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) kf[j][e] = (__bf16)0.0f;
+        }
+      }
+    }
+    // ---- values: VJ loads, row 16-key-tile index vj * VPI + vrow
+    uint4 vf[VJ];
+#pragma unroll
+    for (int vj = 0; vj < VJ; ++vj) {
+      const int kp = kv0 + vj * VPI + vrow;
+      const bool ok = kp >= lo && kp <= pos;
+      int page = ok ? table[kp / bs] : -1;
+      if (ok && page >= 0)
+        vf[vj] = *reinterpret_cast<const uint4*>(vc + (((int64_t)page * bs + kp % bs) * p.nkv + kvh) * HD + vchunk * 8);
+      else
+        vf[vj] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    // ---- scores S^T: lane (r, s) gets keys 4s..4s+3 of head r
+    f32x4_t sc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < NF; ++j) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j], qf[j], sc, 0, 0, 0);
+    float sv[4];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int kp = kv0 + 4 * s + i;
+      sv[i] = (kp >= lo && kp <= pos) ? sc[i] * p.scale : -INFINITY;
+      tmax = fmaxf(tmax, sv[i]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);
+    float alpha = 1.0f, psum = 0.0f;
+    float pv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (m_new != -INFINITY) {
+      alpha = __expf(m_run - m_new);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pv[i] = __expf(sv[i] - m_new);
+        psum += pv[i];
+      }
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    // ---- probabilities and rescale factors of this wave -> LDS -> every lane
+#pragma unroll
+    for (int i = 0; i < 4; ++i) P_s[wave][4 * s + i][r] = pv[i];
+    if (s == 0) A_s[wave][r] = alpha;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int g = 0; g < GH; ++g) {
+        const float a = A_s[wave][g];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] *= a;
+      }
+    }
+#pragma unroll
+    for (int vj = 0; vj < VJ; ++vj) {
+      const uint32_t w[4] = {vf[vj].x, vf[vj].y, vf[vj].z, vf[vj].w};
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+      }
+      const float* prow = &P_s[wave][vj * VPI + vrow][0];
+#pragma unroll
+      for (int g = 0; g < GH; ++g) {
+        const float pw = prow[g];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pw, v[e], acc[g][e]);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+
+  // ---- merge the waves (and the lane groups of each wave)
+  if (s == 0) { M_s[wave][r] = m_run; L_s[wave][r] = l_run; }
+#pragma unroll
+  for (int g = 0; g < GH; ++g)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc_s[((wave * VPI + vrow) * GH + g) * HD + vchunk * 8 + e] = acc[g][e];
+  __syncthreads();
+  const int64_t base = ((int64_t)item * gridDim.y + blockIdx.y) * p.n_splits + split;
+  for (int idx = threadIdx.x; idx < GH * HD; idx += 256) {
+    const int g = idx / HD, d = idx - g * HD;
+    const int hig = chunk * GH + g;
+    if (hig >= group) continue;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, M_s[w][g]);
+    float L = 0.0f, O = 0.0f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) {
+      const float mw = M_s[w][g];
+      if (mw == -INFINITY) continue;
+      const float wgt = __expf(mw - M);
+      L = fmaf(L_s[w][g], wgt, L);
+      float o = 0.0f;
+#pragma unroll
+      for (int v = 0; v < VPI; ++v) o += acc_s[((w * VPI + v) * GH + g) * HD + d];
+      O = fmaf(o, wgt, O);
+    }
+    if (p.n_splits == 1) {
+      ((bf16_t*)p.out)[(int64_t)(q_begin + tok0) * p.out_stride + (kvh * group + hig) * HD + d] =
+          __float2bfloat16(O / L);
+    } else {
+      p.part_o[(base * GH + g) * HD + d] = O;
+      if (d == 0) {
+        p.part_ml[(base * GH + g) * 2] = M;
+        p.part_ml[(base * GH + g) * 2 + 1] = L;
+      }
+    }
+  }
+}
+
+// Merge of the decode kernel's splits: one workgroup per (item, head), one thread per element.
+template <int HD>
+__global__ void attn_decode_merge_kernel(AttnParams p, int gh) {
+  const int item = blockIdx.x;
+  const int y = blockIdx.y / gh, g = blockIdx.y % gh;
+  const int kvh = y / p.n_chunks, chunk = y % p.n_chunks;
+  const int group = p.nh / p.nkv;
+  const int hig = chunk * gh + g;
+  if (hig >= group) return;
+  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1];
+  const int q_begin = p.cu_q[req];
+  const int64_t base = ((int64_t)item * (p.nkv * p.n_chunks) + y) * p.n_splits;
+  float M = -INFINITY;
+  for (int sp = 0; sp < p.n_splits; ++sp) M = fmaxf(M, p.part_ml[((base + sp) * gh + g) * 2]);
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float L = 0.0f, O = 0.0f;
+    for (int sp = 0; sp < p.n_splits; ++sp) {
+      const float m = p.part_ml[((base + sp) * gh + g) * 2];
+      if (m == -INFINITY) continue;
+      const float w = __expf(m - M);
+      L = fmaf(p.part_ml[((base + sp) * gh + g) * 2 + 1], w, L);
+      O = fmaf(p.part_o[((base + sp) * gh + g) * HD + d], w, O);
+    }
+    ((bf16_t*)p.out)[(int64_t)(q_begin + tok0) * p.out_stride + (kvh * group + hig) * HD + d] =
+        __float2bfloat16(O / L);
+  }
+}
+
+#if CW_HD % 32 == 0 && (64 % (CW_HD / 8) == 0)
+#define CW_HAS_DECODE 1
+#else
+#define CW_HAS_DECODE 0
+#endif
+
+// 1 when this head size has the bfloat16 decode kernel (32, 64, 128, 256).
+CW_EXPORT int cw_attention_decode_supported() { return CW_HAS_DECODE; }
+
+// Heads of a group one workgroup of the decode kernel takes, for a group of this size.
+CW_EXPORT int cw_attention_decode_gh(int group) {
+  if (group <= 1) return 1;
+  if (group <= 2) return 2;
+  if (group <= 4) return 4;
+  if (group <= 6) return 6;
+  return 8;
+}
+
+CW_EXPORT int64_t cw_attention_decode_workspace_floats(int n_items, int nh, int nkv, int n_splits) {
+  if (n_splits <= 1) return 0;
+  const int group = nh / nkv;
+  const int gh = cw_attention_decode_gh(group);
+  const int n_chunks = (group + gh - 1) / gh;
+  return (int64_t)n_items * nkv * n_chunks * n_splits * gh * (CW_HD + 2);
+}
+
+#if CW_HAS_DECODE
+template <int GH>
+static int launch_decode(AttnParams& p, int n_items, hipStream_t stream) {
+  constexpr int HD = CW_HD;
+  constexpr int VPI = 64 / (HD / 8);
+  const size_t smem = sizeof(float) * DEC_WAVES * VPI * GH * HD;
+  static bool raised = false;
+  if (!raised) {
+    if (hipFuncSetAttribute((const void*)attn_decode_bf16_kernel<HD, GH>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return CW_ERR_LAUNCH;
+    raised = true;
+  }
+  dim3 grid(n_items, p.nkv * p.n_chunks, p.n_splits), block(256);
+  hipLaunchKernelGGL((attn_decode_bf16_kernel<HD, GH>), grid, block, smem, stream, p);
+  if (p.n_splits > 1) {
+    dim3 mgrid(n_items, p.nkv * p.n_chunks * GH);
+    hipLaunchKernelGGL((attn_decode_merge_kernel<HD>), mgrid, dim3(HD < 64 ? 64 : HD), 0, stream, p, GH);
+  }
+  return cw_launch_status();
+}
+#endif
+
+// Single-token items (every item: one token), bfloat16. Same arguments as cw_attention.
+CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride,
+                                       const void* k_cache, const void* v_cache, const int* block_tables,
+                                       int table_stride, const int* ctx_lens, const int* cu_q,
+                                       const int* items, int n_items, int nh, int nkv, int block_size,
+                                       int n_splits, int window, float scale, float* workspace,
+                                       int64_t workspace_floats, hipStream_t stream) {
+#if CW_HAS_DECODE
+  if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || block_size <= 0 || table_stride <= 0)
+    return CW_ERR_ARG;
+  if (n_splits < 1 || n_splits > 65535 || window < 0) return CW_ERR_ARG;
+  if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || (q_stride & 7))
+    return CW_ERR_ARG;
+  if (n_items == 0) return CW_OK;
+  const int group = nh / nkv;
+  AttnParams p;
+  p.q = q; p.q_stride = q_stride; p.out = out; p.out_stride = out_stride;
+  p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
+  p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
+  p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.gh = cw_attention_decode_gh(group);
+  p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = n_splits; p.window = window; p.scale = scale;
+  if ((int64_t)nkv * p.n_chunks * p.gh > 65535) return CW_ERR_SIZE;
+  const int64_t need = cw_attention_decode_workspace_floats(n_items, nh, nkv, n_splits);
+  if (need > 0 && (workspace == nullptr || workspace_floats < need)) return CW_ERR_ARG;
+  p.part_o = workspace;
+  p.part_ml = workspace ? workspace + need / (CW_HD + 2) * CW_HD : nullptr;
+  switch (p.gh) {
+    case 1: return launch_decode<1>(p, n_items, stream);
+    case 2: return launch_decode<2>(p, n_items, stream);
+    case 4: return launch_decode<4>(p, n_items, stream);
+    case 6: return launch_decode<6>(p, n_items, stream);
+    default: return launch_decode<8>(p, n_items, stream);
+  }
+#else
+  return CW_ERR_ARG;
+#endif
+}

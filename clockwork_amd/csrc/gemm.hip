@@ -98,3 +98,158 @@ CW_EXPORT int cw_gemm_f32(const float* A, int64_t lda, const float* W, const flo
   hipLaunchKernelGGL(gemm_f32_kernel, grid, block, 0, stream, A, lda, W, bias, C, ldc, M, N, K);
   return cw_launch_status();
 }
+
+// =====================================================================================
+// bfloat16 products with few rows of x (decode: 1 to 64 tokens): the weight matrix is streamed
+// once at memory speed. A workgroup of 4 waves owns RT * 16 weight rows; its waves split the K
+// loop and are summed through LDS at the end (no atomics: the result does not depend on timing).
+// Each wave feeds 16 weight rows x 32 k-values to one MFMA (v_mfma_f32_16x16x32_bf16) as the A
+// operand, loaded from global memory directly in operand layout (lane = row l%16, 8 consecutive
+// k at slot l/16), and 16 tokens x the same k-values as the B operand.
+//
+// MODE 0: y bfloat16 [M, N]; MODE 1: y float32 [M, N] (logits); MODE 2: W is [2I, K] with gate
+// rows first, y[m, i] = silu(gate_i) * up_i as bfloat16 [M, I]: a row tile holds 8 gate rows and
+// the 8 up rows that belong to them.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+template <int MT, int RT, int MODE>
+__global__ __launch_bounds__(256) void gemm_skinny_bf16_kernel(const bf16_t* __restrict__ X, int64_t ldx,
+                                                               const bf16_t* __restrict__ W,
+                                                               void* __restrict__ C, int64_t ldc,
+                                                               int M, int N, int K) {
+  __shared__ float red[4][RT * MT * 256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, s = lane >> 4;
+  const int I = N / 2;  // MODE 2 only
+
+  // weight rows of this lane, one per row tile
+  const bf16_t* wrow[RT];
+  bool wok[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    int64_t n;
+    if (MODE == 2) {
+      const int64_t i = ((int64_t)blockIdx.x * RT + rt) * 8 + (r & 7);
+      n = (r < 8) ? i : I + i;
+      wok[rt] = i < I;
+    } else {
+      n = ((int64_t)blockIdx.x * RT + rt) * 16 + r;
+      wok[rt] = n < N;
+    }
+    wrow[rt] = W + (wok[rt] ? n : 0) * K;
+  }
+  const bf16_t* xrow[MT];
+  bool xok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + r;
+    xok[mt] = m < M;
+    xrow[mt] = X + (int64_t)(xok[mt] ? m : 0) * ldx;
+  }
+
+  f32x4_t acc[RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+
+  bf16x8_t zero;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) zero[e] = (__bf16)0.0f;
+
+  const int k_steps = (K + 31) / 32;
+  constexpr int U = 4;  // k-steps in flight per wave
+  for (int ks0 = wave * U; ks0 < k_steps; ks0 += 4 * U) {
+    bf16x8_t wf[U][RT], xf[U][MT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = (ks0 + u) * 32 + s * 8;
+      const bool kok = (ks0 + u) < k_steps && k + 8 <= K;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+        wf[u][rt] = (kok && wok[rt]) ? *reinterpret_cast<const bf16x8_t*>(wrow[rt] + k) : zero;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        xf[u][mt] = (kok && xok[mt]) ? *reinterpret_cast<const bf16x8_t*>(xrow[mt] + k) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][rt], xf[u][mt], acc[rt][mt], 0, 0, 0);
+  }
+
+  // D tile of (rt, mt): lane (r, s) holds weight rows 4s..4s+3 of token r -> red[wave][tile][row][token]
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][(rt * MT + mt) * 256 + (4 * s + i) * 16 + r] = acc[rt][mt][i];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < RT * MT * 256; idx += 256)
+    red[0][idx] = (red[0][idx] + red[1][idx]) + (red[2][idx] + red[3][idx]);
+  __syncthreads();
+
+  if (MODE == 2) {
+    // outputs: 8 per row tile and token; idx -> (token, rt, j) with j fastest
+    for (int idx = threadIdx.x; idx < RT * MT * 128; idx += 256) {
+      const int j = idx & 7, rt = (idx >> 3) % RT, m = idx / (8 * RT);
+      const int mt = m >> 4, tok = m & 15;
+      const int64_t i = ((int64_t)blockIdx.x * RT + rt) * 8 + j;
+      if (m >= M || i >= I) continue;
+      const float g = red[0][(rt * MT + mt) * 256 + j * 16 + tok];
+      const float u = red[0][(rt * MT + mt) * 256 + (j + 8) * 16 + tok];
+      ((bf16_t*)C)[(int64_t)m * ldc + i] = __float2bfloat16(g / (1.0f + __expf(-g)) * u);
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < RT * MT * 256; idx += 256) {
+      const int j = idx & 15, rt = (idx >> 4) % RT, m = idx / (16 * RT);
+      const int mt = m >> 4, tok = m & 15;
+      const int64_t n = ((int64_t)blockIdx.x * RT + rt) * 16 + j;
+      if (m >= M || n >= N) continue;
+      const float v = red[0][(rt * MT + mt) * 256 + j * 16 + tok];
+      if (MODE == 1) ((float*)C)[(int64_t)m * ldc + n] = v;
+      else ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(v);
+    }
+  }
+}
+
+#define CW_SKINNY_MAX_M 64
+
+template <int MT, int RT>
+static int launch_skinny(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W, void* C, int64_t ldc,
+                         int M, int N, int K, hipStream_t stream) {
+  const int rows_per_group = (mode == 2 ? 8 : 16) * RT;
+  const int rows = mode == 2 ? N / 2 : N;
+  dim3 grid((rows + rows_per_group - 1) / rows_per_group), block(256);
+  if (mode == 0) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 0>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  else if (mode == 1) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 1>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  else hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 2>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  return cw_launch_status();
+}
+
+// y = x W^T for M <= 64 rows of bfloat16 x [M, K] (row stride ldx) and bfloat16 W [N, K].
+// mode 0: y bfloat16 [M, N]; 1: y float32 [M, N]; 2: y = silu(gate) * up, bfloat16 [M, N / 2].
+// K must be a multiple of 8 (16-byte rows).
+CW_EXPORT int cw_gemm_bf16_skinny(int mode, const void* X, int64_t ldx, const void* W, void* C,
+                                  int64_t ldc, int M, int N, int K, hipStream_t stream) {
+  if (M < 0 || N <= 0 || K <= 0 || mode < 0 || mode > 2) return CW_ERR_ARG;
+  if (M > CW_SKINNY_MAX_M) return CW_ERR_SIZE;
+  if ((K & 7) || (ldx & 7) || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return CW_ERR_ARG;
+  if (mode == 2 && (N & 1)) return CW_ERR_ARG;
+  if (ldx < K || ldc < (mode == 2 ? N / 2 : N)) return CW_ERR_ARG;
+  if (M == 0) return CW_OK;
+  const bf16_t* x = (const bf16_t*)X;
+  const bf16_t* w = (const bf16_t*)W;
+  const int rows = mode == 2 ? N / 2 : N;
+  // more weight rows per workgroup when there are many tokens: x is then re-read less often
+  if (M <= 16) return launch_skinny<1, 1>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+  if (M <= 32) return rows >= 4096 ? launch_skinny<2, 2>(mode, x, ldx, w, C, ldc, M, N, K, stream)
+                                   : launch_skinny<2, 1>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+  return rows >= 4096 ? launch_skinny<4, 2>(mode, x, ldx, w, C, ldc, M, N, K, stream)
+                      : launch_skinny<4, 1>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+}

@@ -40,6 +40,7 @@ class AttentionPlan:
     gh_single: int = 1
     chunks_single: int = 1
     single_splits: int = 1
+    decode_splits: int = 1   # splits of the bfloat16 decode kernel (finer: it walks 16-key tiles)
 
 
 class _Packer:
@@ -126,6 +127,9 @@ class StepContext:
             by_occupancy = -(-4 * self.num_compute_units // groups_running)
             by_length = max(1, longest_single // 256)
             plan.single_splits = max(1, min(by_occupancy, by_length, 64))
+            # decode kernel: a workgroup per (request, kv head, split); at least 128 keys a split
+            base = plan.n_single * nkv * -(-group // min(group, 8))
+            plan.decode_splits = max(1, min(-(-3 * self.num_compute_units // base), longest_single // 128, 64))
         packer = _Packer()
         packer.add(wide)
         packer.add(single)

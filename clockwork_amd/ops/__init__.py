@@ -85,6 +85,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
         },
         "gemm": {
             "cw_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
+            "cw_gemm_bf16_skinny": [I, P, L, P, P, L, I, I, I, P],
         },
         "sampling": {
             "cw_argmax_chunks": [I],
@@ -95,12 +96,16 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_attention_head_dim": [],
             "cw_attention_workspace_floats": [I, I, I, I, I],
             "cw_attention": [I, I, P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P, L, P],
+            "cw_attention_decode_supported": [],
+            "cw_attention_decode_gh": [I],
+            "cw_attention_decode_workspace_floats": [I, I, I, I],
+            "cw_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, P],
         },
     }[name]
     for fn, argtypes in sigs.items():
         f = getattr(lib, fn)
         f.argtypes = argtypes
-        f.restype = c_int64 if fn == "cw_attention_workspace_floats" else c_int
+        f.restype = c_int64 if fn.endswith("workspace_floats") else c_int
 
 
 def _stream() -> int:
@@ -235,12 +240,76 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None) -> 
         _check(_load("gemm").cw_gemm_f32(_ptr(x), K, _ptr(weight), _ptr(bias), _ptr(out), N, M, N, K, _stream()), "gemm_f32")
         return out
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "a bfloat16 product needs bfloat16 operands")
+    if M <= SKINNY_MAX_ROWS and K % 8 == 0 and bias is None:
+        want_f32 = out_dtype == torch.float32
+        out = torch.empty((M, N), dtype=torch.float32 if want_f32 else torch.bfloat16, device=x.device)
+        _check(_load("gemm").cw_gemm_bf16_skinny(1 if want_f32 else 0, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, _stream()),
+               "gemm_bf16_skinny")
+        return out
     y = torch.mm(x, weight.t()) if bias is None else torch.addmm(bias, x, weight.t())
     if out_dtype == torch.float32:
         out = torch.empty((M, N), dtype=torch.float32, device=x.device)
         _check(_load("core").cw_bf16_to_f32(_ptr(y), _ptr(out), M * N, _stream()), "bf16_to_f32")
         return out
     return y
+
+
+SKINNY_MAX_ROWS = 64
+
+
+def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+    """silu(x @ gate.T) * (x @ up.T) for gate_up_weight = [gate; up] stacked along dim 0.
+
+    Few bfloat16 rows: one kernel that streams the weights once and applies the gate in its
+    epilogue. Otherwise the product followed by the gate kernel."""
+    _gpu(x, gate_up_weight)
+    M, K = x.shape
+    two_i = gate_up_weight.shape[0]
+    _need(gate_up_weight.shape[1] == K and two_i % 2 == 0, "gate_up weight must be [2 I, K]")
+    out = torch.empty((M, two_i // 2), dtype=x.dtype, device=x.device)
+    if x.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and K % 8 == 0:
+        _need(gate_up_weight.dtype == torch.bfloat16, "a bfloat16 product needs bfloat16 operands")
+        _check(_load("gemm").cw_gemm_bf16_skinny(2, _ptr(x), K, _ptr(gate_up_weight), _ptr(out), two_i // 2, M, two_i, K, _stream()),
+               "gemm_bf16_skinny(swiglu)")
+        return out
+    return silu_mul(linear(x, gate_up_weight), out)
+
+
+def decode_attention_supported(hd: int, dtype: torch.dtype) -> bool:
+    return dtype == torch.bfloat16 and bool(_load("attention", hd).cw_attention_decode_supported())
+
+
+def decode_attention_workspace_floats(hd: int, n_items: int, nh: int, nkv: int, n_splits: int) -> int:
+    return int(_load("attention", hd).cw_attention_decode_workspace_floats(n_items, nh, nkv, n_splits))
+
+
+def attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
+                     nh: int, nkv: int, hd: int, block_size: int, n_splits: int, window: int, scale: float,
+                     n_tokens: int, n_requests: int, workspace=None) -> None:
+    """Single-token items through the bfloat16 decode kernel; arguments as for ``attention``."""
+    _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, workspace)
+    _need(q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16, "the decode kernel is bfloat16")
+    _need(out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd, "attention output must be [T, nh * hd]")
+    _need(q_stride >= nh * hd, "query rows overlap")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= n_requests, "block_tables must be int32 [R, max_blocks]")
+    _i32(ctx_lens, n_requests, "ctx_lens")
+    _i32(cu_q, n_requests + 1, "cu_q")
+    _need(items.dtype == torch.int32 and items.numel() >= 4 * n_items, "items must be int32 [n_items, 4]")
+    _need(tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape, "cache must be [..., nkv, hd]")
+    lib = _load("attention", hd)
+    need = lib.cw_attention_decode_workspace_floats(n_items, nh, nkv, n_splits)
+    ws_floats = 0
+    if need > 0:
+        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need,
+              f"decode attention needs a float32 workspace of {need} elements")
+        ws_floats = workspace.numel()
+    _check(
+        lib.cw_attention_decode_bf16(
+            q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+            block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, nh, nkv, block_size, n_splits,
+            window, float(scale), _ptr(workspace), ws_floats, _stream()),
+        "attention_decode_bf16",
+    )
 
 
 def attention(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,

@@ -73,7 +73,14 @@ class PagedAttention(Part):
         if plan.n_wide:
             ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide,
                           n_splits=1, **common)
-        if plan.n_single:
+        if plan.n_single and ops.decode_attention_supported(hd, x.dtype):
+            workspace = None
+            if plan.decode_splits > 1:
+                need = ops.decode_attention_workspace_floats(hd, plan.n_single, nh, nkv, plan.decode_splits)
+                workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+            ops.attention_decode(items=plan.single_items, n_items=plan.n_single, n_splits=plan.decode_splits,
+                                 workspace=workspace, **common)
+        elif plan.n_single:
             workspace = None
             if plan.single_splits > 1:
                 need = ops.attention_workspace_floats(hd, 16, plan.n_single, nkv, plan.chunks_single, plan.single_splits)

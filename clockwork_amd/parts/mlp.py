@@ -26,7 +26,4 @@ class SwiGLU(Part):
         self.down = params["down_weight"]
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        gu = ops.linear(x, self.gate_up)
-        act = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
-        ops.silu_mul(gu, act)
-        return ops.linear(act, self.down)
+        return ops.linear(ops.linear_swiglu(x, self.gate_up), self.down)

@@ -173,11 +173,43 @@ def test_gemm_f32_rows_do_not_depend_on_batch():
         assert torch.equal(ops.linear(x[i : i + 1].contiguous(), w)[0], whole[i])
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(100, 176), (2048, 1536), (48, 64), (5000, 200)])
+def test_skinny_bf16_product(M, N, K):
+    """Few rows of x against a streamed weight matrix: bfloat16 and float32 outputs."""
+    from clockwork_amd import ops
+
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV) / K ** 0.5).to(torch.bfloat16)
+    want = x.float() @ w.float().t()
+    got32 = ops.linear(x, w, out_dtype=torch.float32)
+    assert got32.dtype == torch.float32
+    torch.testing.assert_close(got32, want, rtol=1e-4, atol=1e-4)  # float32 accumulation of exact products
+    got = ops.linear(x, w)
+    assert got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float(), want, rtol=1e-2, atol=1e-2)
+    # a row's result does not depend on the other rows
+    assert torch.equal(ops.linear(x[M - 1 :].contiguous(), w, out_dtype=torch.float32)[0], got32[M - 1])
+
+
+@pytest.mark.parametrize("M", [1, 8, 20, 64, 100])
+@pytest.mark.parametrize("I,K", [(176, 64), (8960, 1536), (100, 80), (52, 200)])
+def test_fused_swiglu_product(M, I, K):
+    from clockwork_amd import ops
+
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(2 * I, K, device=DEV) / K ** 0.5).to(torch.bfloat16)
+    got = ops.linear_swiglu(x, w)
+    y = x.float() @ w.float().t()
+    want = torch.nn.functional.silu(y[:, :I]) * y[:, I:]
+    torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_linear_library_path_and_float32_logits(dtype):
     from clockwork_amd import ops
 
-    x = torch.randn(5, 96, device=DEV).to(dtype)
+    x = torch.randn(70, 96, device=DEV).to(dtype)
     w = torch.randn(50, 96, device=DEV).to(dtype)
     got = ops.linear(x, w, out_dtype=torch.float32)
     assert got.dtype == torch.float32
@@ -227,7 +259,8 @@ def _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens, poison=100.0)
     return kc, vc, ks, vs
 
 
-def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs, window=0, splits=None, scale=None):
+def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs, window=0, splits=None, scale=None,
+                   decode_kernel=False):
     from clockwork_amd import ops
     from clockwork_amd.engine.batch import StepContext
 
@@ -255,7 +288,15 @@ def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs,
                   cu_q=cu, nh=nh, nkv=nkv, hd=hd, block_size=bs, window=window, scale=scale, n_tokens=T, n_requests=R)
     if plan.n_wide:
         ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide, n_splits=1, **common)
-    if plan.n_single:
+    if plan.n_single and decode_kernel:
+        assert ops.decode_attention_supported(hd, dtype)
+        n_splits = splits if splits is not None else plan.decode_splits
+        ws = None
+        if n_splits > 1:
+            ws = torch.empty(ops.decode_attention_workspace_floats(hd, plan.n_single, nh, nkv, n_splits),
+                             dtype=torch.float32, device=DEV)
+        ops.attention_decode(items=plan.single_items, n_items=plan.n_single, n_splits=n_splits, workspace=ws, **common)
+    elif plan.n_single:
         ws = None
         if plan.single_splits > 1:
             ws = torch.empty(ops.attention_workspace_floats(hd, 16, plan.n_single, nkv, plan.chunks_single, plan.single_splits),
@@ -342,6 +383,74 @@ def test_attention_window(dtype, window):
         want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5, window=window)
         torch.testing.assert_close(out[at : at + q_len].float().cpu(), want, **tol(dtype))
         at += q_len
+
+
+# sizes of the bfloat16 decode kernel: head sizes 32..256, groups of 1 to 20 heads, pages of 4 to 32
+DECODE_KERNEL_CASES = [
+    (8, 2, 32, 4, [1, 7, 16, 3]),
+    (6, 3, 64, 8, [23, 8, 31, 200]),
+    (12, 2, 128, 16, [17, 64, 49, 2, 700]),
+    (6, 1, 32, 16, [300, 33]),
+    (40, 2, 64, 8, [70, 129]),
+    (3, 3, 128, 32, [5, 1000]),
+    (5, 1, 256, 16, [77, 300]),
+    (14, 2, 128, 16, [2304]),
+]
+
+
+@pytest.mark.parametrize("nh,nkv,hd,bs,ctx_lens", DECODE_KERNEL_CASES)
+@pytest.mark.parametrize("splits", [1, 2, 7])
+def test_decode_attention_kernel(nh, nkv, hd, bs, ctx_lens, splits):
+    dtype = torch.bfloat16
+    num_blocks = sum(-(-c // bs) for c in ctx_lens) + 5
+    perm = torch.randperm(num_blocks).tolist()
+    tables, at = [], 0
+    for c in ctx_lens:
+        n = -(-c // bs)
+        tables.append(perm[at : at + n])
+        at += n
+    kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens, poison=float("nan"))
+    qs = [torch.randn(1, nh, hd, device=DEV).to(dtype) for _ in ctx_lens]
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, [1] * len(ctx_lens), kc, vc, qs, splits=splits,
+                         decode_kernel=True)
+    assert not torch.isnan(out.float()).any()
+    for r in range(len(ctx_lens)):
+        want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5)
+        torch.testing.assert_close(out[r : r + 1].float().cpu(), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("window", [1, 5, 16, 40])
+def test_decode_attention_kernel_window_and_mixed_batch(window):
+    """Single tokens beside a portion in one batch; pages behind the window are gone (-1)."""
+    dtype = torch.bfloat16
+    nh, nkv, hd, bs = 4, 2, 32, 8
+    ctx_lens, q_lens = [90, 50, 70, 9], [1, 1, 30, 1]
+    tables = [list(range(0, 12)), list(range(12, 19)), list(range(19, 28)), [30, 31]]
+    kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, 40, tables, ctx_lens, poison=float("nan"))
+    tables_dev = [list(t) for t in tables]
+    for r, (c, q) in enumerate(zip(ctx_lens, q_lens)):
+        for b in range(max(0, (c - q) - window + 1) // bs):
+            tables_dev[r][b] = -1
+    qs = [torch.randn(q, nh, hd, device=DEV).to(dtype) for q in q_lens]
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables_dev, ctx_lens, q_lens, kc, vc, qs, window=window, decode_kernel=True)
+    at = 0
+    for r, q_len in enumerate(q_lens):
+        want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5, window=window)
+        torch.testing.assert_close(out[at : at + q_len].float().cpu(), want, **tol(dtype))
+        at += q_len
+
+
+def test_decode_attention_far_key_stands_out():
+    nh, nkv, hd, bs = 12, 2, 128, 16
+    ctx = 700
+    for where in (0, 15, 16, 511, 512, 698, 699):
+        tables = [list(range(44))]
+        kc, vc, ks, vs = _paged_setup(torch.bfloat16, nkv, hd, bs, 50, tables, [ctx])
+        q = torch.randn(1, nh, hd, device=DEV).to(torch.bfloat16)
+        slot = tables[0][where // bs] * bs + where % bs
+        kc[slot, 1] = (60.0 * q[0, 7].float() / q[0, 7].float().norm()).to(torch.bfloat16)
+        out = _run_attention(torch.bfloat16, nh, nkv, hd, bs, tables, [ctx], [1], kc, vc, [q], splits=3, decode_kernel=True)
+        torch.testing.assert_close(out[0, 7].float(), vc[slot, 1].float(), rtol=2e-2, atol=2e-2)
 
 
 def test_attention_far_key_stands_out():
