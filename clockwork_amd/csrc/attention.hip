@@ -717,3 +717,236 @@ CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* ou
   return CW_ERR_ARG;
 #endif
 }
+
+// =====================================================================================
+// bfloat16 attention for portions of prompts on the matrix cores, without LDS.
+//
+// A wave owns 32 query rows (row = token * gh + head of the group, so the group shares every key
+// and value it fetches) and walks tiles of 32 keys up to its last token's position.
+//   S^T[key, row] = K * Q^T     v_mfma_f32_16x16x32_bf16, K and Q fragments loaded from global
+//                               memory directly in operand layout (lane = key or row l%16, 8
+//                               consecutive head elements at slot l/16);
+//   softmax per row in float32: a lane holds 8 keys of one row, two shuffles finish a row;
+//   O^T[d, row] += V^T * P^T    P^T is already in operand layout (the lane's 8 keys of its row).
+//                               V^T is made from V with one small MFMA per 16x16 block: V times
+//                               the identity comes back with keys in the lane's registers, which
+//                               is the transposed layout the product needs.
+// The element order inside an MFMA's k dimension is free as long as both operands agree; that
+// is what lets every fragment be filled by plain 8- and 16-byte loads.
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+
+template <int HD>
+__global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnParams p) {
+  constexpr int NF = HD / 32;  // k-steps of the score product
+  constexpr int ND = HD / 16;  // 16-wide blocks of the head dimension
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, s = lane >> 4;
+  const int item = blockIdx.x;
+  const int kvh = blockIdx.y / p.n_chunks, chunk = blockIdx.y % p.n_chunks;
+  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1], ntok = p.items[4 * item + 2];
+  const int gh = p.gh;
+  const int tpw = 32 / gh;  // tokens of a wave
+  if (wave * tpw >= ntok) return;
+  const int ctx = p.ctx_lens[req];
+  const int q_begin = p.cu_q[req];
+  const int qlen = p.cu_q[req + 1] - q_begin;
+  const int group = p.nh / p.nkv;
+  const int pos0 = ctx - qlen + tok0;
+  const int p_first = pos0 + wave * tpw;
+  const int p_last = pos0 + min(ntok, (wave + 1) * tpw) - 1;
+  const int lo = p.window > 0 ? max(0, p_first - p.window + 1) : 0;
+  const int* table = p.block_tables + (int64_t)req * p.table_stride;
+  const bf16_t* kc = (const bf16_t*)p.k_cache;
+  const bf16_t* vc = (const bf16_t*)p.v_cache;
+  const int bs = p.block_size;
+
+  // ---- the wave's rows: block b, column c -> row b * 16 + c
+  int row_pos[2];      // position of the row's token, -1 for an unused row
+  int64_t row_off[2];  // offset of the row's head in q / out, in elements
+  bf16x8_t qf[2][NF];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const int row = b * 16 + c;
+    const int tl = row / gh, g = row - tl * gh;
+    const int tokw = wave * tpw + tl;
+    const int hig = chunk * gh + g;
+    const bool ok = tl < tpw && tokw < ntok && hig < group;
+    row_pos[b] = ok ? pos0 + tokw : -1;
+    row_off[b] = ok ? (int64_t)(kvh * group + hig) * HD : 0;
+    const bf16_t* qrow = (const bf16_t*)p.q + (int64_t)(q_begin + tok0 + (ok ? tokw : 0)) * p.q_stride + row_off[b];
+#pragma unroll
+    for (int j = 0; j < NF; ++j) {
+      if (ok) qf[b][j] = *reinterpret_cast<const bf16x8_t*>(qrow + (j * 4 + s) * 8);
+      else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[b][j][e] = (__bf16)0.0f;
+      }
+    }
+  }
+  // identity as the B operand of the 16x16x16 product: element (k = 4s + e, n = c)
+  s16x4_t ident;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) ident[e] = (4 * s + e == c) ? (short)0x3F80 : (short)0;
+
+  f32x4_t o[2][ND];
+#pragma unroll
+  for (int b = 0; b < 2; ++b)
+#pragma unroll
+    for (int db = 0; db < ND; ++db) o[b][db] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
+
+  for (int t = lo / 32; t <= p_last / 32; ++t) {
+    const int kv0 = t * 32;
+    // ---- this lane's two keys (one per 16-key block) and where they live
+    const bf16_t* krow[2];
+    const bf16_t* vrow[2];
+    bool have[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int kp = kv0 + kb * 16 + c;
+      const bool ok = kp >= lo && kp <= p_last;
+      const int page = ok ? table[kp / bs] : -1;
+      have[kb] = ok && page >= 0;
+      const int64_t off = (((int64_t)(have[kb] ? page : 0) * bs + kp % bs) * p.nkv + kvh) * HD;
+      krow[kb] = kc + off;
+      vrow[kb] = vc + off;
+    }
+    // ---- S^T = K Q^T
+    f32x4_t sc[2][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      bf16x8_t kf[NF];
+#pragma unroll
+      for (int j = 0; j < NF; ++j) {
+        if (have[kb]) kf[j] = *reinterpret_cast<const bf16x8_t*>(krow[kb] + (j * 4 + s) * 8);
+        else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) kf[j][e] = (__bf16)0.0f;
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        sc[kb][b] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < NF; ++j)
+          sc[kb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j], qf[b][j], sc[kb][b], 0, 0, 0);
+      }
+    }
+    // ---- softmax per row; P^T packed as the B operand of the output product
+    bf16x8_t pf[2];
+    float alpha[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int rp = row_pos[b];
+      const int rlo = p.window > 0 ? rp - p.window + 1 : 0;
+      float sv[8];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int kp = kv0 + kb * 16 + 4 * s + i;
+          const float v = (kp <= rp && kp >= rlo) ? sc[kb][b][i] * p.scale : -INFINITY;
+          sv[kb * 4 + i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m_run[b], tmax);
+      float a = 1.0f, psum = 0.0f;
+      if (m_new != -INFINITY) {
+        a = __expf(m_run[b] - m_new);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float pe = __expf(sv[e] - m_new);
+          psum += pe;
+          pf[b][e] = (__bf16)pe;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pf[b][e] = (__bf16)0.0f;
+      }
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+      l_run[b] = l_run[b] * a + psum;
+      m_run[b] = m_new;
+      alpha[b] = a;
+    }
+    if (__any(alpha[0] != 1.0f || alpha[1] != 1.0f)) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int db = 0; db < ND; ++db) o[b][db] *= alpha[b];
+    }
+    // ---- O^T += V^T P^T, one 16-wide block of the head dimension at a time
+#pragma unroll
+    for (int db = 0; db < ND; ++db) {
+      bf16x8_t vt;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        s16x4_t vf = {0, 0, 0, 0};
+        if (have[kb]) vf = *reinterpret_cast<const s16x4_t*>(vrow[kb] + db * 16 + 4 * s);
+        const f32x4_t tr = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, ident, (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vt[kb * 4 + i] = (__bf16)tr[i];
+      }
+#pragma unroll
+      for (int b = 0; b < 2; ++b) o[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pf[b], o[b][db], 0, 0, 0);
+    }
+  }
+
+  // ---- out[row][d]: lane (c, s) holds d = db * 16 + 4s .. + 3 of row (b, c)
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    if (row_pos[b] < 0) continue;
+    const float inv = 1.0f / l_run[b];
+    bf16_t* orow = (bf16_t*)p.out + (int64_t)(q_begin + (row_pos[b] - (ctx - qlen))) * p.out_stride + row_off[b];
+#pragma unroll
+    for (int db = 0; db < ND; ++db) {
+      uint2 packed;
+      packed.x = (uint32_t)cw_float_to_bf16_bits(o[b][db][0] * inv) | ((uint32_t)cw_float_to_bf16_bits(o[b][db][1] * inv) << 16);
+      packed.y = (uint32_t)cw_float_to_bf16_bits(o[b][db][2] * inv) | ((uint32_t)cw_float_to_bf16_bits(o[b][db][3] * inv) << 16);
+      *reinterpret_cast<uint2*>(orow + db * 16 + 4 * s) = packed;
+    }
+  }
+}
+
+#if CW_HD % 32 == 0
+#define CW_HAS_PREFILL 1
+#else
+#define CW_HAS_PREFILL 0
+#endif
+
+// 1 when this head size has the bfloat16 matrix-core kernel for portions (multiples of 32).
+CW_EXPORT int cw_attention_prefill_supported() { return CW_HAS_PREFILL; }
+
+// Portions of prompts, bfloat16. items: (request, first token, tokens, 0) with
+// tokens <= 4 * (32 / gh), gh = min(group, 32) heads of a group per workgroup.
+CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride,
+                                        const void* k_cache, const void* v_cache, const int* block_tables,
+                                        int table_stride, const int* ctx_lens, const int* cu_q,
+                                        const int* items, int n_items, int nh, int nkv, int block_size,
+                                        int window, float scale, hipStream_t stream) {
+#if CW_HAS_PREFILL
+  if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || block_size <= 0 || table_stride <= 0 || window < 0)
+    return CW_ERR_ARG;
+  if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || ((uintptr_t)out & 7) ||
+      (q_stride & 7) || (out_stride & 3))
+    return CW_ERR_ARG;
+  if (n_items == 0) return CW_OK;
+  const int group = nh / nkv;
+  AttnParams p;
+  p.q = q; p.q_stride = q_stride; p.out = out; p.out_stride = out_stride;
+  p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
+  p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
+  p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.gh = group < 32 ? group : 32;
+  p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = 1; p.window = window; p.scale = scale;
+  p.part_o = nullptr; p.part_ml = nullptr;
+  if ((int64_t)nkv * p.n_chunks > 65535) return CW_ERR_SIZE;
+  dim3 grid(n_items, nkv * p.n_chunks), block(256);
+  hipLaunchKernelGGL((attn_prefill_bf16_kernel<CW_HD>), grid, block, 0, stream, p);
+  return cw_launch_status();
+#else
+  return CW_ERR_ARG;
+#endif
+}

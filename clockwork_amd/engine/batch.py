@@ -35,6 +35,8 @@ class AttentionPlan:
     wide_items: Optional[torch.Tensor] = None
     n_wide: int = 0
     gh_wide: int = 1
+    mfma_items: Optional[torch.Tensor] = None   # the same portions cut for the bfloat16 matrix-core kernel
+    n_mfma: int = 0
     single_items: Optional[torch.Tensor] = None
     n_single: int = 0
     gh_single: int = 1
@@ -110,6 +112,8 @@ class StepContext:
         tokens_per_tile = 64 // gh_wide
         gh_single = min(group, 16)
         wide: list[int] = []
+        mfma: list[int] = []
+        tokens_per_mfma_item = 4 * (32 // min(group, 32))
         single: list[int] = []
         longest_single = 0
         for r, q_len in enumerate(self.h_q_lens):
@@ -119,8 +123,11 @@ class StepContext:
             else:
                 for tok0 in range(0, q_len, tokens_per_tile):
                     wide += [r, tok0, min(tokens_per_tile, q_len - tok0), 0]
+                # longest key ranges first: the last tokens of a portion have the most work
+                for tok0 in reversed(range(0, q_len, tokens_per_mfma_item)):
+                    mfma += [r, tok0, min(tokens_per_mfma_item, q_len - tok0), 0]
         plan = AttentionPlan(gh_wide=gh_wide, gh_single=gh_single)
-        plan.n_wide, plan.n_single = len(wide) // 4, len(single) // 4
+        plan.n_wide, plan.n_single, plan.n_mfma = len(wide) // 4, len(single) // 4, len(mfma) // 4
         plan.chunks_single = -(-group // gh_single)
         if plan.n_single:
             groups_running = plan.n_single * nkv * plan.chunks_single
@@ -133,7 +140,8 @@ class StepContext:
         packer = _Packer()
         packer.add(wide)
         packer.add(single)
-        plan.wide_items, plan.single_items = packer.upload(self.device)
+        packer.add(mfma)
+        plan.wide_items, plan.single_items, plan.mfma_items = packer.upload(self.device)
         self._keep = getattr(self, "_keep", []) + [packer]
         return plan
 

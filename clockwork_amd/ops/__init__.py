@@ -96,6 +96,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_attention_head_dim": [],
             "cw_attention_workspace_floats": [I, I, I, I, I],
             "cw_attention": [I, I, P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P, L, P],
+            "cw_attention_prefill_supported": [],
+            "cw_attention_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, P],
             "cw_attention_decode_supported": [],
             "cw_attention_decode_gh": [I],
             "cw_attention_decode_workspace_floats": [I, I, I, I],
@@ -273,6 +275,33 @@ def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor
                "gemm_bf16_skinny(swiglu)")
         return out
     return silu_mul(linear(x, gate_up_weight), out)
+
+
+def prefill_attention_supported(hd: int, dtype: torch.dtype) -> bool:
+    return dtype == torch.bfloat16 and bool(_load("attention", hd).cw_attention_prefill_supported())
+
+
+def attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
+                      nh: int, nkv: int, hd: int, block_size: int, window: int, scale: float,
+                      n_tokens: int, n_requests: int) -> None:
+    """Portions of prompts through the bfloat16 matrix-core kernel; an item holds at most
+    4 * (32 // min(group, 32)) tokens. Other arguments as for ``attention``."""
+    _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items)
+    _need(q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16, "the kernel is bfloat16")
+    _need(out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd, "attention output must be [T, nh * hd]")
+    _need(q_stride >= nh * hd, "query rows overlap")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= n_requests, "block_tables must be int32 [R, max_blocks]")
+    _i32(ctx_lens, n_requests, "ctx_lens")
+    _i32(cu_q, n_requests + 1, "cu_q")
+    _need(items.dtype == torch.int32 and items.numel() >= 4 * n_items, "items must be int32 [n_items, 4]")
+    _need(tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape, "cache must be [..., nkv, hd]")
+    _check(
+        _load("attention", hd).cw_attention_prefill_bf16(
+            q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+            block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, nh, nkv, block_size,
+            window, float(scale), _stream()),
+        "attention_prefill_bf16",
+    )
 
 
 def decode_attention_supported(hd: int, dtype: torch.dtype) -> bool:

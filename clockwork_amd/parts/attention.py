@@ -70,7 +70,9 @@ class PagedAttention(Part):
             nh=nh, nkv=nkv, hd=hd, block_size=cache.block_size, window=s.window or 0,
             scale=s.scale, n_tokens=T, n_requests=ctx.num_requests,
         )
-        if plan.n_wide:
+        if plan.n_wide and ops.prefill_attention_supported(hd, x.dtype):
+            ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, **common)
+        elif plan.n_wide:
             ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide,
                           n_splits=1, **common)
         if plan.n_single and ops.decode_attention_supported(hd, x.dtype):

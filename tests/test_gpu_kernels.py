@@ -260,7 +260,7 @@ def _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens, poison=100.0)
 
 
 def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs, window=0, splits=None, scale=None,
-                   decode_kernel=False):
+                   decode_kernel=False, prefill_kernel=False):
     from clockwork_amd import ops
     from clockwork_amd.engine.batch import StepContext
 
@@ -286,7 +286,10 @@ def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs,
     scale = scale if scale is not None else hd ** -0.5
     common = dict(q=qbuf, q_stride=qbuf.shape[1], out=out, k_cache=kc, v_cache=vc, block_tables=bt, ctx_lens=cl,
                   cu_q=cu, nh=nh, nkv=nkv, hd=hd, block_size=bs, window=window, scale=scale, n_tokens=T, n_requests=R)
-    if plan.n_wide:
+    if plan.n_wide and prefill_kernel:
+        assert ops.prefill_attention_supported(hd, dtype)
+        ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, **common)
+    elif plan.n_wide:
         ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide, n_splits=1, **common)
     if plan.n_single and decode_kernel:
         assert ops.decode_attention_supported(hd, dtype)
@@ -417,6 +420,59 @@ def test_decode_attention_kernel(nh, nkv, hd, bs, ctx_lens, splits):
     for r in range(len(ctx_lens)):
         want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5)
         torch.testing.assert_close(out[r : r + 1].float().cpu(), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("nh,nkv,hd,bs", [(4, 2, 32, 4), (6, 1, 32, 8), (3, 3, 64, 16), (12, 2, 128, 16), (2, 1, 256, 16),
+                                          (40, 1, 64, 8), (7, 7, 96, 16)])
+@pytest.mark.parametrize("window", [0, 9, 40])
+def test_prefill_attention_kernel(nh, nkv, hd, bs, window):
+    """The matrix-core kernel for portions: cached prefix + new tokens, ragged sizes, groups that
+    do not divide 32, a group larger than 32, single tokens in the same batch, poisoned pages."""
+    dtype = torch.bfloat16
+    ctx_lens = [21, 150, 2, 77, 1, 64, 333]
+    q_lens = [6, 150, 2, 1, 1, 33, 40]
+    num_blocks = sum(-(-c // bs) for c in ctx_lens) + 3
+    perm = torch.randperm(num_blocks).tolist()
+    tables, at = [], 0
+    for c in ctx_lens:
+        n = -(-c // bs)
+        tables.append(perm[at : at + n])
+        at += n
+    kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens, poison=float("nan"))
+    tables_dev = [list(t) for t in tables]
+    if window:
+        for r, (c, q) in enumerate(zip(ctx_lens, q_lens)):
+            for b in range(max(0, (c - q) - window + 1) // bs):
+                tables_dev[r][b] = -1
+    qs = [torch.randn(q, nh, hd, device=DEV).to(dtype) for q in q_lens]
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables_dev, ctx_lens, q_lens, kc, vc, qs, window=window,
+                         prefill_kernel=True, decode_kernel=ops_decode_ok(hd))
+    assert not torch.isnan(out.float()).any()
+    at = 0
+    for r, q_len in enumerate(q_lens):
+        want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5,
+                                     window=window or None)
+        torch.testing.assert_close(out[at : at + q_len].float().cpu(), want, **tol(dtype))
+        at += q_len
+
+
+def ops_decode_ok(hd):
+    from clockwork_amd import ops
+
+    return ops.decode_attention_supported(hd, torch.bfloat16)
+
+
+def test_prefill_attention_kernel_sharp_scores():
+    """Scores of very different size, so that the running maximum moves from tile to tile and one
+    far key dominates a row: rescaling and masking errors cannot hide behind near-uniform weights."""
+    dtype = torch.bfloat16
+    nh, nkv, hd, bs, T = 12, 2, 128, 16, 300
+    tables = [torch.randperm(20).tolist()[:19]]
+    kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, 20, tables, [T])
+    q = (3.0 * torch.randn(T, nh, hd, device=DEV)).to(dtype)
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables, [T], [T], kc, vc, [q], prefill_kernel=True, scale=0.5)
+    want = plain.attention_dense(q.float().cpu(), ks[0].float().cpu(), vs[0].float().cpu(), 0.5)
+    torch.testing.assert_close(out.float().cpu(), want, rtol=3e-2, atol=3e-2)
 
 
 @pytest.mark.parametrize("window", [1, 5, 16, 40])
