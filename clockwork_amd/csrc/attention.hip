@@ -31,6 +31,7 @@ struct AttnParams {
   const int* cu_q;        // [requests + 1] offsets of each request's tokens in the batch
   const int* items;       // [n_items, 4]: request, first token (relative), tokens, unused
   int nh, nkv, block_size;
+  int bs_shift;           // log2(block_size) when it is a power of two, else -1
   int gh;                 // query heads of a group handled by one workgroup
   int n_chunks;           // ceil(group / gh)
   int n_splits;
@@ -38,7 +39,21 @@ struct AttnParams {
   float scale;
   float* part_o;          // [n_items, nkv * n_chunks, n_splits, ROWS, HD] unnormalised outputs
   float* part_ml;         // [n_items, nkv * n_chunks, n_splits, ROWS, 2] running max, sum
+  int* counters;          // decode kernel: one arrival counter per (item, head chunk), zero between launches
+  const void* zeros;      // at least HD zero elements: what a masked key or value row is loaded from
 };
+
+// page of a position and the offset inside it; POW2: the page size is a power of two (shift given)
+template <bool POW2> __device__ __forceinline__ int cw_page_index(int pos, int bs, int shift) {
+  return POW2 ? pos >> shift : pos / bs;
+}
+template <bool POW2> __device__ __forceinline__ int cw_page_offset(int pos, int bs, int shift) {
+  return POW2 ? pos & (bs - 1) : pos % bs;
+}
+static inline int cw_log2_or_minus1(int v) {
+  for (int s = 0; s < 31; ++s) if ((1 << s) == v) return s;
+  return -1;
+}
 
 template <typename T> struct Vec16;
 template <> struct Vec16<float> {
@@ -372,7 +387,7 @@ CW_EXPORT int cw_attention(int rows, int dtype, const void* q, int64_t q_stride,
   p.q = q; p.q_stride = q_stride; p.out = out; p.out_stride = out_stride;
   p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
   p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
-  p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.gh = gh;
+  p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.bs_shift = cw_log2_or_minus1(block_size); p.gh = gh;
   p.n_chunks = (group + gh - 1) / gh; p.n_splits = n_splits; p.window = window; p.scale = scale;
   if ((int64_t)nkv * p.n_chunks > 65535) return CW_ERR_SIZE;
   const int64_t need = cw_attention_workspace_floats(rows, n_items, nkv, p.n_chunks, n_splits);
@@ -380,6 +395,8 @@ CW_EXPORT int cw_attention(int rows, int dtype, const void* q, int64_t q_stride,
   const int64_t n_o = need / (CW_HD + 2) * CW_HD;
   p.part_o = workspace;
   p.part_ml = workspace ? workspace + n_o : nullptr;
+  p.counters = nullptr;
+  p.zeros = nullptr;
   constexpr int BN = CW_HD <= 128 ? 64 : 32;
   if (dtype == CW_F32) {
     return rows == 64 ? launch_attention<float, 64, BN>(p, n_items, stream)
@@ -392,36 +409,37 @@ CW_EXPORT int cw_attention(int rows, int dtype, const void* q, int64_t q_stride,
 }
 
 // =====================================================================================
-// bfloat16 decode attention: one query token per work item, keys streamed at memory speed.
+// bfloat16 decode attention: one query token per work item, keys and values streamed at memory
+// speed, all products on the matrix cores.
 //
-// A workgroup (4 waves) takes one (request, key/value head, split of the key range); each wave
-// walks tiles of 16 keys. Scores come from one MFMA chain per tile: S^T[16 keys, 16 heads] =
-// K[16 keys, HD] * Q^T[HD, 16 heads], with K fragments loaded straight from the pages into the
-// MFMA operand layout (lane = key l%16, 8 consecutive head elements at slot l/16) and the same
-// element order used for Q, so no LDS transpose is needed. Softmax statistics are float32,
-// per head, per wave. P*V runs on the vector ALUs: the wave's probabilities go through LDS
-// so that lane (l/16, l%16) can weight the 8 value elements it loaded (key 4j + l/16, elements
-// 8*(l%16)..) for every head of the group. Waves and lane groups are merged once at the end.
+// A workgroup (4 waves) takes one (request, key/value head, split of the key range); its waves
+// take turns on tiles of 32 keys. Per tile:
+//   S^T[key, head] = K * Q^T        v_mfma_f32_16x16x32_bf16; the up to 16 heads of the group are
+//                                   the columns, so every key is fetched once for the whole group;
+//   softmax per head in float32: a lane holds 8 keys of one head, two shuffles finish a head;
+//   V^T from V: V times a 0/1 selector matrix comes back with keys in the lane's registers
+//                                   (the layout the next product needs), values bit-exact;
+//   O^T[d, head] += V^T * P^T       P^T is the softmax output as it lies in the registers.
+// K and V fragments are loaded from the pages straight into operand layout with 16-byte loads;
+// the next tile's loads are issued before the current tile is computed. Waves are merged through
+// LDS at the end; splits are merged by a second, small kernel.
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 #define DEC_WAVES 4
 
-template <int HD, int GH>
+template <int HD, bool POW2>
 __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnParams p) {
-  constexpr int NF = HD / 32;   // MFMA k-steps over the head dimension
-  constexpr int NC = HD / 8;    // 16-byte chunks of a key/value row
-  constexpr int VPI = 64 / NC;  // value rows one load instruction of a wave covers (hd 128: 4)
-  constexpr int VJ = 16 / VPI;  // load instructions per 16-key tile
-  static_assert(HD % 32 == 0 && NC <= 64 && 64 % NC == 0 && VPI <= 16, "head size of the decode kernel");
-  __shared__ float P_s[DEC_WAVES][16][16];
-  __shared__ float A_s[DEC_WAVES][16];
+  constexpr int NF = HD / 32;  // 32-element steps over the head dimension
+  constexpr int ND = HD / 16;  // 16-wide blocks of the head dimension
+  extern __shared__ __align__(16) float dyn_s[];  // [waves][16 heads][HD] outputs, then this split's pages
+  float* o_s = dyn_s;
+  int* tbl = reinterpret_cast<int*>(dyn_s + DEC_WAVES * 16 * HD);
   __shared__ float M_s[DEC_WAVES][16];
   __shared__ float L_s[DEC_WAVES][16];
-  extern __shared__ __align__(16) float acc_s[];  // [waves][VPI][GH][HD]
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r = lane & 15, s = lane >> 4;
+  const int c = lane & 15, s = lane >> 4;
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / p.n_chunks, chunk = blockIdx.y % p.n_chunks;
   const int split = blockIdx.z;
@@ -430,151 +448,147 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnParams p) {
   const int q_begin = p.cu_q[req];
   const int qlen = p.cu_q[req + 1] - q_begin;
   const int group = p.nh / p.nkv;
+  const int gh = p.gh;
   const int pos = ctx - qlen + tok0;
   const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
-  const int tile0 = lo / 16;
-  const int n_tiles = pos / 16 + 1 - tile0;
+  const int tile0 = lo / 32;
+  const int n_tiles = pos / 32 + 1 - tile0;
   const int tps = (n_tiles + p.n_splits - 1) / p.n_splits;
   const int t_begin = tile0 + split * tps;
   const int t_end = min(tile0 + n_tiles, t_begin + tps);
-  const int* table = p.block_tables + (int64_t)req * p.table_stride;
   const bf16_t* kc = (const bf16_t*)p.k_cache;
   const bf16_t* vc = (const bf16_t*)p.v_cache;
-  const int bs = p.block_size;
-
-  // query fragments: lane (r, s) holds head r, elements (j * 4 + s) * 8 .. + 7
-  bf16x8_t qf[NF];
+  const bf16_t* zrow = (const bf16_t*)p.zeros;
+  const int bs = p.block_size, sh = p.bs_shift;
+  // the pages of this split's keys -> LDS, so that no tile waits for a table entry from memory
+  const int page0 = cw_page_index<POW2>(t_begin * 32, bs, sh);
   {
-    const int hig = chunk * GH + r;
-    const bool ok = r < GH && hig < group;
-    const bf16_t* qrow = (const bf16_t*)p.q + (int64_t)(q_begin + tok0) * p.q_stride + (kvh * group + (ok ? hig : 0)) * HD;
+    const int* table = p.block_tables + (int64_t)req * p.table_stride;
+    const int last_key = min(pos, t_end * 32 - 1);
+    const int n_pages = t_end > t_begin ? cw_page_index<POW2>(last_key, bs, sh) - page0 + 1 : 0;
+    for (int i = threadIdx.x; i < n_pages; i += 256) tbl[i] = table[page0 + i];
+  }
+  __syncthreads();
+
+  // query fragments (B operand): lane (c, s) holds head c, elements (j * 4 + s) * 8 .. + 7
+  bf16x8_t qf[NF];
+  const int hig = chunk * gh + c;
+  const bool head_ok = c < gh && hig < group;
+  {
+    const bf16_t* qrow = head_ok ? (const bf16_t*)p.q + (int64_t)(q_begin + tok0) * p.q_stride + (kvh * group + hig) * HD : zrow;
 #pragma unroll
-    for (int j = 0; j < NF; ++j) {
-      if (ok) qf[j] = *reinterpret_cast<const bf16x8_t*>(qrow + (j * 4 + s) * 8);
-      else {
+    for (int j = 0; j < NF; ++j) qf[j] = *reinterpret_cast<const bf16x8_t*>(qrow + (j * 4 + s) * 8);
+  }
+  // selectors (B operand) that pick elements 0..15 / 16..31 of a 32-element step: (k = 8s + e, n = c)
+  bf16x8_t sel_lo, sel_hi;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qf[j][e] = (__bf16)0.0f;
-      }
-    }
+  for (int e = 0; e < 8; ++e) {
+    sel_lo[e] = (8 * s + e == c) ? (__bf16)1.0f : (__bf16)0.0f;
+    sel_hi[e] = (8 * s + e == 16 + c) ? (__bf16)1.0f : (__bf16)0.0f;
   }
 
-  float m_run = -INFINITY, l_run = 0.0f;  // of head r, the same in all four lane groups
-  float acc[GH][8];
+  // loads of one 32-key tile, always issued: a masked key is read from a row of zeros
+  auto load_tile = [&](int t, bf16x8_t (*kf)[NF], bf16x8_t (*vf)[NF]) {
 #pragma unroll
-  for (int g = 0; g < GH; ++g)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
-  // value loads: lane covers row (lane / NC) of each group of VPI rows, chunk lane % NC
-  const int vrow = lane / NC, vchunk = lane % NC;
-
-  for (int t = t_begin + wave; t < t_end; t += DEC_WAVES) {
-    const int kv0 = t * 16;
-    // ---- keys: one row per lane r, NF fragments
-    bf16x8_t kf[NF];
-    {
-      const int kp = kv0 + r;
-      const bool ok = kp >= lo && kp <= pos;
-      int page = ok ? table[kp / bs] : -1;
+    for (int kb = 0; kb < 2; ++kb) {
+      const int kp = t * 32 + kb * 16 + c;
+      const bool ok = t < t_end && kp >= lo && kp <= pos;
+      const int page = tbl[ok ? cw_page_index<POW2>(kp, bs, sh) - page0 : 0];
       const bool have = ok && page >= 0;
-      const bf16_t* krow = kc + (((int64_t)(have ? page : 0) * bs + kp % bs) * p.nkv + kvh) * HD;
+      const int64_t off = (((int64_t)page * bs + cw_page_offset<POW2>(kp, bs, sh)) * p.nkv + kvh) * HD;
+      const bf16_t* kr = have ? kc + off : zrow;
+      const bf16_t* vr = have ? vc + off : zrow;
 #pragma unroll
-      for (int j = 0; j < NF; ++j) {
-        if (have) kf[j] = *reinterpret_cast<const bf16x8_t*>(krow + (j * 4 + s) * 8);
-        else {
+      for (int j = 0; j < NF; ++j) kf[kb][j] = *reinterpret_cast<const bf16x8_t*>(kr + (j * 4 + s) * 8);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) kf[j][e] = (__bf16)0.0f;
-        }
-      }
+      for (int j = 0; j < NF; ++j) vf[kb][j] = *reinterpret_cast<const bf16x8_t*>(vr + j * 32 + s * 8);
     }
-    // ---- values: VJ loads, row 16-key-tile index vj * VPI + vrow
-    uint4 vf[VJ];
+  };
+
+  f32x4_t o[ND];
 #pragma unroll
-    for (int vj = 0; vj < VJ; ++vj) {
-      const int kp = kv0 + vj * VPI + vrow;
-      const bool ok = kp >= lo && kp <= pos;
-      int page = ok ? table[kp / bs] : -1;
-      if (ok && page >= 0)
-        vf[vj] = *reinterpret_cast<const uint4*>(vc + (((int64_t)page * bs + kp % bs) * p.nkv + kvh) * HD + vchunk * 8);
-      else
-        vf[vj] = make_uint4(0u, 0u, 0u, 0u);
-    }
-    // ---- scores S^T: lane (r, s) gets keys 4s..4s+3 of head r
-    f32x4_t sc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int j = 0; j < NF; ++j) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j], qf[j], sc, 0, 0, 0);
-    float sv[4];
+  for (int db = 0; db < ND; ++db) o[db] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+  float m_run = -INFINITY, l_run = 0.0f;  // of head c, the same in all four lane groups
+  bf16x8_t kf[2][NF], vf[2][NF], kf_n[2][NF], vf_n[2][NF];
+  load_tile(t_begin + wave, kf, vf);
+  for (int t = t_begin + wave; t < t_end; t += DEC_WAVES) {
+    const int kv0 = t * 32;
+    load_tile(t + DEC_WAVES, kf_n, vf_n);  // the wave's next tile is on its way meanwhile
+    // ---- S^T = K Q^T, keys 4s..4s+3 of each 16-key block for head c
+    float sv[8];
     float tmax = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int kp = kv0 + 4 * s + i;
-      sv[i] = (kp >= lo && kp <= pos) ? sc[i] * p.scale : -INFINITY;
-      tmax = fmaxf(tmax, sv[i]);
+    for (int kb = 0; kb < 2; ++kb) {
+      f32x4_t sc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int j = 0; j < NF; ++j) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kb][j], qf[j], sc, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int kp = kv0 + kb * 16 + 4 * s + i;
+        const float v = (kp >= lo && kp <= pos) ? sc[i] * p.scale : -INFINITY;
+        sv[kb * 4 + i] = v;
+        tmax = fmaxf(tmax, v);
+      }
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float m_new = fmaxf(m_run, tmax);
     float alpha = 1.0f, psum = 0.0f;
-    float pv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    bf16x8_t pf;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) pf[e] = (__bf16)0.0f;
     if (m_new != -INFINITY) {
       alpha = __expf(m_run - m_new);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        pv[i] = __expf(sv[i] - m_new);
-        psum += pv[i];
+      for (int e = 0; e < 8; ++e) {
+        const float pe = __expf(sv[e] - m_new);
+        psum += pe;
+        pf[e] = (__bf16)pe;
       }
     }
     psum += __shfl_xor(psum, 16, 64);
     psum += __shfl_xor(psum, 32, 64);
     l_run = l_run * alpha + psum;
     m_run = m_new;
-    // ---- probabilities and rescale factors of this wave -> LDS -> every lane
-#pragma unroll
-    for (int i = 0; i < 4; ++i) P_s[wave][4 * s + i][r] = pv[i];
-    if (s == 0) A_s[wave][r] = alpha;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (__any(alpha != 1.0f)) {
 #pragma unroll
-      for (int g = 0; g < GH; ++g) {
-        const float a = A_s[wave][g];
+      for (int db = 0; db < ND; ++db) o[db] *= alpha;
+    }
+    // ---- O^T += V^T P^T
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] *= a;
+    for (int j = 0; j < NF; ++j) {
+      bf16x8_t vt_lo, vt_hi;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const f32x4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        const f32x4_t tl = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[kb][j], sel_lo, zero, 0, 0, 0);
+        const f32x4_t th = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[kb][j], sel_hi, zero, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          vt_lo[kb * 4 + i] = (__bf16)tl[i];
+          vt_hi[kb * 4 + i] = (__bf16)th[i];
+        }
       }
+      o[2 * j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt_lo, pf, o[2 * j], 0, 0, 0);
+      o[2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt_hi, pf, o[2 * j + 1], 0, 0, 0);
     }
 #pragma unroll
-    for (int vj = 0; vj < VJ; ++vj) {
-      const uint32_t w[4] = {vf[vj].x, vf[vj].y, vf[vj].z, vf[vj].w};
-      float v[8];
+    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        v[2 * i] = __uint_as_float(w[i] << 16);
-        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-      }
-      const float* prow = &P_s[wave][vj * VPI + vrow][0];
-#pragma unroll
-      for (int g = 0; g < GH; ++g) {
-        const float pw = prow[g];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pw, v[e], acc[g][e]);
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+      for (int j = 0; j < NF; ++j) { kf[kb][j] = kf_n[kb][j]; vf[kb][j] = vf_n[kb][j]; }
   }
 
-  // ---- merge the waves (and the lane groups of each wave)
-  if (s == 0) { M_s[wave][r] = m_run; L_s[wave][r] = l_run; }
+  // ---- merge the waves: o_s[wave][head c][d], lane (c, s) holds d = db * 16 + 4s .. + 3
+  if (s == 0) { M_s[wave][c] = m_run; L_s[wave][c] = l_run; }
 #pragma unroll
-  for (int g = 0; g < GH; ++g)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc_s[((wave * VPI + vrow) * GH + g) * HD + vchunk * 8 + e] = acc[g][e];
+  for (int db = 0; db < ND; ++db)
+    *reinterpret_cast<f32x4_t*>(&o_s[(wave * 16 + c) * HD + db * 16 + 4 * s]) = o[db];
   __syncthreads();
   const int64_t base = ((int64_t)item * gridDim.y + blockIdx.y) * p.n_splits + split;
-  for (int idx = threadIdx.x; idx < GH * HD; idx += 256) {
+  for (int idx = threadIdx.x; idx < gh * HD; idx += 256) {
     const int g = idx / HD, d = idx - g * HD;
-    const int hig = chunk * GH + g;
-    if (hig >= group) continue;
+    const int hg = chunk * gh + g;
+    if (hg >= group) continue;
     float M = -INFINITY;
 #pragma unroll
     for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, M_s[w][g]);
@@ -582,72 +596,79 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnParams p) {
 #pragma unroll
     for (int w = 0; w < DEC_WAVES; ++w) {
       const float mw = M_s[w][g];
-      if (mw == -INFINITY) continue;
-      const float wgt = __expf(mw - M);
+      const float wgt = mw == -INFINITY ? 0.0f : __expf(mw - M);
       L = fmaf(L_s[w][g], wgt, L);
-      float o = 0.0f;
-#pragma unroll
-      for (int v = 0; v < VPI; ++v) o += acc_s[((w * VPI + v) * GH + g) * HD + d];
-      O = fmaf(o, wgt, O);
+      O = fmaf(o_s[(w * 16 + g) * HD + d], wgt, O);
     }
     if (p.n_splits == 1) {
-      ((bf16_t*)p.out)[(int64_t)(q_begin + tok0) * p.out_stride + (kvh * group + hig) * HD + d] =
+      ((bf16_t*)p.out)[(int64_t)(q_begin + tok0) * p.out_stride + (kvh * group + hg) * HD + d] =
           __float2bfloat16(O / L);
     } else {
-      p.part_o[(base * GH + g) * HD + d] = O;
+      p.part_o[(base * gh + g) * HD + d] = O;
       if (d == 0) {
-        p.part_ml[(base * GH + g) * 2] = M;
-        p.part_ml[(base * GH + g) * 2 + 1] = L;
+        p.part_ml[(base * gh + g) * 2] = M;
+        p.part_ml[(base * gh + g) * 2 + 1] = L;
       }
     }
   }
 }
 
 // Merge of the decode kernel's splits: one workgroup per (item, head), one thread per element.
+// The statistics of all splits go through LDS first, and partial outputs are fetched four at
+// a time, so the kernel is a few memory round trips long whatever the number of splits.
 template <int HD>
-__global__ void attn_decode_merge_kernel(AttnParams p, int gh) {
+__global__ void attn_decode_merge_kernel(AttnParams p) {
+  __shared__ float ms[64], ls[64];
+  const int gh = p.gh;
   const int item = blockIdx.x;
   const int y = blockIdx.y / gh, g = blockIdx.y % gh;
   const int kvh = y / p.n_chunks, chunk = y % p.n_chunks;
   const int group = p.nh / p.nkv;
-  const int hig = chunk * gh + g;
-  if (hig >= group) return;
+  const int hg = chunk * gh + g;
+  if (hg >= group) return;
   const int req = p.items[4 * item], tok0 = p.items[4 * item + 1];
   const int q_begin = p.cu_q[req];
   const int64_t base = ((int64_t)item * (p.nkv * p.n_chunks) + y) * p.n_splits;
+  for (int sp = threadIdx.x; sp < p.n_splits; sp += blockDim.x) {
+    const float2 ml = *reinterpret_cast<const float2*>(&p.part_ml[((base + sp) * gh + g) * 2]);
+    ms[sp] = ml.x;
+    ls[sp] = ml.y;
+  }
+  __syncthreads();
   float M = -INFINITY;
-  for (int sp = 0; sp < p.n_splits; ++sp) M = fmaxf(M, p.part_ml[((base + sp) * gh + g) * 2]);
+  for (int sp = 0; sp < p.n_splits; ++sp) M = fmaxf(M, ms[sp]);
   for (int d = threadIdx.x; d < HD; d += blockDim.x) {
     float L = 0.0f, O = 0.0f;
-    for (int sp = 0; sp < p.n_splits; ++sp) {
-      const float m = p.part_ml[((base + sp) * gh + g) * 2];
-      if (m == -INFINITY) continue;
-      const float w = __expf(m - M);
-      L = fmaf(p.part_ml[((base + sp) * gh + g) * 2 + 1], w, L);
-      O = fmaf(p.part_o[((base + sp) * gh + g) * HD + d], w, O);
+    for (int sp0 = 0; sp0 < p.n_splits; sp0 += 4) {
+      float ov[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        ov[u] = sp0 + u < p.n_splits ? p.part_o[((base + sp0 + u) * gh + g) * HD + d] : 0.0f;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (sp0 + u >= p.n_splits) continue;
+        const float mv = ms[sp0 + u];
+        const float wgt = mv == -INFINITY ? 0.0f : __expf(mv - M);
+        L = fmaf(ls[sp0 + u], wgt, L);
+        O = fmaf(ov[u], wgt, O);
+      }
     }
-    ((bf16_t*)p.out)[(int64_t)(q_begin + tok0) * p.out_stride + (kvh * group + hig) * HD + d] =
+    ((bf16_t*)p.out)[(int64_t)(q_begin + tok0) * p.out_stride + (kvh * group + hg) * HD + d] =
         __float2bfloat16(O / L);
   }
 }
 
-#if CW_HD % 32 == 0 && (64 % (CW_HD / 8) == 0)
+#if CW_HD % 32 == 0
 #define CW_HAS_DECODE 1
 #else
 #define CW_HAS_DECODE 0
 #endif
 
-// 1 when this head size has the bfloat16 decode kernel (32, 64, 128, 256).
+// 1 when this head size has the bfloat16 decode kernel (multiples of 32).
 CW_EXPORT int cw_attention_decode_supported() { return CW_HAS_DECODE; }
 
 // Heads of a group one workgroup of the decode kernel takes, for a group of this size.
-CW_EXPORT int cw_attention_decode_gh(int group) {
-  if (group <= 1) return 1;
-  if (group <= 2) return 2;
-  if (group <= 4) return 4;
-  if (group <= 6) return 6;
-  return 8;
-}
+CW_EXPORT int cw_attention_decode_gh(int group) { return group < 16 ? group : 16; }
 
 CW_EXPORT int64_t cw_attention_decode_workspace_floats(int n_items, int nh, int nkv, int n_splits) {
   if (n_splits <= 1) return 0;
@@ -658,61 +679,65 @@ CW_EXPORT int64_t cw_attention_decode_workspace_floats(int n_items, int nh, int 
 }
 
 #if CW_HAS_DECODE
-template <int GH>
+template <bool POW2>
 static int launch_decode(AttnParams& p, int n_items, hipStream_t stream) {
   constexpr int HD = CW_HD;
-  constexpr int VPI = 64 / (HD / 8);
-  const size_t smem = sizeof(float) * DEC_WAVES * VPI * GH * HD;
-  static bool raised = false;
-  if (!raised) {
-    if (hipFuncSetAttribute((const void*)attn_decode_bf16_kernel<HD, GH>,
+  // keys of a split: at most ceil(tiles / splits) tiles of 32; their pages go to LDS
+  const int64_t max_tiles = ((int64_t)p.table_stride * p.block_size + 31) / 32;
+  const int64_t tiles_per_split = (max_tiles + p.n_splits - 1) / p.n_splits;
+  const int64_t pages = (tiles_per_split * 32 + p.block_size - 1) / p.block_size + 2;
+  const size_t smem = sizeof(float) * DEC_WAVES * 16 * HD + sizeof(int) * (size_t)pages;
+  if (smem > 160 * 1024) return CW_ERR_SIZE;
+  static size_t raised = 0;
+  if (smem > raised) {
+    if (hipFuncSetAttribute((const void*)attn_decode_bf16_kernel<HD, POW2>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
       return CW_ERR_LAUNCH;
-    raised = true;
+    raised = smem;
   }
   dim3 grid(n_items, p.nkv * p.n_chunks, p.n_splits), block(256);
-  hipLaunchKernelGGL((attn_decode_bf16_kernel<HD, GH>), grid, block, smem, stream, p);
+  hipLaunchKernelGGL((attn_decode_bf16_kernel<HD, POW2>), grid, block, smem, stream, p);
   if (p.n_splits > 1) {
-    dim3 mgrid(n_items, p.nkv * p.n_chunks * GH);
-    hipLaunchKernelGGL((attn_decode_merge_kernel<HD>), mgrid, dim3(HD < 64 ? 64 : HD), 0, stream, p, GH);
+    dim3 mgrid(n_items, p.nkv * p.n_chunks * p.gh);
+    hipLaunchKernelGGL((attn_decode_merge_kernel<HD>), mgrid, dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0, stream, p);
   }
   return cw_launch_status();
 }
 #endif
 
-// Single-token items (every item: one token), bfloat16. Same arguments as cw_attention.
+// Single-token items (every item: one token), bfloat16. Same arguments as cw_attention;
+// ``zeros``: at least CW_HD zero elements (16-byte aligned) that masked rows are read from.
 CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride,
                                        const void* k_cache, const void* v_cache, const int* block_tables,
                                        int table_stride, const int* ctx_lens, const int* cu_q,
                                        const int* items, int n_items, int nh, int nkv, int block_size,
                                        int n_splits, int window, float scale, float* workspace,
-                                       int64_t workspace_floats, hipStream_t stream) {
+                                       int64_t workspace_floats, const void* zeros, hipStream_t stream) {
 #if CW_HAS_DECODE
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || block_size <= 0 || table_stride <= 0)
     return CW_ERR_ARG;
-  if (n_splits < 1 || n_splits > 65535 || window < 0) return CW_ERR_ARG;
+  if (n_splits < 1 || n_splits > 64 || window < 0) return CW_ERR_ARG;
   if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || (q_stride & 7))
     return CW_ERR_ARG;
+  if (zeros == nullptr || ((uintptr_t)zeros & 15)) return CW_ERR_ARG;
   if (n_items == 0) return CW_OK;
   const int group = nh / nkv;
   AttnParams p;
   p.q = q; p.q_stride = q_stride; p.out = out; p.out_stride = out_stride;
   p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
   p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
-  p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.gh = cw_attention_decode_gh(group);
+  p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.bs_shift = cw_log2_or_minus1(block_size);
+  p.gh = cw_attention_decode_gh(group);
   p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = n_splits; p.window = window; p.scale = scale;
   if ((int64_t)nkv * p.n_chunks * p.gh > 65535) return CW_ERR_SIZE;
   const int64_t need = cw_attention_decode_workspace_floats(n_items, nh, nkv, n_splits);
   if (need > 0 && (workspace == nullptr || workspace_floats < need)) return CW_ERR_ARG;
+  if ((uintptr_t)workspace & 7) return CW_ERR_ARG;
   p.part_o = workspace;
   p.part_ml = workspace ? workspace + need / (CW_HD + 2) * CW_HD : nullptr;
-  switch (p.gh) {
-    case 1: return launch_decode<1>(p, n_items, stream);
-    case 2: return launch_decode<2>(p, n_items, stream);
-    case 4: return launch_decode<4>(p, n_items, stream);
-    case 6: return launch_decode<6>(p, n_items, stream);
-    default: return launch_decode<8>(p, n_items, stream);
-  }
+  p.counters = nullptr;
+  p.zeros = zeros;
+  return p.bs_shift >= 0 ? launch_decode<true>(p, n_items, stream) : launch_decode<false>(p, n_items, stream);
 #else
   return CW_ERR_ARG;
 #endif
@@ -735,10 +760,11 @@ CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* ou
 // is what lets every fragment be filled by plain 8- and 16-byte loads.
 typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 
-template <int HD>
+template <int HD, bool POW2>
 __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnParams p) {
   constexpr int NF = HD / 32;  // k-steps of the score product
   constexpr int ND = HD / 16;  // 16-wide blocks of the head dimension
+  constexpr bool PIPE = HD <= 128;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, s = lane >> 4;
   const int item = blockIdx.x;
@@ -746,19 +772,28 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnParams p) {
   const int req = p.items[4 * item], tok0 = p.items[4 * item + 1], ntok = p.items[4 * item + 2];
   const int gh = p.gh;
   const int tpw = 32 / gh;  // tokens of a wave
-  if (wave * tpw >= ntok) return;
   const int ctx = p.ctx_lens[req];
   const int q_begin = p.cu_q[req];
   const int qlen = p.cu_q[req + 1] - q_begin;
   const int group = p.nh / p.nkv;
   const int pos0 = ctx - qlen + tok0;
+  // the pages of every key this workgroup may read -> LDS: no tile waits for a table entry
+  extern __shared__ int tbl[];
+  const int wg_lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
+  const int page0 = cw_page_index<POW2>(wg_lo, p.block_size, p.bs_shift);
+  {
+    const int* table = p.block_tables + (int64_t)req * p.table_stride;
+    const int n_pages = cw_page_index<POW2>(pos0 + ntok - 1, p.block_size, p.bs_shift) - page0 + 1;
+    for (int i = threadIdx.x; i < n_pages; i += 256) tbl[i] = table[page0 + i];
+  }
+  __syncthreads();
+  if (wave * tpw >= ntok) return;
   const int p_first = pos0 + wave * tpw;
   const int p_last = pos0 + min(ntok, (wave + 1) * tpw) - 1;
   const int lo = p.window > 0 ? max(0, p_first - p.window + 1) : 0;
-  const int* table = p.block_tables + (int64_t)req * p.table_stride;
   const bf16_t* kc = (const bf16_t*)p.k_cache;
   const bf16_t* vc = (const bf16_t*)p.v_cache;
-  const int bs = p.block_size;
+  const int bs = p.block_size, sh = p.bs_shift;
 
   // ---- the wave's rows: block b, column c -> row b * 16 + c
   int row_pos[2];      // position of the row's token, -1 for an unused row
@@ -795,43 +830,60 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnParams p) {
     for (int db = 0; db < ND; ++db) o[b][db] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
   float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
 
-  for (int t = lo / 32; t <= p_last / 32; ++t) {
-    const int kv0 = t * 32;
-    // ---- this lane's two keys (one per 16-key block) and where they live
-    const bf16_t* krow[2];
-    const bf16_t* vrow[2];
-    bool have[2];
+  // Software pipeline over the key tiles: while tile t is being computed, the key and value
+  // fragments of tile t + 1 are already on their way, and the pages of tile t + 2 are looked up.
+  const int t_first = lo / 32, t_last = p_last / 32;
+  const bf16_t* zrow = (const bf16_t*)p.zeros;
+  // offset of the lane's key of tile t, block kb, in the caches; -1 when it is masked or its page is
+  // gone. A masked key is loaded from a row of zeros, so every load is issued unconditionally and
+  // the number of loads in flight is known at compile time.
+  auto lookup = [&](int t, int kb) -> int64_t {
+    const int kp = t * 32 + kb * 16 + c;
+    bool ok = t <= t_last && kp >= lo && kp <= p_last;
+    const int page = tbl[ok ? cw_page_index<POW2>(kp, bs, sh) - page0 : 0];
+    ok = ok && page >= 0;
+    return ok ? (((int64_t)page * bs + cw_page_offset<POW2>(kp, bs, sh)) * p.nkv + kvh) * HD : -1;
+  };
+  bf16x8_t kf[2][NF], kf_n[2][NF];
+  s16x4_t vf[2][ND], vf_n[2][ND];
+  int64_t off_nn[2];
+  bf16x8_t zero8;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      const int kp = kv0 + kb * 16 + c;
-      const bool ok = kp >= lo && kp <= p_last;
-      const int page = ok ? table[kp / bs] : -1;
-      have[kb] = ok && page >= 0;
-      const int64_t off = (((int64_t)(have[kb] ? page : 0) * bs + kp % bs) * p.nkv + kvh) * HD;
-      krow[kb] = kc + off;
-      vrow[kb] = vc + off;
+  for (int e = 0; e < 8; ++e) zero8[e] = (__bf16)0.0f;
+  auto load_frags = [&](int64_t off, bf16x8_t* kf_, s16x4_t* vf_) {
+    const bf16_t* kr = off >= 0 ? kc + off : zrow;
+    const bf16_t* vr = off >= 0 ? vc + off : zrow;
+#pragma unroll
+    for (int j = 0; j < NF; ++j) kf_[j] = *reinterpret_cast<const bf16x8_t*>(kr + (j * 4 + s) * 8);
+#pragma unroll
+    for (int db = 0; db < ND; ++db) vf_[db] = *reinterpret_cast<const s16x4_t*>(vr + db * 16 + 4 * s);
+  };
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+    load_frags(lookup(t_first, kb), kf[kb], vf[kb]);
+    off_nn[kb] = lookup(t_first + 1, kb);
+  }
+
+  for (int t = t_first; t <= t_last; ++t) {
+    const int kv0 = t * 32;
+    // ---- issue the loads of tile t + 1 and the page lookups of tile t + 2
+    // (head sizes above 128 have no registers to spare for this: they load tile t + 1 late)
+#pragma unroll
+    for (int kb = 0; kb < 2 && PIPE; ++kb) {
+      load_frags(off_nn[kb], kf_n[kb], vf_n[kb]);
+      off_nn[kb] = lookup(t + 2, kb);
     }
     // ---- S^T = K Q^T
     f32x4_t sc[2][2];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      bf16x8_t kf[NF];
-#pragma unroll
-      for (int j = 0; j < NF; ++j) {
-        if (have[kb]) kf[j] = *reinterpret_cast<const bf16x8_t*>(krow[kb] + (j * 4 + s) * 8);
-        else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) kf[j][e] = (__bf16)0.0f;
-        }
-      }
+    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
         sc[kb][b] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int j = 0; j < NF; ++j)
-          sc[kb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j], qf[b][j], sc[kb][b], 0, 0, 0);
+          sc[kb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kb][j], qf[b][j], sc[kb][b], 0, 0, 0);
       }
-    }
     // ---- softmax per row; P^T packed as the B operand of the output product
     bf16x8_t pf[2];
     float alpha[2];
@@ -863,8 +915,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnParams p) {
           pf[b][e] = (__bf16)pe;
         }
       } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) pf[b][e] = (__bf16)0.0f;
+        pf[b] = zero8;
       }
       psum += __shfl_xor(psum, 16, 64);
       psum += __shfl_xor(psum, 32, 64);
@@ -884,14 +935,25 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnParams p) {
       bf16x8_t vt;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
-        s16x4_t vf = {0, 0, 0, 0};
-        if (have[kb]) vf = *reinterpret_cast<const s16x4_t*>(vrow[kb] + db * 16 + 4 * s);
-        const f32x4_t tr = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, ident, (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        const f32x4_t tr = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[kb][db], ident, (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) vt[kb * 4 + i] = (__bf16)tr[i];
       }
 #pragma unroll
       for (int b = 0; b < 2; ++b) o[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pf[b], o[b][db], 0, 0, 0);
+    }
+    // ---- tile t + 1 becomes the current tile
+#pragma unroll
+    for (int kb = 0; kb < 2 && !PIPE; ++kb) {
+      load_frags(off_nn[kb], kf[kb], vf[kb]);
+      off_nn[kb] = lookup(t + 2, kb);
+    }
+#pragma unroll
+    for (int kb = 0; kb < 2 && PIPE; ++kb) {
+#pragma unroll
+      for (int j = 0; j < NF; ++j) kf[kb][j] = kf_n[kb][j];
+#pragma unroll
+      for (int db = 0; db < ND; ++db) vf[kb][db] = vf_n[kb][db];
     }
   }
 
@@ -926,8 +988,9 @@ CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* o
                                         const void* k_cache, const void* v_cache, const int* block_tables,
                                         int table_stride, const int* ctx_lens, const int* cu_q,
                                         const int* items, int n_items, int nh, int nkv, int block_size,
-                                        int window, float scale, hipStream_t stream) {
+                                        int window, float scale, const void* zeros, hipStream_t stream) {
 #if CW_HAS_PREFILL
+  if (zeros == nullptr || ((uintptr_t)zeros & 15)) return CW_ERR_ARG;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || block_size <= 0 || table_stride <= 0 || window < 0)
     return CW_ERR_ARG;
   if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || ((uintptr_t)out & 7) ||
@@ -939,12 +1002,32 @@ CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* o
   p.q = q; p.q_stride = q_stride; p.out = out; p.out_stride = out_stride;
   p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
   p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
-  p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.gh = group < 32 ? group : 32;
+  p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.bs_shift = cw_log2_or_minus1(block_size); p.gh = group < 32 ? group : 32;
   p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = 1; p.window = window; p.scale = scale;
-  p.part_o = nullptr; p.part_ml = nullptr;
+  p.part_o = nullptr; p.part_ml = nullptr; p.counters = nullptr; p.zeros = zeros;
   if ((int64_t)nkv * p.n_chunks > 65535) return CW_ERR_SIZE;
   dim3 grid(n_items, nkv * p.n_chunks), block(256);
-  hipLaunchKernelGGL((attn_prefill_bf16_kernel<CW_HD>), grid, block, 0, stream, p);
+  const size_t smem = sizeof(int) * ((size_t)table_stride + 2);  // a request's whole table fits
+  if (smem > 160 * 1024) return CW_ERR_SIZE;
+  if (p.bs_shift >= 0) {
+    static size_t raised = 0;
+    if (smem > raised && smem > 48 * 1024) {
+      if (hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<CW_HD, true>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return CW_ERR_LAUNCH;
+      raised = smem;
+    }
+    hipLaunchKernelGGL((attn_prefill_bf16_kernel<CW_HD, true>), grid, block, smem, stream, p);
+  } else {
+    static size_t raised = 0;
+    if (smem > raised && smem > 48 * 1024) {
+      if (hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<CW_HD, false>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return CW_ERR_LAUNCH;
+      raised = smem;
+    }
+    hipLaunchKernelGGL((attn_prefill_bf16_kernel<CW_HD, false>), grid, block, smem, stream, p);
+  }
   return cw_launch_status();
 #else
   return CW_ERR_ARG;

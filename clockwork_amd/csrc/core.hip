@@ -70,15 +70,113 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
   }
 }
 
+// The same for rows of up to 4096 elements with H % 4 == 0: every thread keeps its (at most four)
+// 4-element chunks of the row in registers, so the row is read once, and all loads are in flight
+// together. The order of the sum of squares depends on H alone here too.
+template <typename T> struct Chunk4;
+template <> struct Chunk4<float> {
+  __device__ static void load(const float* p, float* o) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+  }
+  __device__ static void store(float* p, const float* v) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <> struct Chunk4<bf16_t> {
+  __device__ static void load(const bf16_t* p, float* o) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+    o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+  }
+  __device__ static void store(bf16_t* p, const float* v) {
+    uint2 u;
+    u.x = (uint32_t)cw_float_to_bf16_bits(v[0]) | ((uint32_t)cw_float_to_bf16_bits(v[1]) << 16);
+    u.y = (uint32_t)cw_float_to_bf16_bits(v[2]) | ((uint32_t)cw_float_to_bf16_bits(v[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+  }
+};
+
+template <typename T, typename WT>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+                                                              const WT* __restrict__ weight, float eps,
+                                                              T* __restrict__ out, const int* __restrict__ rows, int H) {
+  __shared__ float partial[4];
+  const int i = blockIdx.x;
+  const int t = rows ? rows[i] : i;
+  float* x = resid + (int64_t)t * H;
+  const T* dl = delta ? delta + (int64_t)t * H : nullptr;
+  T* o = out + (int64_t)i * H;
+  const bool write_back = rows == nullptr && dl != nullptr;
+  const int n_chunks = H / 4;
+  float v[4][4], w[4][4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int ch = threadIdx.x + k * 256;
+    if (ch < n_chunks) {
+      Chunk4<float>::load(x + ch * 4, v[k]);
+      Chunk4<WT>::load(weight + ch * 4, w[k]);
+    } else {
+      v[k][0] = v[k][1] = v[k][2] = v[k][3] = 0.0f;
+    }
+  }
+  if (dl) {
+    float d[4][4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int ch = threadIdx.x + k * 256;
+      if (ch < n_chunks) Chunk4<T>::load(dl + ch * 4, d[k]);
+      else d[k][0] = d[k][1] = d[k][2] = d[k][3] = 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[k][e] += d[k][e];
+  }
+  float ss = 0.0f;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int ch = threadIdx.x + k * 256;
+    if (ch < n_chunks) {
+      if (write_back) Chunk4<float>::store(x + ch * 4, v[k]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += v[k][e] * v[k][e];
+    }
+  }
+  ss = cw_wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float total = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+  const float inv = 1.0f / sqrtf(total / (float)H + eps);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int ch = threadIdx.x + k * 256;
+    if (ch < n_chunks) {
+      float r[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = w[k][e] * cw_to_float(cw_from_float<T>(v[k][e] * inv));
+      Chunk4<T>::store(o + ch * 4, r);
+    }
+  }
+}
+
 CW_EXPORT int cw_add_rmsnorm(float* resid, const void* delta, const void* weight, int w_dtype,
                              float eps, void* out, int dtype, const int* rows, int n, int H,
                              hipStream_t stream) {
   if (n < 0 || H <= 0) return CW_ERR_ARG;
   if (n == 0) return CW_OK;
   dim3 grid(n), block(256);
-#define CW_LAUNCH(T, WT)                                                                         \
-  hipLaunchKernelGGL((add_rmsnorm_kernel<T, WT>), grid, block, 0, stream, resid, (const T*)delta, \
-                     (const WT*)weight, eps, (T*)out, rows, H)
+  const bool vec = (H % 4 == 0) && H <= 4096 && !((uintptr_t)resid & 15) && !((uintptr_t)out & 15) &&
+                   !((uintptr_t)weight & 15) && !((uintptr_t)delta & 15);
+#define CW_LAUNCH(T, WT)                                                                              \
+  do {                                                                                                \
+    if (vec)                                                                                          \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, WT>), grid, block, 0, stream, resid,              \
+                         (const T*)delta, (const WT*)weight, eps, (T*)out, rows, H);                  \
+    else                                                                                              \
+      hipLaunchKernelGGL((add_rmsnorm_kernel<T, WT>), grid, block, 0, stream, resid, (const T*)delta, \
+                         (const WT*)weight, eps, (T*)out, rows, H);                                   \
+  } while (0)
   if (dtype == CW_F32 && w_dtype == CW_F32) CW_LAUNCH(float, float);
   else if (dtype == CW_BF16 && w_dtype == CW_BF16) CW_LAUNCH(bf16_t, bf16_t);
   else if (dtype == CW_BF16 && w_dtype == CW_F32) CW_LAUNCH(bf16_t, float);
@@ -107,38 +205,37 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const BT* __restrict__
   if (slot >= cache_rows) slot = -1;
   const int half = rotary_dim / 2;
   const int rest = hd - rotary_dim;
-  const int per_head = half + rest;  // work items of a q or k head: pairs, then pass-through
-  const int n_qk = (nh + nkv) * per_head;
-  for (int w = threadIdx.x; w < n_qk; w += blockDim.x) {
-    const int head = w / per_head;
-    const int i = w % per_head;
-    T* h = row + head * hd;
-    const BT* hb = bias ? bias + head * hd : nullptr;
-    T* kdst = (head >= nh && slot >= 0)
-                  ? k_cache + (slot * nkv + (head - nh)) * (int64_t)hd
-                  : nullptr;
-    if (i < half) {
-      float a = cw_to_float(h[i]);
-      float b = cw_to_float(h[i + half]);
-      if (hb) { a += cw_to_float(hb[i]); b += cw_to_float(hb[i + half]); }
-      float ra = a, rb = b;
-      if (inv_freq) {
-        float s, c;
-        sincosf(pos * inv_freq[i], &s, &c);
-        ra = a * c - b * s;
-        rb = b * c + a * s;
+  // rotated pairs: thread = (pair i, head stripe); the angle of pair i is computed once per thread
+  if (half > 0) {
+    const int i = threadIdx.x % half;
+    const int stripe = threadIdx.x / half;
+    const int n_stripes = blockDim.x / half;
+    if (stripe < n_stripes) {
+      float sn = 0.0f, cs = 1.0f;
+      if (inv_freq) sincosf(pos * inv_freq[i], &sn, &cs);
+      for (int head = stripe; head < nh + nkv; head += n_stripes) {
+        T* h = row + head * hd;
+        float a = cw_to_float(h[i]);
+        float b = cw_to_float(h[i + half]);
+        if (bias) { a += cw_to_float(bias[head * hd + i]); b += cw_to_float(bias[head * hd + i + half]); }
+        const T oa = cw_from_float<T>(a * cs - b * sn), ob = cw_from_float<T>(b * cs + a * sn);
+        if (head < nh) { h[i] = oa; h[i + half] = ob; }
+        else if (slot >= 0) {
+          T* kdst = k_cache + (slot * nkv + (head - nh)) * (int64_t)hd;
+          kdst[i] = oa; kdst[i + half] = ob;
+        }
       }
-      const T oa = cw_from_float<T>(ra), ob = cw_from_float<T>(rb);
-      if (head < nh) { h[i] = oa; h[i + half] = ob; }
-      else if (kdst) { kdst[i] = oa; kdst[i + half] = ob; }
-    } else {
-      const int j = rotary_dim + (i - half);
-      float a = cw_to_float(h[j]);
-      if (hb) a += cw_to_float(hb[j]);
-      const T oa = cw_from_float<T>(a);
-      if (head < nh) h[j] = oa;
-      else if (kdst) kdst[j] = oa;
     }
+  }
+  // elements past the rotary dimension pass through (bias added)
+  for (int w = threadIdx.x; w < (nh + nkv) * rest; w += blockDim.x) {
+    const int head = w / rest, j = rotary_dim + w % rest;
+    T* h = row + head * hd;
+    float a = cw_to_float(h[j]);
+    if (bias) a += cw_to_float(bias[head * hd + j]);
+    const T oa = cw_from_float<T>(a);
+    if (head < nh) h[j] = oa;
+    else if (slot >= 0) k_cache[(slot * nkv + (head - nh)) * (int64_t)hd + j] = oa;
   }
   if (slot >= 0) {
     const int n_v = nkv * hd;
@@ -188,19 +285,64 @@ __global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ o
   }
 }
 
+// 8 (bfloat16) or 4 (float32) consecutive elements per thread, 16-byte loads and stores.
+template <typename T> struct Vec16B;
+template <> struct Vec16B<float> {
+  static constexpr int N = 4;
+  __device__ static void load(const float* p, float* o) { Chunk4<float>::load(p, o); }
+  __device__ static void store(float* p, const float* v) { Chunk4<float>::store(p, v); }
+};
+template <> struct Vec16B<bf16_t> {
+  static constexpr int N = 8;
+  __device__ static void load(const bf16_t* p, float* o) {
+    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(w[i] << 16); o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+  }
+  __device__ static void store(bf16_t* p, const float* v) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)cw_float_to_bf16_bits(v[2 * i]) | ((uint32_t)cw_float_to_bf16_bits(v[2 * i + 1]) << 16);
+    *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+};
+
+template <typename T>
+__global__ void silu_mul_vec_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int64_t n_vec, int I) {
+  constexpr int N = Vec16B<T>::N;
+  const int per_row = I / N;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n_vec;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = idx / per_row;
+    const int i = (int)(idx - t * per_row) * N;
+    float g[N], u[N], r[N];
+    Vec16B<T>::load(gate_up + t * 2 * I + i, g);
+    Vec16B<T>::load(gate_up + t * 2 * I + I + i, u);
+#pragma unroll
+    for (int e = 0; e < N; ++e) r[e] = g[e] / (1.0f + expf(-g[e])) * u[e];
+    Vec16B<T>::store(out + t * I + i, r);
+  }
+}
+
 CW_EXPORT int cw_silu_mul(const void* gate_up, void* out, int dtype, int T, int I, hipStream_t stream) {
   if (T < 0 || I <= 0) return CW_ERR_ARG;
   if (T == 0) return CW_OK;
-  const int64_t n = (int64_t)T * I;
+  const int vec_n = dtype == CW_BF16 ? 8 : 4;
+  const bool vec = (I % vec_n == 0) && !((uintptr_t)gate_up & 15) && !((uintptr_t)out & 15);
+  const int64_t n = vec ? (int64_t)T * (I / vec_n) : (int64_t)T * I;
   int64_t blocks = (n + 255) / 256;
-  if (blocks > 65536) blocks = 65536;
+  if (blocks > 262144) blocks = 262144;
   dim3 grid((unsigned)blocks), block(256);
-  if (dtype == CW_F32)
-    hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gate_up, (float*)out, n, I);
-  else if (dtype == CW_BF16)
-    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gate_up, (bf16_t*)out, n, I);
-  else
+  if (dtype == CW_F32) {
+    if (vec) hipLaunchKernelGGL(silu_mul_vec_kernel<float>, grid, block, 0, stream, (const float*)gate_up, (float*)out, n, I);
+    else hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gate_up, (float*)out, n, I);
+  } else if (dtype == CW_BF16) {
+    if (vec) hipLaunchKernelGGL(silu_mul_vec_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gate_up, (bf16_t*)out, n, I);
+    else hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gate_up, (bf16_t*)out, n, I);
+  } else {
     return CW_ERR_DTYPE;
+  }
   return cw_launch_status();
 }
 

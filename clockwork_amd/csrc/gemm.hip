@@ -101,8 +101,10 @@ CW_EXPORT int cw_gemm_f32(const float* A, int64_t lda, const float* W, const flo
 
 // =====================================================================================
 // bfloat16 products with few rows of x (decode: 1 to 64 tokens): the weight matrix is streamed
-// once at memory speed. A workgroup of 4 waves owns RT * 16 weight rows; its waves split the K
-// loop and are summed through LDS at the end (no atomics: the result does not depend on timing).
+// once at memory speed. A workgroup of WAVES waves owns RT * 16 weight rows; its waves split the K
+// loop and are summed through LDS at the end, in a fixed order (no atomics: the result does not
+// depend on timing). Few weight rows (a narrow output) get more waves each, so that enough loads
+// are in flight on every compute unit that has work.
 // Each wave feeds 16 weight rows x 32 k-values to one MFMA (v_mfma_f32_16x16x32_bf16) as the A
 // operand, loaded from global memory directly in operand layout (lane = row l%16, 8 consecutive
 // k at slot l/16), and 16 tokens x the same k-values as the B operand.
@@ -113,12 +115,12 @@ CW_EXPORT int cw_gemm_f32(const float* A, int64_t lda, const float* W, const flo
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-template <int MT, int RT, int MODE>
-__global__ __launch_bounds__(256) void gemm_skinny_bf16_kernel(const bf16_t* __restrict__ X, int64_t ldx,
+template <int MT, int RT, int MODE, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16_t* __restrict__ X, int64_t ldx,
                                                                const bf16_t* __restrict__ W,
                                                                void* __restrict__ C, int64_t ldc,
                                                                int M, int N, int K) {
-  __shared__ float red[4][RT * MT * 256];
+  __shared__ float red[WAVES][RT * MT * 256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, s = lane >> 4;
   const int I = N / 2;  // MODE 2 only
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_bf16_kernel(const bf16_t* __r
 
   const int k_steps = (K + 31) / 32;
   constexpr int U = 4;  // k-steps in flight per wave
-  for (int ks0 = wave * U; ks0 < k_steps; ks0 += 4 * U) {
+  for (int ks0 = wave * U; ks0 < k_steps; ks0 += WAVES * U) {
     bf16x8_t wf[U][RT], xf[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -190,13 +192,17 @@ __global__ __launch_bounds__(256) void gemm_skinny_bf16_kernel(const bf16_t* __r
 #pragma unroll
       for (int i = 0; i < 4; ++i) red[wave][(rt * MT + mt) * 256 + (4 * s + i) * 16 + r] = acc[rt][mt][i];
   __syncthreads();
-  for (int idx = threadIdx.x; idx < RT * MT * 256; idx += 256)
-    red[0][idx] = (red[0][idx] + red[1][idx]) + (red[2][idx] + red[3][idx]);
+  for (int idx = threadIdx.x; idx < RT * MT * 256; idx += WAVES * 64) {
+    float sum = red[0][idx];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) sum += red[w][idx];
+    red[0][idx] = sum;
+  }
   __syncthreads();
 
   if (MODE == 2) {
     // outputs: 8 per row tile and token; idx -> (token, rt, j) with j fastest
-    for (int idx = threadIdx.x; idx < RT * MT * 128; idx += 256) {
+    for (int idx = threadIdx.x; idx < RT * MT * 128; idx += WAVES * 64) {
       const int j = idx & 7, rt = (idx >> 3) % RT, m = idx / (8 * RT);
       const int mt = m >> 4, tok = m & 15;
       const int64_t i = ((int64_t)blockIdx.x * RT + rt) * 8 + j;
@@ -206,7 +212,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_bf16_kernel(const bf16_t* __r
       ((bf16_t*)C)[(int64_t)m * ldc + i] = __float2bfloat16(g / (1.0f + __expf(-g)) * u);
     }
   } else {
-    for (int idx = threadIdx.x; idx < RT * MT * 256; idx += 256) {
+    for (int idx = threadIdx.x; idx < RT * MT * 256; idx += WAVES * 64) {
       const int j = idx & 15, rt = (idx >> 4) % RT, m = idx / (16 * RT);
       const int mt = m >> 4, tok = m & 15;
       const int64_t n = ((int64_t)blockIdx.x * RT + rt) * 16 + j;
@@ -220,15 +226,15 @@ __global__ __launch_bounds__(256) void gemm_skinny_bf16_kernel(const bf16_t* __r
 
 #define CW_SKINNY_MAX_M 64
 
-template <int MT, int RT>
+template <int MT, int RT, int WAVES>
 static int launch_skinny(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W, void* C, int64_t ldc,
                          int M, int N, int K, hipStream_t stream) {
   const int rows_per_group = (mode == 2 ? 8 : 16) * RT;
   const int rows = mode == 2 ? N / 2 : N;
-  dim3 grid((rows + rows_per_group - 1) / rows_per_group), block(256);
-  if (mode == 0) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 0>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
-  else if (mode == 1) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 1>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
-  else hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 2>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  dim3 grid((rows + rows_per_group - 1) / rows_per_group), block(WAVES * 64);
+  if (mode == 0) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 0, WAVES>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  else if (mode == 1) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 1, WAVES>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  else hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 2, WAVES>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
   return cw_launch_status();
 }
 
@@ -246,10 +252,20 @@ CW_EXPORT int cw_gemm_bf16_skinny(int mode, const void* X, int64_t ldx, const vo
   const bf16_t* x = (const bf16_t*)X;
   const bf16_t* w = (const bf16_t*)W;
   const int rows = mode == 2 ? N / 2 : N;
-  // more weight rows per workgroup when there are many tokens: x is then re-read less often
-  if (M <= 16) return launch_skinny<1, 1>(mode, x, ldx, w, C, ldc, M, N, K, stream);
-  if (M <= 32) return rows >= 4096 ? launch_skinny<2, 2>(mode, x, ldx, w, C, ldc, M, N, K, stream)
-                                   : launch_skinny<2, 1>(mode, x, ldx, w, C, ldc, M, N, K, stream);
-  return rows >= 4096 ? launch_skinny<4, 2>(mode, x, ldx, w, C, ldc, M, N, K, stream)
-                      : launch_skinny<4, 1>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+  // Few row tiles: more waves on each (a long K loop split 16 ways keeps the loads coming).
+  // Many tokens: more weight rows per workgroup, so x is re-read less often.
+  const int tiles = (rows + (mode == 2 ? 7 : 15)) / (mode == 2 ? 8 : 16);
+  if (M <= 16) {
+    if (tiles <= 256 && K >= 1024) return launch_skinny<1, 1, 16>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+    if (tiles <= 1024 && K >= 512) return launch_skinny<1, 1, 8>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+    return launch_skinny<1, 1, 4>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+  }
+  if (M <= 32) {
+    if (tiles <= 256 && K >= 1024) return launch_skinny<2, 1, 16>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+    return rows >= 4096 ? launch_skinny<2, 2, 4>(mode, x, ldx, w, C, ldc, M, N, K, stream)
+                        : launch_skinny<2, 1, 4>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+  }
+  if (tiles <= 256 && K >= 1024) return launch_skinny<4, 1, 8>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+  return rows >= 4096 ? launch_skinny<4, 2, 4>(mode, x, ldx, w, C, ldc, M, N, K, stream)
+                      : launch_skinny<4, 1, 4>(mode, x, ldx, w, C, ldc, M, N, K, stream);
 }

@@ -134,9 +134,11 @@ class StepContext:
             by_occupancy = -(-4 * self.num_compute_units // groups_running)
             by_length = max(1, longest_single // 256)
             plan.single_splits = max(1, min(by_occupancy, by_length, 64))
-            # decode kernel: a workgroup per (request, kv head, split); at least 128 keys a split
-            base = plan.n_single * nkv * -(-group // min(group, 8))
-            plan.decode_splits = max(1, min(-(-3 * self.num_compute_units // base), longest_single // 128, 64))
+            # decode kernel: a workgroup per (request, kv head, split); a split is at least 128 keys
+            # (one 32-key tile for each of its four waves), and about two workgroups per compute
+            # unit are enough to keep memory busy
+            base = plan.n_single * nkv * -(-group // min(group, 16))
+            plan.decode_splits = max(1, min(-(-2 * self.num_compute_units // base), longest_single // 128, 64))
         packer = _Packer()
         packer.add(wide)
         packer.add(single)
@@ -207,3 +209,101 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int
         ctx.slots.append(views[i_slots])
         ctx.block_tables.append(views[i_table].view(len(entries), width))
     return ctx
+
+
+class StaticDecodeBatch:
+    """A decode-only batch with fixed shapes, for a captured HIP graph.
+
+    ``size`` requests of one token each; every index array lives at a fixed device address and
+    is refreshed by one host-to-device copy per step. Rows past the live requests are padding:
+    token 0 at position 0, no cache slot (-1) and no pages, so they write nothing and read
+    nothing. ``key_capacity`` (the longest context the graph is planned for) only fixes how
+    finely the attention kernel splits its keys.
+    """
+
+    def __init__(self, size: int, key_capacity: int, table_width: int, manager, device, geometries,
+                 num_compute_units: int) -> None:
+        self.size = size
+        self.table_width = table_width
+        n_groups = len(manager.kv_groups)
+        self.block_size = manager.block_size
+        # layout of the packed buffer
+        offsets = {}
+        at = 0
+
+        def take(name, n):
+            nonlocal at
+            offsets[name] = (at, n)
+            at += -(-n // 4) * 4
+
+        for name in ("token_ids", "positions", "ctx_lens", "starts", "state_slots"):
+            take(name, size)
+        for g in range(n_groups):
+            take(f"slots{g}", size)
+            take(f"table{g}", size * table_width)
+        self._offsets = offsets
+        self.host = torch.zeros(at, dtype=torch.int32, pin_memory=True)
+        self.device_buf = torch.zeros(at, dtype=torch.int32, device=device)
+        self._np = self.host.numpy()
+
+        def view(name):
+            o, n = offsets[name]
+            return self.device_buf[o : o + n]
+
+        ctx = StepContext()
+        ctx.device = device
+        ctx.block_size = manager.block_size
+        ctx.num_tokens = ctx.num_requests = ctx.num_logit_rows = size
+        ctx.token_ids, ctx.positions = view("token_ids"), view("positions")
+        ctx.ctx_lens, ctx.starts, ctx.state_slots = view("ctx_lens"), view("starts"), view("state_slots")
+        ctx.cu_q = torch.arange(size + 1, dtype=torch.int32, device=device)
+        ctx.logit_rows = torch.arange(size, dtype=torch.int32, device=device)
+        for g in range(n_groups):
+            ctx.slots.append(view(f"slots{g}"))
+            ctx.block_tables.append(view(f"table{g}").view(size, table_width))
+        ctx.h_q_lens = [1] * size
+        ctx.h_ctx_lens = [key_capacity] * size
+        ctx.h_starts = [0] * size
+        ctx.h_state_slots = [-1] * size
+        ctx.seq_ids = [""] * size
+        ctx.num_compute_units = num_compute_units
+        for nh, nkv in geometries:  # work items are the same every step: made once, outside the graph
+            ctx.attention_plan(nh, nkv)
+        self.ctx = ctx
+
+    def fill(self, entries: Sequence[StepEntry], manager) -> None:
+        """Write this step's indices into the pinned buffer and send them to the device."""
+        n = len(entries)
+        size, width = self.size, self.table_width
+        a = self._np
+
+        def region(name):
+            o, cnt = self._offsets[name]
+            return a[o : o + cnt]
+
+        tok, pos = region("token_ids"), region("positions")
+        ctx_lens, starts, state = region("ctx_lens"), region("starts"), region("state_slots")
+        tok[:] = 0
+        pos[:] = 0
+        ctx_lens[:] = 1
+        starts[:] = 0
+        state[:] = -1
+        for r, e in enumerate(entries):
+            tok[r] = e.tokens[0]
+            pos[r] = e.start
+            ctx_lens[r] = e.start + 1
+            starts[r] = e.start
+            state[r] = manager.state_slot(e.seq_id)
+        for g in range(len(manager.kv_groups)):
+            slots = region(f"slots{g}")
+            table = region(f"table{g}").reshape(size, width)
+            slots[:] = -1
+            table[:] = -1
+            for r, e in enumerate(entries):
+                row = manager.block_table(e.seq_id, g)
+                if len(row) > width:
+                    raise ValueError(f"request {e.seq_id} holds {len(row)} pages, the graph was sized for {width}")
+                table[r, : len(row)] = row
+                slots[r] = manager.slot_mapping(e.seq_id, e.start, e.start + 1, g)[0]
+        self.device_buf.copy_(self.host, non_blocking=True)
+        self.ctx.seq_ids = [e.seq_id for e in entries] + [""] * (size - n)

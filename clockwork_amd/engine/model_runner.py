@@ -19,10 +19,15 @@ from clockwork_amd import ops
 from clockwork_amd.cache.manager import CacheManager, cache_needs_of, plan_groups
 from clockwork_amd.cache.pools import CachePools
 from clockwork_amd.config.engine import EngineConfig
-from clockwork_amd.engine.batch import StepContext, StepEntry, build_context
+from clockwork_amd.engine.batch import StaticDecodeBatch, StepContext, StepEntry, build_context
 from clockwork_amd.parts.model import DecoderModel
 from clockwork_amd.registry import resolve_architecture
 from clockwork_amd.weights.loader import load_parameters, read_config_json
+
+
+# padded batch sizes a decode graph is captured for, and the step in which the planned context grows
+GRAPH_BATCH_SIZES = (1, 2, 4, 8, 16, 24, 32, 48, 64)
+GRAPH_KEY_BUCKET = 512
 
 
 def require_gpu() -> torch.device:
@@ -36,7 +41,7 @@ def require_gpu() -> torch.device:
 
 class ModelRunner:
     def __init__(self, cfg: EngineConfig, weight_source=None, config_dict: Optional[dict] = None,
-                 cache_fill: float = 0.0) -> None:
+                 cache_fill: float = 0.0, use_graphs: bool = True) -> None:
         self.cfg = cfg
         if cfg.model.device not in ("cuda", "cuda:0", "gpu"):
             raise ValueError(f"device {cfg.model.device!r}: this engine runs on the GPU only")
@@ -68,6 +73,11 @@ class ModelRunner:
         )
         self.caches = [self.pools.entry_cache(i, e.cache_from) for i, e in enumerate(self.spec.run)]
         self.num_compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
+        # decode-only steps replay captured HIP graphs: one per (padded batch size, context bucket)
+        self.use_graphs = use_graphs and self.model.graph_safe()
+        self._graphs: dict = {}
+        self._graph_pool = None
+        self._table_width = -(-cfg.model.max_model_len // cfg.cache.block_size)
 
     # ------------------------------------------------------------------ pages
     def reserve(self, seq_id: str, start: int, num_tokens: int, total_len: Optional[int] = None) -> None:
@@ -93,6 +103,50 @@ class ModelRunner:
         if self.manager.has(seq_id):
             self.manager.free(seq_id)
 
+    # ------------------------------------------------------------------ decode steps as graphs
+    def _graph_step(self, entries: Sequence[StepEntry]):
+        """Replay the captured graph for this batch shape. The first step of a shape runs eagerly
+        (it loads and initialises whatever is still lazy), the second is captured, later ones
+        replay. Returns NotImplemented when the step has to take the ordinary path."""
+        n = len(entries)
+        size = next(b for b in GRAPH_BATCH_SIZES if b >= n)
+        longest = max(e.start + 1 for e in entries)
+        if longest > self._table_width * self.manager.block_size:
+            return NotImplemented
+        capacity = GRAPH_KEY_BUCKET * -(-longest // GRAPH_KEY_BUCKET)
+        key = (size, capacity)
+        state = self._graphs.get(key)
+        if state is None:
+            self._graphs[key] = "seen"
+            return NotImplemented
+        for e in entries:
+            if not 0 <= int(e.tokens[0]) < self.spec.vocab_size:
+                raise ValueError(f"request {e.seq_id}: token id {e.tokens[0]} outside the vocabulary")
+            if any(w != 0 for w in e.want):
+                raise ValueError(f"request {e.seq_id}: wanted index outside its 1 token")
+        if state == "seen":
+            batch = StaticDecodeBatch(size, capacity, self._table_width, self.manager, self.device,
+                                      self.model.attention_geometries(), self.num_compute_units)
+            batch.fill(entries, self.manager)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                out = self.model.forward(batch.ctx, self.caches)
+            if self._graph_pool is None:
+                self._graph_pool = graph.pool()
+            state = self._graphs[key] = (batch, graph, out)
+        batch, graph, out = state
+        batch.fill(entries, self.manager)
+        graph.replay()
+        for e in entries:
+            self.manager.release_behind_window(e.seq_id, e.start + 1)
+        rows = [r for r, e in enumerate(entries) if len(e.want)]
+        if not rows:
+            return None
+        if len(rows) == n:
+            return out[:n]
+        return out[torch.tensor(rows, device=self.device)]
+
     # ------------------------------------------------------------------ the step
     @torch.no_grad()
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
@@ -100,6 +154,11 @@ class ModelRunner:
         entries and of each entry's ``want`` (None when nothing is wanted)."""
         if not entries:
             return None
+        if (self.use_graphs and not self.manager.state_groups and len(entries) <= GRAPH_BATCH_SIZES[-1]
+                and all(len(e.tokens) == 1 for e in entries)):
+            logits = self._graph_step(entries)
+            if logits is not NotImplemented:
+                return logits
         if self.manager.state_groups:
             for e in entries:
                 if e.start == 0:

@@ -97,11 +97,11 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_attention_workspace_floats": [I, I, I, I, I],
             "cw_attention": [I, I, P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P, L, P],
             "cw_attention_prefill_supported": [],
-            "cw_attention_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, P],
+            "cw_attention_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, P, P],
             "cw_attention_decode_supported": [],
             "cw_attention_decode_gh": [I],
             "cw_attention_decode_workspace_floats": [I, I, I, I],
-            "cw_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, P],
+            "cw_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, P, P],
         },
     }[name]
     for fn, argtypes in sigs.items():
@@ -256,7 +256,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None) -> 
     return y
 
 
-SKINNY_MAX_ROWS = 64
+# above this many rows the library product is faster than the streaming kernel (measured)
+SKINNY_MAX_ROWS = 16
 
 
 def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
@@ -275,6 +276,17 @@ def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor
                "gemm_bf16_skinny(swiglu)")
         return out
     return silu_mul(linear(x, gate_up_weight), out)
+
+
+_zero_rows: dict = {}
+
+
+def _zero_row(device) -> int:
+    """Address of 1 KiB of zeros on ``device``: what the attention kernels read masked rows from."""
+    t = _zero_rows.get(device)
+    if t is None:
+        t = _zero_rows[device] = torch.zeros(512, dtype=torch.bfloat16, device=device)
+    return t.data_ptr()
 
 
 def prefill_attention_supported(hd: int, dtype: torch.dtype) -> bool:
@@ -299,7 +311,7 @@ def attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx
         _load("attention", hd).cw_attention_prefill_bf16(
             q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
             block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, nh, nkv, block_size,
-            window, float(scale), _stream()),
+            window, float(scale), _zero_row(out.device), _stream()),
         "attention_prefill_bf16",
     )
 
@@ -315,7 +327,8 @@ def decode_attention_workspace_floats(hd: int, n_items: int, nh: int, nkv: int, 
 def attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
                      nh: int, nkv: int, hd: int, block_size: int, n_splits: int, window: int, scale: float,
                      n_tokens: int, n_requests: int, workspace=None) -> None:
-    """Single-token items through the bfloat16 decode kernel; arguments as for ``attention``."""
+    """Single-token items through the bfloat16 decode kernel; arguments as for ``attention``.
+    With more than one split it needs a float32 ``workspace``."""
     _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, workspace)
     _need(q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16, "the decode kernel is bfloat16")
     _need(out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd, "attention output must be [T, nh * hd]")
@@ -336,7 +349,7 @@ def attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_
         lib.cw_attention_decode_bf16(
             q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
             block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, nh, nkv, block_size, n_splits,
-            window, float(scale), _ptr(workspace), ws_floats, _stream()),
+            window, float(scale), _ptr(workspace), ws_floats, _zero_row(out.device), _stream()),
         "attention_decode_bf16",
     )
 

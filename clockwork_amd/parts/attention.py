@@ -19,6 +19,7 @@ from clockwork_amd.registry import build_part
 
 
 class PagedAttention(Part):
+    graph_safe = True
     def __init__(self, spec: AttentionSpec) -> None:
         self.spec = spec
         self.position = build_part(spec.position) if spec.position is not None else NoPosition()

@@ -14,6 +14,7 @@ from clockwork_amd.parts.specs import SwiGLUSpec
 
 
 class SwiGLU(Part):
+    graph_safe = True
     def __init__(self, spec: SwiGLUSpec) -> None:
         self.spec = spec
 

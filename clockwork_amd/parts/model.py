@@ -75,6 +75,25 @@ class DecoderModel:
                 dims.append(int(hd))
         return dims
 
+    def attention_geometries(self) -> list[tuple[int, int]]:
+        """(heads, kv heads) of every attention mixer: what attention work plans are made for."""
+        found = []
+        for layer in self.layers:
+            spec = getattr(layer.mixer, "spec", None)
+            if hasattr(layer.mixer, "position") and spec is not None:
+                geo = (spec.num_heads, spec.num_kv_heads)
+                if geo not in found:
+                    found.append(geo)
+        return found
+
+    def graph_safe(self) -> bool:
+        """True when every part says its step is a fixed sequence of GPU launches (no host reads,
+        no data-dependent shapes), so that a decode step can be captured into a HIP graph."""
+        parts = [self.final_norm]
+        for layer in self.layers:
+            parts += list(layer.parts().values())
+        return all(getattr(part, "graph_safe", False) for part in parts)
+
     def bind(self, params: dict, device, dtype) -> None:
         self.device, self.dtype = device, dtype
         self.embed = params["embed.weight"]

@@ -11,6 +11,7 @@ from clockwork_amd.parts.specs import RMSNormSpec
 
 
 class RMSNorm(Part):
+    graph_safe = True
     def __init__(self, spec: RMSNormSpec) -> None:
         self.spec = spec
 

@@ -10,12 +10,13 @@ from clockwork_amd.engine.batch import StepEntry
 from clockwork_amd.engine.model_runner import ModelRunner
 
 
-def make_runner(model_dir, dtype: str, block_size: int, num_blocks: int, poison: float = float("nan")) -> ModelRunner:
+def make_runner(model_dir, dtype: str, block_size: int, num_blocks: int, poison: float = float("nan"),
+                use_graphs: bool = True, max_model_len: int = 512) -> ModelRunner:
     cfg = EngineConfig.defaults(
         str(model_dir), dtype=dtype, block_size=block_size, num_blocks=num_blocks,
-        enable_prefix_cache=False, watermark=0.0,
+        enable_prefix_cache=False, watermark=0.0, max_model_len=max_model_len,
     )
-    return ModelRunner(cfg, cache_fill=poison)
+    return ModelRunner(cfg, cache_fill=poison, use_graphs=use_graphs)
 
 
 def run_trace(runner: ModelRunner, steps) -> dict:

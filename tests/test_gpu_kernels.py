@@ -184,12 +184,24 @@ def test_skinny_bf16_product(M, N, K):
     want = x.float() @ w.float().t()
     got32 = ops.linear(x, w, out_dtype=torch.float32)
     assert got32.dtype == torch.float32
-    torch.testing.assert_close(got32, want, rtol=1e-4, atol=1e-4)  # float32 accumulation of exact products
+    if M <= ops.SKINNY_MAX_ROWS:
+        torch.testing.assert_close(got32, want, rtol=1e-4, atol=1e-4)  # float32 accumulation of exact products
+    else:
+        torch.testing.assert_close(got32, want, rtol=1e-2, atol=1e-2)  # the library product rounds to bfloat16
     got = ops.linear(x, w)
     assert got.dtype == torch.bfloat16
     torch.testing.assert_close(got.float(), want, rtol=1e-2, atol=1e-2)
-    # a row's result does not depend on the other rows
-    assert torch.equal(ops.linear(x[M - 1 :].contiguous(), w, out_dtype=torch.float32)[0], got32[M - 1])
+    # a row's result does not depend on the other rows, beyond the rounding of a different split of K
+    alone = ops.linear(x[M - 1 :].contiguous(), w, out_dtype=torch.float32)[0]
+    if M <= ops.SKINNY_MAX_ROWS:
+        torch.testing.assert_close(alone, got32[M - 1], rtol=1e-5, atol=1e-5)
+    else:
+        torch.testing.assert_close(alone, got32[M - 1], rtol=1e-2, atol=1e-2)
+    # and not at all on rows that share its launch shape
+    if M > 1:
+        other = x.clone()
+        other[0] = 0
+        assert torch.equal(ops.linear(other, w, out_dtype=torch.float32)[M - 1], got32[M - 1])
 
 
 @pytest.mark.parametrize("M", [1, 8, 20, 64, 100])
@@ -296,8 +308,8 @@ def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs,
         n_splits = splits if splits is not None else plan.decode_splits
         ws = None
         if n_splits > 1:
-            ws = torch.empty(ops.decode_attention_workspace_floats(hd, plan.n_single, nh, nkv, n_splits),
-                             dtype=torch.float32, device=DEV)
+            ws = torch.full((ops.decode_attention_workspace_floats(hd, plan.n_single, nh, nkv, n_splits),), float("nan"),
+                            dtype=torch.float32, device=DEV)
         ops.attention_decode(items=plan.single_items, n_items=plan.n_single, n_splits=n_splits, workspace=ws, **common)
     elif plan.n_single:
         ws = None

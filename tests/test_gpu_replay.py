@@ -74,6 +74,56 @@ def test_first_tokens_and_long_decoding(model_dirs, dtype):
     replay.compare(got, ref, **TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(model_dirs, dtype):
+    """Decode steps replay a captured HIP graph. Every replay is checked against the same step run
+    eagerly by a second runner, over many replays with eager work (prompt portions of another
+    request, a request ending and its pages going to a new one) and synchronisations in between."""
+    name = "B"
+    cfg, _, block_size = TINY_CONFIGS[name]
+    gen = torch.Generator().manual_seed(21)
+    toks = {k: torch.randint(0, cfg["vocab_size"], (n,), generator=gen).tolist() for k, n in
+            {"a": 90, "b": 75, "c": 60, "d": 41}.items()}
+    steps = [{"entries": [{"id": "a", "tokens": toks["a"][:30], "want": [29]}, {"id": "b", "tokens": toks["b"][:20], "want": [19]}], "end": []}]
+    at = {"a": 30, "b": 20, "c": 0, "d": 0}
+
+    def one(ids):
+        entries = []
+        for i in ids:
+            entries.append({"id": i, "tokens": toks[i][at[i] : at[i] + 1], "want": [0]})
+            at[i] += 1
+        return entries
+
+    for i in range(55):
+        if i % 7 == 3 and at["c"] < 40:  # an eager step: a portion of c beside the single tokens
+            entries = one(["a", "b"]) + [{"id": "c", "tokens": toks["c"][at["c"] : at["c"] + 10], "want": [9]}]
+            at["c"] += 10
+            steps.append({"entries": entries, "end": []})
+        elif at["b"] == len(toks["b"]) - 1:
+            steps.append({"entries": one(["a", "b"]), "end": ["b"]})
+        elif at["b"] >= len(toks["b"]):
+            ids = ["a", "c"] + (["d"] if i % 2 else [])  # batch sizes 2 and 3: two graph shapes
+            steps.append({"entries": one([x for x in ids if at[x] < len(toks[x])]), "end": []})
+        else:
+            steps.append({"entries": one(["a", "b"]), "end": []})
+    pages = 40
+    with_graphs = replay.make_runner(model_dirs[name], dtype, block_size, pages, use_graphs=True)
+    eager = replay.make_runner(model_dirs[name], dtype, block_size, pages, use_graphs=False)
+    got_g = replay.run_trace(with_graphs, [dict(s) for s in steps])
+    got_e = replay.run_trace(eager, [dict(s) for s in steps])
+    assert any(isinstance(v, tuple) for v in with_graphs._graphs.values()), "no graph was captured"
+    assert got_g.keys() == got_e.keys() and len(got_g) > 100
+    # the graph plans its attention splits for a padded batch and a context bucket, so sums may be
+    # taken in another order than in the eager step: equal up to that rounding, far inside the
+    # bar that both must meet against the plain implementation
+    close = dict(rtol=2e-6, atol=2e-6) if dtype == "float32" else dict(rtol=1e-2, atol=1e-2)
+    for key in got_e:
+        torch.testing.assert_close(got_g[key], got_e[key], **close, msg=lambda m: f"graph replay differs from the eager step at {key}: {m}")
+    model = PlainQwen2(model_dirs[name])
+    ref = {k: model.logits(v) for k, v in toks.items()}
+    replay.compare(got_g, ref, **TOL[dtype])
+
+
 def test_negative_control_a_small_weight_change_breaks_the_match(model_dirs, tmp_path):
     """tests/test_hf_equivalence.py:141-153: the 1e-5 bar must bite. One q_proj row of layer 1
     moved by 2^-7 is far more than the bar allows."""
