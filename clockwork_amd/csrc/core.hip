@@ -37,22 +37,31 @@ CW_EXPORT int cw_embedding(const void* table, int dtype, const int* ids, float* 
 // rows != nullptr: for i < n: x = resid[rows[i]] + delta[rows[i]], out[i] = norm(x); resid untouched.
 // norm(x) = weight * cast_T(x * 1/sqrt(mean(x^2) + eps)): the cast to T comes before the weight
 // multiply. The sum of squares of a row is reduced in an order that depends on H alone.
-template <typename T, typename WT>
-__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta,
-                                   const WT* __restrict__ weight, float eps, T* __restrict__ out,
-                                   const int* __restrict__ rows, int H) {
+// DT is the type of delta: T, or float when delta is a stack of ``parts`` float32 partial sums
+// [parts, n_rows_of_resid, H] (a product whose K loop was split over workgroups) that are added in order.
+template <typename DT>
+__device__ __forceinline__ float delta_at(const DT* dl, int64_t part_stride, int parts, int j) {
+  float v = cw_to_float(dl[j]);
+  for (int q = 1; q < parts; ++q) v += cw_to_float(dl[q * part_stride + j]);
+  return v;
+}
+
+template <typename T, typename WT, typename DT>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const DT* __restrict__ delta, int parts,
+                                   int64_t part_stride, const WT* __restrict__ weight, float eps,
+                                   T* __restrict__ out, const int* __restrict__ rows, int H) {
   __shared__ float partial[4];
   const int i = blockIdx.x;
   const int t = rows ? rows[i] : i;
   float* x = resid + (int64_t)t * H;
-  const T* dl = delta ? delta + (int64_t)t * H : nullptr;
+  const DT* dl = delta ? delta + (int64_t)t * H : nullptr;
   T* o = out + (int64_t)i * H;
   const bool write_back = rows == nullptr && dl != nullptr;
 
   float ss = 0.0f;
   for (int j = threadIdx.x; j < H; j += 256) {
     float v = x[j];
-    if (dl) v += cw_to_float(dl[j]);
+    if (dl) v += delta_at(dl, part_stride, parts, j);
     if (write_back) x[j] = v;
     ss += v * v;
   }
@@ -64,7 +73,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
   const float inv = 1.0f / sqrtf(total / (float)H + eps);
   for (int j = threadIdx.x; j < H; j += 256) {
     float v = x[j];
-    if (dl && !write_back) v += cw_to_float(dl[j]);
+    if (dl && !write_back) v += delta_at(dl, part_stride, parts, j);
     const T n = cw_from_float<T>(v * inv);
     o[j] = cw_from_float<T>(cw_to_float(weight[j]) * cw_to_float(n));
   }
@@ -97,15 +106,16 @@ template <> struct Chunk4<bf16_t> {
   }
 };
 
-template <typename T, typename WT>
-__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+template <typename T, typename WT, typename DT>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const DT* __restrict__ delta,
+                                                              int parts, int64_t part_stride,
                                                               const WT* __restrict__ weight, float eps,
                                                               T* __restrict__ out, const int* __restrict__ rows, int H) {
   __shared__ float partial[4];
   const int i = blockIdx.x;
   const int t = rows ? rows[i] : i;
   float* x = resid + (int64_t)t * H;
-  const T* dl = delta ? delta + (int64_t)t * H : nullptr;
+  const DT* dl = delta ? delta + (int64_t)t * H : nullptr;
   T* o = out + (int64_t)i * H;
   const bool write_back = rows == nullptr && dl != nullptr;
   const int n_chunks = H / 4;
@@ -121,17 +131,24 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     }
   }
   if (dl) {
-    float d[4][4];
+    float acc[4][4];
+    for (int q = 0; q < parts; ++q) {
+      float d[4][4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int ch = threadIdx.x + k * 256;
-      if (ch < n_chunks) Chunk4<T>::load(dl + ch * 4, d[k]);
-      else d[k][0] = d[k][1] = d[k][2] = d[k][3] = 0.0f;
+      for (int k = 0; k < 4; ++k) {
+        const int ch = threadIdx.x + k * 256;
+        if (ch < n_chunks) Chunk4<DT>::load(dl + q * part_stride + ch * 4, d[k]);
+        else d[k][0] = d[k][1] = d[k][2] = d[k][3] = 0.0f;
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[k][e] = q == 0 ? d[k][e] : acc[k][e] + d[k][e];
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[k][e] += d[k][e];
+      for (int e = 0; e < 4; ++e) v[k][e] += acc[k][e];
   }
   float ss = 0.0f;
 #pragma unroll
@@ -160,27 +177,37 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   }
 }
 
-CW_EXPORT int cw_add_rmsnorm(float* resid, const void* delta, const void* weight, int w_dtype,
-                             float eps, void* out, int dtype, const int* rows, int n, int H,
-                             hipStream_t stream) {
-  if (n < 0 || H <= 0) return CW_ERR_ARG;
+// delta: nullptr, or [T, H] in the activation type (delta_parts == 0), or float32 [delta_parts, T, H].
+CW_EXPORT int cw_add_rmsnorm(float* resid, const void* delta, int delta_parts, int T_rows,
+                             const void* weight, int w_dtype, float eps, void* out, int dtype,
+                             const int* rows, int n, int H, hipStream_t stream) {
+  if (n < 0 || H <= 0 || delta_parts < 0 || delta_parts > 64) return CW_ERR_ARG;
   if (n == 0) return CW_OK;
   dim3 grid(n), block(256);
   const bool vec = (H % 4 == 0) && H <= 4096 && !((uintptr_t)resid & 15) && !((uintptr_t)out & 15) &&
                    !((uintptr_t)weight & 15) && !((uintptr_t)delta & 15);
-#define CW_LAUNCH(T, WT)                                                                              \
-  do {                                                                                                \
-    if (vec)                                                                                          \
-      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, WT>), grid, block, 0, stream, resid,              \
-                         (const T*)delta, (const WT*)weight, eps, (T*)out, rows, H);                  \
-    else                                                                                              \
-      hipLaunchKernelGGL((add_rmsnorm_kernel<T, WT>), grid, block, 0, stream, resid, (const T*)delta, \
-                         (const WT*)weight, eps, (T*)out, rows, H);                                   \
+  const int parts = delta_parts > 0 ? delta_parts : 1;
+  const int64_t part_stride = (int64_t)T_rows * H;
+#define CW_LAUNCH(T, WT, DT)                                                                           \
+  do {                                                                                                 \
+    if (vec)                                                                                           \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, WT, DT>), grid, block, 0, stream, resid,           \
+                         (const DT*)delta, parts, part_stride, (const WT*)weight, eps, (T*)out, rows, H); \
+    else                                                                                               \
+      hipLaunchKernelGGL((add_rmsnorm_kernel<T, WT, DT>), grid, block, 0, stream, resid,               \
+                         (const DT*)delta, parts, part_stride, (const WT*)weight, eps, (T*)out, rows, H); \
   } while (0)
-  if (dtype == CW_F32 && w_dtype == CW_F32) CW_LAUNCH(float, float);
-  else if (dtype == CW_BF16 && w_dtype == CW_BF16) CW_LAUNCH(bf16_t, bf16_t);
-  else if (dtype == CW_BF16 && w_dtype == CW_F32) CW_LAUNCH(bf16_t, float);
-  else return CW_ERR_DTYPE;
+  if (delta_parts > 0) {
+    if (dtype == CW_F32 && w_dtype == CW_F32) CW_LAUNCH(float, float, float);
+    else if (dtype == CW_BF16 && w_dtype == CW_BF16) CW_LAUNCH(bf16_t, bf16_t, float);
+    else if (dtype == CW_BF16 && w_dtype == CW_F32) CW_LAUNCH(bf16_t, float, float);
+    else return CW_ERR_DTYPE;
+  } else {
+    if (dtype == CW_F32 && w_dtype == CW_F32) CW_LAUNCH(float, float, float);
+    else if (dtype == CW_BF16 && w_dtype == CW_BF16) CW_LAUNCH(bf16_t, bf16_t, bf16_t);
+    else if (dtype == CW_BF16 && w_dtype == CW_F32) CW_LAUNCH(bf16_t, float, bf16_t);
+    else return CW_ERR_DTYPE;
+  }
 #undef CW_LAUNCH
   return cw_launch_status();
 }

@@ -111,11 +111,17 @@ CW_EXPORT int cw_gemm_f32(const float* A, int64_t lda, const float* W, const flo
 //
 // MODE 0: y bfloat16 [M, N]; MODE 1: y float32 [M, N] (logits); MODE 2: W is [2I, K] with gate
 // rows first, y[m, i] = silu(gate_i) * up_i as bfloat16 [M, I]: a row tile holds 8 gate rows and
-// the 8 up rows that belong to them.
+// the 8 up rows that belong to them. MODE 3: K is also split over gridDim.y workgroups, each
+// writing its float32 partial product [split, M, N]; whoever reads y next sums the partials in
+// order (the residual-add + norm kernel does): a narrow output with a long K (96 row tiles for
+// 27 MB of weights) then streams on all compute units instead of 96.
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-template <int MT, int RT, int MODE, int WAVES>
+// ROWS (16, 8 or 4) is the number of weight rows a tile really holds: a narrow output with a long K
+// is cut into more, smaller tiles so that every compute unit streams a share of the matrix (the
+// unused rows of the MFMA tile are zeros). MODE 2 needs ROWS == 16.
+template <int MT, int RT, int MODE, int WAVES, int ROWS>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16_t* __restrict__ X, int64_t ldx,
                                                                const bf16_t* __restrict__ W,
                                                                void* __restrict__ C, int64_t ldc,
@@ -136,8 +142,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
       n = (r < 8) ? i : I + i;
       wok[rt] = i < I;
     } else {
-      n = ((int64_t)blockIdx.x * RT + rt) * 16 + r;
-      wok[rt] = n < N;
+      n = ((int64_t)blockIdx.x * RT + rt) * ROWS + r;
+      wok[rt] = r < ROWS && n < N;
     }
     wrow[rt] = W + (wok[rt] ? n : 0) * K;
   }
@@ -162,7 +168,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
 
   const int k_steps = (K + 31) / 32;
   constexpr int U = 4;  // k-steps in flight per wave
-  for (int ks0 = wave * U; ks0 < k_steps; ks0 += WAVES * U) {
+  const int n_ksplit = MODE == 3 ? gridDim.y : 1;
+  for (int ks0 = ((MODE == 3 ? blockIdx.y : 0) * WAVES + wave) * U; ks0 < k_steps; ks0 += n_ksplit * WAVES * U) {
     bf16x8_t wf[U][RT], xf[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -215,10 +222,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
     for (int idx = threadIdx.x; idx < RT * MT * 256; idx += WAVES * 64) {
       const int j = idx & 15, rt = (idx >> 4) % RT, m = idx / (16 * RT);
       const int mt = m >> 4, tok = m & 15;
-      const int64_t n = ((int64_t)blockIdx.x * RT + rt) * 16 + j;
-      if (m >= M || n >= N) continue;
+      const int64_t n = ((int64_t)blockIdx.x * RT + rt) * ROWS + j;
+      if (m >= M || n >= N || j >= ROWS) continue;
       const float v = red[0][(rt * MT + mt) * 256 + j * 16 + tok];
-      if (MODE == 1) ((float*)C)[(int64_t)m * ldc + n] = v;
+      if (MODE == 3) ((float*)C)[((int64_t)blockIdx.y * M + m) * ldc + n] = v;
+      else if (MODE == 1) ((float*)C)[(int64_t)m * ldc + n] = v;
       else ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(v);
     }
   }
@@ -226,24 +234,38 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
 
 #define CW_SKINNY_MAX_M 64
 
-template <int MT, int RT, int WAVES>
+template <int MT, int RT, int WAVES, int ROWS = 16>
 static int launch_skinny(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W, void* C, int64_t ldc,
-                         int M, int N, int K, hipStream_t stream) {
-  const int rows_per_group = (mode == 2 ? 8 : 16) * RT;
+                         int M, int N, int K, int k_splits, hipStream_t stream) {
+  const int rows_per_group = (mode == 2 ? 8 : ROWS) * RT;
   const int rows = mode == 2 ? N / 2 : N;
-  dim3 grid((rows + rows_per_group - 1) / rows_per_group), block(WAVES * 64);
-  if (mode == 0) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 0, WAVES>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
-  else if (mode == 1) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 1, WAVES>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
-  else hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 2, WAVES>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  dim3 grid((rows + rows_per_group - 1) / rows_per_group, mode == 3 ? k_splits : 1), block(WAVES * 64);
+  if (mode == 0) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 0, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  else if (mode == 1) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 1, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  else if (mode == 3) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 3, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  else if (ROWS == 16) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 2, WAVES, 16>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  else return CW_ERR_ARG;
   return cw_launch_status();
 }
 
+// How many ways cw_gemm_bf16_skinny would split K for a partial-sum product of this shape
+// (1: not worth it). The caller allocates [splits, M, N] float32 and passes mode 3.
+CW_EXPORT int cw_gemm_bf16_skinny_ksplits(int M, int N, int K) {
+  const int tiles = (N + 15) / 16;
+  if (M > 16 || tiles > 128 || K < 4096) return 1;
+  int s = 512 / tiles;  // about two workgroups per compute unit
+  if (s > 8) s = 8;
+  while (s > 1 && K / s < 1024) --s;
+  return s < 1 ? 1 : s;
+}
+
 // y = x W^T for M <= 64 rows of bfloat16 x [M, K] (row stride ldx) and bfloat16 W [N, K].
-// mode 0: y bfloat16 [M, N]; 1: y float32 [M, N]; 2: y = silu(gate) * up, bfloat16 [M, N / 2].
+// mode 0: y bfloat16 [M, N]; 1: y float32 [M, N]; 2: y = silu(gate) * up, bfloat16 [M, N / 2];
+// 3: float32 partial products [cw_gemm_bf16_skinny_ksplits(M, N, K), M, N] (M <= 16).
 // K must be a multiple of 8 (16-byte rows).
 CW_EXPORT int cw_gemm_bf16_skinny(int mode, const void* X, int64_t ldx, const void* W, void* C,
                                   int64_t ldc, int M, int N, int K, hipStream_t stream) {
-  if (M < 0 || N <= 0 || K <= 0 || mode < 0 || mode > 2) return CW_ERR_ARG;
+  if (M < 0 || N <= 0 || K <= 0 || mode < 0 || mode > 3) return CW_ERR_ARG;
   if (M > CW_SKINNY_MAX_M) return CW_ERR_SIZE;
   if ((K & 7) || (ldx & 7) || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return CW_ERR_ARG;
   if (mode == 2 && (N & 1)) return CW_ERR_ARG;
@@ -252,20 +274,26 @@ CW_EXPORT int cw_gemm_bf16_skinny(int mode, const void* X, int64_t ldx, const vo
   const bf16_t* x = (const bf16_t*)X;
   const bf16_t* w = (const bf16_t*)W;
   const int rows = mode == 2 ? N / 2 : N;
-  // Few row tiles: more waves on each (a long K loop split 16 ways keeps the loads coming).
-  // Many tokens: more weight rows per workgroup, so x is re-read less often.
   const int tiles = (rows + (mode == 2 ? 7 : 15)) / (mode == 2 ? 8 : 16);
+  if (mode == 3) {
+    const int ks = cw_gemm_bf16_skinny_ksplits(M, N, K);
+    if (M > 16) return CW_ERR_SIZE;
+    return launch_skinny<1, 1, 8>(3, x, ldx, w, C, ldc, M, N, K, ks, stream);
+  }
   if (M <= 16) {
-    if (tiles <= 256 && K >= 1024) return launch_skinny<1, 1, 16>(mode, x, ldx, w, C, ldc, M, N, K, stream);
-    if (tiles <= 1024 && K >= 512) return launch_skinny<1, 1, 8>(mode, x, ldx, w, C, ldc, M, N, K, stream);
-    return launch_skinny<1, 1, 4>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+    // few tiles: many waves on each tile keep enough loads in flight
+    if (tiles <= 256 && K >= 1024) return launch_skinny<1, 1, 16>(mode, x, ldx, w, C, ldc, M, N, K, 1, stream);
+    // very many tiles: several per workgroup, so that x is fetched from L2 less often
+    if (tiles >= 4096) return launch_skinny<1, 4, 4>(mode, x, ldx, w, C, ldc, M, N, K, 1, stream);
+    if (tiles <= 1024 && K >= 512) return launch_skinny<1, 1, 8>(mode, x, ldx, w, C, ldc, M, N, K, 1, stream);
+    return launch_skinny<1, 1, 4>(mode, x, ldx, w, C, ldc, M, N, K, 1, stream);
   }
   if (M <= 32) {
-    if (tiles <= 256 && K >= 1024) return launch_skinny<2, 1, 16>(mode, x, ldx, w, C, ldc, M, N, K, stream);
-    return rows >= 4096 ? launch_skinny<2, 2, 4>(mode, x, ldx, w, C, ldc, M, N, K, stream)
-                        : launch_skinny<2, 1, 4>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+    if (tiles <= 256 && K >= 1024) return launch_skinny<2, 1, 16>(mode, x, ldx, w, C, ldc, M, N, K, 1, stream);
+    return rows >= 4096 ? launch_skinny<2, 2, 4>(mode, x, ldx, w, C, ldc, M, N, K, 1, stream)
+                        : launch_skinny<2, 1, 4>(mode, x, ldx, w, C, ldc, M, N, K, 1, stream);
   }
-  if (tiles <= 256 && K >= 1024) return launch_skinny<4, 1, 8>(mode, x, ldx, w, C, ldc, M, N, K, stream);
-  return rows >= 4096 ? launch_skinny<4, 2, 4>(mode, x, ldx, w, C, ldc, M, N, K, stream)
-                      : launch_skinny<4, 1, 4>(mode, x, ldx, w, C, ldc, M, N, K, stream);
+  if (tiles <= 256 && K >= 1024) return launch_skinny<4, 1, 8>(mode, x, ldx, w, C, ldc, M, N, K, 1, stream);
+  return rows >= 4096 ? launch_skinny<4, 2, 4>(mode, x, ldx, w, C, ldc, M, N, K, 1, stream)
+                      : launch_skinny<4, 1, 4>(mode, x, ldx, w, C, ldc, M, N, K, 1, stream);
 }

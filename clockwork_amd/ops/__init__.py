@@ -77,7 +77,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
     sigs = {
         "core": {
             "cw_embedding": [P, I, P, P, I, I, I, P],
-            "cw_add_rmsnorm": [P, P, P, I, F, P, I, P, I, I, P],
+            "cw_add_rmsnorm": [P, P, I, I, P, I, F, P, I, P, I, I, P],
             "cw_rope_kv_write": [P, I, P, I, P, P, P, I, I, I, I, I, P, P, L, P],
             "cw_silu_mul": [P, P, I, I, I, P],
             "cw_copy_pages": [P, I, L, L, P, I, P],
@@ -86,6 +86,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
         "gemm": {
             "cw_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
             "cw_gemm_bf16_skinny": [I, P, L, P, P, L, I, I, I, P],
+            "cw_gemm_bf16_skinny_ksplits": [I, I, I],
         },
         "sampling": {
             "cw_argmax_chunks": [I],
@@ -151,10 +152,34 @@ def embedding(table: torch.Tensor, ids: torch.Tensor, out_resid: torch.Tensor) -
     return out_resid
 
 
+class PartialSums:
+    """A product whose K loop was split over workgroups: ``parts`` is float32 [splits, M, N] and the
+    value is their sum, taken in order by whoever reads it next (``add_rmsnorm`` does)."""
+
+    __slots__ = ("parts",)
+
+    def __init__(self, parts: torch.Tensor) -> None:
+        self.parts = parts
+
+    @property
+    def shape(self):
+        return self.parts.shape[1:]
+
+    def sum(self, dtype=None) -> torch.Tensor:
+        total = self.parts[0].clone()
+        for i in range(1, self.parts.shape[0]):
+            total += self.parts[i]
+        return total if dtype is None else total.to(dtype)
+
+
 def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None) -> torch.Tensor:
     """resid += delta (when given), out = rmsnorm(resid) * weight; with ``rows`` only those rows
     are normed into out[i] and resid is left alone. resid float32 [T, H]; delta/out in the
-    activation type."""
+    activation type, or delta a :class:`PartialSums` of that shape."""
+    parts = 0
+    if isinstance(delta, PartialSums):
+        parts = delta.parts.shape[0]
+        delta = delta.parts
     _gpu(resid, delta, weight, out, rows)
     T, H = resid.shape
     _need(resid.dtype == torch.float32, "the residual stream is float32")
@@ -163,11 +188,13 @@ def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None) -> torch.Tenso
         _i32(rows, n, "rows")
     _need(tuple(out.shape) == (n, H), f"out must be [{n}, {H}]")
     _need(weight.numel() == H, "norm weight has the wrong size")
-    if delta is not None:
+    if parts:
+        _need(tuple(delta.shape) == (parts, T, H) and delta.dtype == torch.float32, "partial sums must be float32 [parts, T, H]")
+    elif delta is not None:
         _need(tuple(delta.shape) == (T, H) and delta.dtype == out.dtype, "delta must be [T, H] in the activation type")
     _check(
         _load("core").cw_add_rmsnorm(
-            _ptr(resid), _ptr(delta), _ptr(weight), dtype_code(weight.dtype), float(eps), _ptr(out),
+            _ptr(resid), _ptr(delta), parts, T, _ptr(weight), dtype_code(weight.dtype), float(eps), _ptr(out),
             dtype_code(out.dtype), _ptr(rows), n, H, _stream()),
         "add_rmsnorm",
     )
@@ -227,9 +254,12 @@ def copy_pages(pool: torch.Tensor, pairs: torch.Tensor) -> None:
     _check(_load("core").cw_copy_pages(_ptr(pool), planes, num_blocks, block_bytes, _ptr(pairs), pairs.shape[0], _stream()), "copy_pages")
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None) -> torch.Tensor:
-    """y = x @ weight.T (+ bias). float32: the true-float32 HIP product; bfloat16: the library
-    product (as the reference's engine uses one), float32 accumulation."""
+def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, partial_ok: bool = False):
+    """y = x @ weight.T (+ bias). float32: the true-float32 HIP product. bfloat16: few rows go
+    through the weight-streaming kernel, many through the library product (as the reference's
+    engine uses one); float32 accumulation either way. With ``partial_ok`` the result may come
+    back as :class:`PartialSums` (a narrow output with a long K, few rows): only for a result
+    that goes straight into ``add_rmsnorm``."""
     _gpu(x, weight, bias)
     M, K = x.shape
     N = weight.shape[0]
@@ -243,6 +273,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None) -> 
         return out
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "a bfloat16 product needs bfloat16 operands")
     if M <= SKINNY_MAX_ROWS and K % 8 == 0 and bias is None:
+        lib = _load("gemm")
+        if partial_ok and out_dtype is None:
+            splits = lib.cw_gemm_bf16_skinny_ksplits(M, N, K)
+            if splits > 1:
+                parts = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
+                _check(lib.cw_gemm_bf16_skinny(3, _ptr(x), K, _ptr(weight), _ptr(parts), N, M, N, K, _stream()),
+                       "gemm_bf16_skinny(partial)")
+                return PartialSums(parts)
         want_f32 = out_dtype == torch.float32
         out = torch.empty((M, N), dtype=torch.float32 if want_f32 else torch.bfloat16, device=x.device)
         _check(_load("gemm").cw_gemm_bf16_skinny(1 if want_f32 else 0, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, _stream()),

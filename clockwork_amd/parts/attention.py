@@ -90,4 +90,4 @@ class PagedAttention(Part):
                 workspace = torch.empty(need, dtype=torch.float32, device=x.device)
             ops.attention(items=plan.single_items, n_items=plan.n_single, rows=16, gh=plan.gh_single,
                           n_splits=plan.single_splits, workspace=workspace, **common)
-        return ops.linear(out, self.out_weight, self.out_bias)
+        return ops.linear(out, self.out_weight, self.out_bias, partial_ok=True)

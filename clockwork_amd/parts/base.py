@@ -11,12 +11,13 @@ knows which model it is in) and goes through three stages:
 Roles and their run methods:
 
 * norm:          ``forward(resid, delta, rows=None) -> normed`` - ``resid`` is the
-                 float32 residual stream [T, H]; ``delta`` (activation type, or None)
+                 float32 residual stream [T, H]; ``delta`` (activation type, an
+                 ``ops.PartialSums`` of that shape, or None)
                  is added to it in place first; returns the normed rows in the
                  activation type. With ``rows`` only those rows are produced and
                  ``resid`` is left untouched.
 * mixer:         ``forward(x, ctx, cache) -> y`` with x, y [T, H] in the activation
-                 type; ``cache_need()`` returns a KVPagesSpec, a StateSpec or None.
+                 type (y may be an ``ops.PartialSums``: it only ever goes to a norm); ``cache_need()`` returns a KVPagesSpec, a StateSpec or None.
                  ``cache`` is the run entry's :class:`EntryCache`.
 * feed-forward:  ``forward(x, ctx) -> y``.
 * position enc.: used by a mixer, not by the block; the attention mixer expects

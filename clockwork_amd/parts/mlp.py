@@ -27,4 +27,4 @@ class SwiGLU(Part):
         self.down = params["down_weight"]
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        return ops.linear(ops.linear_swiglu(x, self.gate_up), self.down)
+        return ops.linear(ops.linear_swiglu(x, self.gate_up), self.down, partial_ok=True)

@@ -64,6 +64,33 @@ def test_add_rmsnorm(dtype, wdtype, T, H, eps):
     torch.testing.assert_close(out2.float(), want[rows.long()], **tol(dtype))
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 1536, 8960), (8, 1536, 8960), (16, 96, 4096), (3, 1000, 5000 * 8)])
+def test_split_k_partial_sums_feed_the_norm(M, N, K):
+    """A narrow product with a long K comes back as float32 partial sums; the norm kernel adds them
+    to the residual stream in order."""
+    from clockwork_amd import ops
+
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV) / K ** 0.5).to(torch.bfloat16)
+    got = ops.linear(x, w, partial_ok=True)
+    assert isinstance(got, ops.PartialSums) and got.parts.shape[0] > 1 and tuple(got.shape) == (M, N)
+    want = x.float() @ w.float().t()
+    torch.testing.assert_close(got.sum(), want, rtol=1e-4, atol=1e-4)
+    resid = torch.randn(M, N, device=DEV)
+    weight = (1 + 0.1 * torch.randn(N, device=DEV)).to(torch.bfloat16)
+    out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    r = resid.clone()
+    ops.add_rmsnorm(r, got, weight, 1e-6, out)
+    torch.testing.assert_close(r, resid + want, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(out.float().cpu(), plain.rmsnorm((resid + want).cpu(), weight.float().cpu(), 1e-6), **tol(torch.bfloat16))
+    rows = torch.tensor([M - 1], dtype=torch.int32, device=DEV)
+    out1 = torch.empty(1, N, device=DEV, dtype=torch.bfloat16)
+    r2 = resid.clone()
+    ops.add_rmsnorm(r2, got, weight, 1e-6, out1, rows)
+    assert torch.equal(r2, resid) and torch.equal(out1[0], out[M - 1])
+    assert not isinstance(ops.linear(x, w), ops.PartialSums)
+
+
 def test_rmsnorm_zero_row_and_scale_invariance():
     from clockwork_amd import ops
 
