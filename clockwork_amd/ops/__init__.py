@@ -87,6 +87,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
             "cw_gemm_bf16_skinny": [I, P, L, P, P, L, I, I, I, P],
             "cw_gemm_bf16_skinny_ksplits": [I, I, I],
+            "cw_gemm_qkv_rope_bf16": [P, L, P, P, I, P, P, P, P, P, P, L, I, I, I, I, I, P],
         },
         "sampling": {
             "cw_argmax_chunks": [I],
@@ -296,6 +297,37 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
 
 # above this many rows the library product is faster than the streaming kernel (measured)
 SKINNY_MAX_ROWS = 16
+
+
+def qkv_rope_fused_supported(x: torch.Tensor, weight: torch.Tensor, rotary_dim: int, hd: int) -> bool:
+    """The fused q/k/v product + rotary + cache write takes few bfloat16 rows and a full rotary dimension."""
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS
+            and x.shape[1] % 8 == 0 and rotary_dim == hd and hd % 16 == 0)
+
+
+def qkv_rope_fused(x, weight, bias, positions, slots, inv_freq, nh: int, nkv: int, hd: int, k_cache, v_cache) -> torch.Tensor:
+    """q = rope(x @ Wq.T + bq) returned as [M, nh * hd]; rope(x @ Wk.T + bk) and x @ Wv.T + bv written
+    to the cache rows ``slots``: one kernel for few bfloat16 rows (see csrc/gemm.hip)."""
+    _gpu(x, weight, bias, positions, slots, inv_freq, k_cache, v_cache)
+    M, K = x.shape
+    _need(qkv_rope_fused_supported(x, weight, hd, hd), "the fused q/k/v kernel does not take these operands")
+    _need(tuple(weight.shape) == ((nh + 2 * nkv) * hd, K), "qkv weight must be [(nh + 2 nkv) hd, K]")
+    _i32(positions, M, "positions")
+    _i32(slots, M, "slots")
+    _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == hd // 2, "inv_freq must be float32 [hd / 2]")
+    _need(k_cache.dtype == torch.bfloat16 and tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape,
+          "cache must be bfloat16 [..., nkv, hd]")
+    if bias is not None:
+        _need(bias.numel() == weight.shape[0] and bias.dtype in (torch.bfloat16, torch.float32), "qkv bias")
+    q = torch.empty((M, nh * hd), dtype=torch.bfloat16, device=x.device)
+    _check(
+        _load("gemm").cw_gemm_qkv_rope_bf16(
+            _ptr(x), K, _ptr(weight), _ptr(bias), int(bias is not None and bias.dtype == torch.float32), _ptr(positions),
+            _ptr(slots), _ptr(inv_freq), _ptr(q), _ptr(k_cache), _ptr(v_cache), k_cache.numel() // (nkv * hd),
+            M, K, nh, nkv, hd, _stream()),
+        "gemm_qkv_rope_bf16",
+    )
+    return q
 
 
 def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:

@@ -53,7 +53,13 @@ class PagedAttention(Part):
         s = self.spec
         nh, nkv, hd = s.num_heads, s.num_kv_heads, s.head_dim
         T = x.shape[0]
-        if cache.writes:
+        fused = getattr(self.position, "project_rotate_store", None) if cache.writes else None
+        qkv = None
+        if fused is not None:
+            qkv = fused(x, self.qkv_weight, self.qkv_bias, ctx.positions, ctx.slots[cache.group], nh, nkv, hd, cache.k, cache.v)
+        if qkv is not None:
+            pass  # q only, [T, nh * hd]: keys and values are in the cache already
+        elif cache.writes:
             qkv = ops.linear(x, self.qkv_weight)
             self.position.rotate_and_store(
                 qkv, self.qkv_bias, ctx.positions, ctx.slots[cache.group], nh, nkv, hd, cache.k, cache.v

@@ -21,7 +21,10 @@ Roles and their run methods:
                  ``cache`` is the run entry's :class:`EntryCache`.
 * feed-forward:  ``forward(x, ctx) -> y``.
 * position enc.: used by a mixer, not by the block; the attention mixer expects
-                 ``rotate_and_store(qkv, bias, positions, slots, nh, nkv, hd, k, v)``.
+                 ``rotate_and_store(qkv, bias, positions, slots, nh, nkv, hd, k, v)``, and
+                 uses ``project_rotate_store(x, weight, bias, positions, slots, nh, nkv, hd,
+                 k, v) -> q or None`` when the part offers it (product, encoding and cache
+                 write in one kernel).
 * arrangement:   ``forward(resid, delta, ctx, cache) -> delta`` - wires norms,
                  mixer and feed-forward around the residual stream; the returned
                  ``delta`` is the last branch output, not yet added.

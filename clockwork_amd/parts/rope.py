@@ -31,6 +31,15 @@ class RopeNeox(Part):
         ops.rope_kv_write(qkv, bias, positions, slots, self.inv_freq, self.spec.rotary_dim, nh, nkv, hd, k_cache, v_cache)
 
 
+    def project_rotate_store(self, x, weight, bias, positions, slots, nh, nkv, hd, k_cache, v_cache):
+        """Optional fast path of the attention mixer: the q/k/v product, this encoding and the cache
+        write as one kernel. Returns q [T, nh * hd], or None when the shapes do not allow it (the
+        mixer then runs the product and ``rotate_and_store`` apart)."""
+        if slots is None or not ops.qkv_rope_fused_supported(x, weight, self.spec.rotary_dim, hd):
+            return None
+        return ops.qkv_rope_fused(x, weight, bias, positions, slots, self.inv_freq, nh, nkv, hd, k_cache, v_cache)
+
+
 class NoPosition(Part):
     """Stands in when a mixer has no position encoding: bias and cache write only."""
 
