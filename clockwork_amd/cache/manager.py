@@ -76,6 +76,7 @@ class RequestPages:
     released: list[int]                  # per kv group: logical blocks below this index were given back
     state_slot: int = -1
     num_shared_prefix: int = 0           # leading logical blocks that came from the prefix cache
+    epoch: int = 0                       # changes whenever an existing table entry changes (not on appends)
 
 
 class CacheManager:
@@ -99,6 +100,7 @@ class CacheManager:
         self.max_num_seqs = max_num_seqs
         self._free_slots = list(range(max_num_seqs - 1, -1, -1))
         self._requests: dict[str, RequestPages] = {}
+        self._epochs = 0
 
     # ------------------------------------------------------------------ queries
     @property
@@ -106,6 +108,10 @@ class CacheManager:
         """Cached pages are a function of the token prefix alone only when every group keeps
         all keys and nothing else is carried from token to token."""
         return bool(self.kv_groups) and not self.state_groups and all(g.window is None for g in self.kv_groups)
+
+    def _next_epoch(self) -> int:
+        self._epochs += 1
+        return self._epochs
 
     def has(self, seq_id: str) -> bool:
         return seq_id in self._requests
@@ -184,6 +190,7 @@ class CacheManager:
             released=[0] * len(self.pools),
             state_slot=self._free_slots.pop() if self.state_groups else -1,
             num_shared_prefix=len(prefix),
+            epoch=self._next_epoch(),
         )
         self._requests[seq_id] = rec
         return rec
@@ -199,11 +206,26 @@ class CacheManager:
             cow = self.pools[g].is_shared(table[logical])
         return new, cow
 
+    def _fits_as_is(self, rec: RequestPages, computed: int, upto: int) -> bool:
+        """The common case of a decode step: the pages are there and the one written to is private."""
+        size = self.block_size
+        logical = computed // size
+        for g, pool in enumerate(self.pools):
+            table = rec.tables[g]
+            if upto > len(table) * size:
+                return False
+            page = table[logical]
+            if page != NO_PAGE and pool._refs[page] > 1:
+                return False
+        return True
+
     def can_extend(self, seq_id: str, computed: int, upto: int) -> bool:
         """Can the request write positions [computed, upto)? A page boundary needs a free page,
         a shared page under the write position needs one for its private copy
         (block_manager.py:44-54)."""
         rec = self._requests[seq_id]
+        if self._fits_as_is(rec, computed, upto):
+            return True
         for g, pool in enumerate(self.pools):
             new, cow = self._growth(rec, g, computed, upto)
             if new + (1 if cow else 0) > pool.num_free:
@@ -214,6 +236,8 @@ class CacheManager:
         """Back positions [computed, upto). Returns ``(group, src_page, dst_page)`` copies the
         caller must perform on the device before the step runs."""
         rec = self._requests[seq_id]
+        if self._fits_as_is(rec, computed, upto):
+            return []
         if not self.can_extend(seq_id, computed, upto):
             raise OutOfPages(f"sequence {seq_id}: no pages to grow to {upto} tokens")
         copies: list[tuple[int, int, int]] = []
@@ -224,6 +248,7 @@ class CacheManager:
                 logical = computed // self.block_size
                 src, dst = pool.private_copy(table[logical])
                 table[logical] = dst
+                rec.epoch = self._next_epoch()
                 copies.append((g, src, dst))
             table.extend(pool.take_many(new))
         return copies
@@ -241,6 +266,7 @@ class CacheManager:
                 if page != NO_PAGE:
                     pool.drop(page)
                     rec.tables[g][b] = NO_PAGE
+                    rec.epoch = self._next_epoch()
                     given_back += 1
             rec.released[g] = max(rec.released[g], first)
         return given_back
@@ -264,6 +290,7 @@ class CacheManager:
             released=list(parent.released),
             state_slot=slot,
             num_shared_prefix=parent.num_shared_prefix,
+            epoch=self._next_epoch(),
         )
         return (parent.state_slot, slot) if self.state_groups else None
 

@@ -272,10 +272,15 @@ class StaticDecodeBatch:
         self.ctx = ctx
 
     def fill(self, entries: Sequence[StepEntry], manager) -> None:
-        """Write this step's indices into the pinned buffer and send them to the device."""
+        """Write this step's indices into the pinned buffer and send them to the device.
+
+        Block-table rows are kept from step to step: a row is rewritten only when another request
+        moves into it or one of its entries changed (the request's ``epoch`` says so); otherwise
+        just the newly taken pages are added."""
         n = len(entries)
         size, width = self.size, self.table_width
         a = self._np
+        bs = self.block_size
 
         def region(name):
             o, cnt = self._offsets[name]
@@ -283,27 +288,46 @@ class StaticDecodeBatch:
 
         tok, pos = region("token_ids"), region("positions")
         ctx_lens, starts, state = region("ctx_lens"), region("starts"), region("state_slots")
-        tok[:] = 0
-        pos[:] = 0
-        ctx_lens[:] = 1
-        starts[:] = 0
-        state[:] = -1
-        for r, e in enumerate(entries):
-            tok[r] = e.tokens[0]
-            pos[r] = e.start
-            ctx_lens[r] = e.start + 1
-            starts[r] = e.start
-            state[r] = manager.state_slot(e.seq_id)
+        tok[n:] = 0
+        pos[n:] = 0
+        ctx_lens[n:] = 1
+        starts[n:] = 0
+        state[n:] = -1
+        tok[:n] = [e.tokens[0] for e in entries]
+        st = [e.start for e in entries]
+        pos[:n] = st
+        starts[:n] = st
+        ctx_lens[:n] = pos[:n] + 1
+        state[:n] = [manager.state_slot(e.seq_id) for e in entries]
+        rows = getattr(self, "_rows", None)
+        if rows is None:
+            rows = self._rows = [[None, 0] for _ in range(size)]  # per row: epoch of the request in it, pages written
         for g in range(len(manager.kv_groups)):
             slots = region(f"slots{g}")
             table = region(f"table{g}").reshape(size, width)
-            slots[:] = -1
-            table[:] = -1
+            slots[n:] = -1
             for r, e in enumerate(entries):
                 row = manager.block_table(e.seq_id, g)
-                if len(row) > width:
-                    raise ValueError(f"request {e.seq_id} holds {len(row)} pages, the graph was sized for {width}")
-                table[r, : len(row)] = row
-                slots[r] = manager.slot_mapping(e.seq_id, e.start, e.start + 1, g)[0]
+                have = len(row)
+                if have > width:
+                    raise ValueError(f"request {e.seq_id} holds {have} pages, the graph was sized for {width}")
+                state_r = rows[r]
+                epoch = manager.record(e.seq_id).epoch
+                if g > 0 or state_r[0] != epoch or state_r[1] > have:
+                    table[r, :have] = row
+                    table[r, have:] = -1
+                elif state_r[1] < have:
+                    table[r, state_r[1] : have] = row[state_r[1] :]
+                if g == len(manager.kv_groups) - 1:
+                    state_r[0], state_r[1] = epoch, have
+                page = row[e.start // bs]
+                if page < 0:
+                    raise ValueError(f"request {e.seq_id}: position {e.start} lies in a page that was given back")
+                slots[r] = page * bs + e.start % bs
+            for r in range(n, size):
+                if rows[r][0] is not None or g > 0:
+                    table[r, :] = -1
+                    if g == len(manager.kv_groups) - 1:
+                        rows[r][0], rows[r][1] = None, 0
         self.device_buf.copy_(self.host, non_blocking=True)
         self.ctx.seq_ids = [e.seq_id for e in entries] + [""] * (size - n)

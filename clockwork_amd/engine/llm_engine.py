@@ -127,7 +127,7 @@ class LLMEngine:
             StepEntry(
                 p.seq.seq_id,
                 p.start,
-                p.seq.token_ids()[p.start : p.start + p.num_tokens],
+                p.seq.tokens_in(p.start, p.start + p.num_tokens),
                 [p.num_tokens - 1] if p.samples else [],
             )
             for p in out.portions
@@ -239,7 +239,7 @@ class LLMEngine:
             seq.status = SequenceStatus.FINISHED_LENGTH
         return RequestOutput(
             request_id=seq.seq_id,
-            prompt_token_ids=list(seq.prompt_token_ids),
+            prompt_token_ids=seq.prompt_token_ids,  # shared, not copied: a prompt never changes
             token_ids=list(seq.output_token_ids),
             text=state.text,
             finished=seq.is_finished(),

@@ -71,6 +71,15 @@ class Sequence:
     def token_ids(self) -> list[int]:
         return self.prompt_token_ids + self.output_token_ids
 
+    def tokens_in(self, start: int, end: int) -> list[int]:
+        """Tokens at positions [start, end) without building the whole list."""
+        n_prompt = len(self.prompt_token_ids)
+        if end <= n_prompt:
+            return self.prompt_token_ids[start:end]
+        if start >= n_prompt:
+            return self.output_token_ids[start - n_prompt : end - n_prompt]
+        return self.prompt_token_ids[start:] + self.output_token_ids[: end - n_prompt]
+
     def __len__(self) -> int:
         return len(self.prompt_token_ids) + len(self.output_token_ids)
 
