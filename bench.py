@@ -40,7 +40,7 @@ def _sync():
 
 def build_runner(args):
     from clockwork_amd.config.engine import EngineConfig
-    from clockwork_amd.engine.model_runner import ModelRunner
+    from clockwork_amd.engine.model_runner import GRAPH_BATCH_SIZES, ModelRunner
     from clockwork_amd.parts.model import model_param_specs
     from clockwork_amd.registry import resolve_architecture
     from clockwork_amd.weights.random_init import RandomSource
@@ -56,7 +56,11 @@ def build_runner(args):
         num_blocks=max_batch * CONTEXT // BLOCK, enable_prefix_cache=False, watermark=0.0,
         max_num_seqs=max_batch, max_num_batched_tokens=max(PROMPT_LEN, max_batch),
     )
-    return cfg, ModelRunner(cfg, weight_source=source, config_dict=config)
+    runner = ModelRunner(cfg, weight_source=source, config_dict=config)
+    if not args.no_tune:
+        # the engine's start-up option ``tune_products``: the library's fastest kernel per product shape
+        runner.tune_products([PROMPT_LEN, *GRAPH_BATCH_SIZES])
+    return cfg, runner
 
 
 def time_decode(cfg, runner, batch: int, steps: int, warmup: int):
@@ -136,6 +140,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--no-tune", action="store_true", help="leave the matrix library's kernel choice at its default")
     ap.add_argument("--only-prefill", action="store_true", help="run the 2048-token prefill alone (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -25,6 +25,9 @@ class ModelConfig:
     max_model_len: int = 4096
     seed: int = 0
     trust_remote_code: bool = False
+    # at start-up, let the matrix library time its kernels for the products of a full prefill
+    # portion and of the wide decode batches and keep the fastest (bfloat16 only)
+    tune_products: bool = False
 
     def torch_dtype(self):
         import torch

@@ -744,28 +744,64 @@ CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* ou
 }
 
 // =====================================================================================
-// bfloat16 attention for portions of prompts on the matrix cores, without LDS.
+// bfloat16 attention for portions of prompts on the matrix cores.
 //
-// A wave owns 32 query rows (row = token * gh + head of the group, so the group shares every key
-// and value it fetches) and walks tiles of 32 keys up to its last token's position.
-//   S^T[key, row] = K * Q^T     v_mfma_f32_16x16x32_bf16, K and Q fragments loaded from global
-//                               memory directly in operand layout (lane = key or row l%16, 8
-//                               consecutive head elements at slot l/16);
-//   softmax per row in float32: a lane holds 8 keys of one row, two shuffles finish a row;
+// A workgroup takes a run of query tokens of one request and one key/value head. Four waves own
+// 32 query rows each (row = token * gh + head of the group, so the group shares every key and
+// value); for head sizes up to 128 a second set of four waves owns the same rows and the two sets
+// split every stage's keys, so each SIMD holds two waves that hide each other's waits, and the
+// sets' running states are merged through LDS at the end. All waves walk the same stages of keys,
+// which are fetched once per workgroup into LDS, double buffered: the loads of stage t + 1 are in
+// flight while stage t is computed.
+//   S^T[key, row] = K * Q^T     v_mfma_f32_16x16x32_bf16; K fragments come from LDS in operand
+//                               layout (lane = key l%16, 8 consecutive head elements at slot l/16),
+//                               Q fragments are loaded once from global memory the same way;
+//   softmax per row in float32: a lane holds 8 keys of one row; the running maximum is shared by
+//                               the row's 4 lanes every tile, the running sum only at the end;
+//                               tiles that no row masks skip the position tests;
 //   O^T[d, row] += V^T * P^T    P^T is already in operand layout (the lane's 8 keys of its row).
-//                               V^T is made from V with one small MFMA per 16x16 block: V times
-//                               the identity comes back with keys in the lane's registers, which
-//                               is the transposed layout the product needs.
+//                               V^T fragments come from the row-major V tile through the LDS
+//                               transposing read (ds_read_b64_tr_b16): in a group of 16 lanes, lane
+//                               i receives element i%4 of what lanes i/4, 4 + i/4, 8 + i/4 and
+//                               12 + i/4 addressed, so four lanes that point at one key's 16 head
+//                               elements hand every lane its column of 4 keys.
 // The element order inside an MFMA's k dimension is free as long as both operands agree; that
-// is what lets every fragment be filled by plain 8- and 16-byte loads.
+// is what lets every fragment be filled by plain 8- and 16-byte reads.
 typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(8))) short s16x8_t;
+typedef __attribute__((address_space(3))) s16x4_t lds_s16x4_t;
+
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+
+template <int HD>
+struct PrefillTile {
+  static constexpr int KROW = HD + 8;   // K rows: 16 bytes of padding spread the 16-byte reads over the banks
+  static constexpr int VROW = HD + 16;  // V rows: 32 bytes, for the 8-byte transposing reads
+  static constexpr int NH = HD <= 128 ? 2 : 1;  // waves that share a row block and split its keys
+  static constexpr int KW = HD <= 128 ? 64 : 32;  // keys a wave takes from a stage
+  static constexpr int KT = KW * NH;            // keys of one stage
+  static constexpr int NT = 256 * NH;           // threads of a workgroup
+  static constexpr int STAGE = KT * (KROW + VROW);  // elements of one stage: a K tile, then a V tile
+  static constexpr size_t BYTES = 2 * STAGE * sizeof(bf16_t);
+};
 
 template <int HD, bool POW2>
-__global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnParams p) {
-  constexpr int NF = HD / 32;  // k-steps of the score product
-  constexpr int ND = HD / 16;  // 16-wide blocks of the head dimension
-  constexpr bool PIPE = HD <= 128;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+__global__ __launch_bounds__(PrefillTile<HD>::NT, (HD <= 128 ? 2 : 1)) void attn_prefill_bf16_kernel(AttnParams p) {
+  using Tile = PrefillTile<HD>;
+  constexpr int NF = HD / 32;     // k-steps of the score product
+  constexpr int ND = HD / 16;     // 16-wide blocks of the head dimension
+  constexpr int KROW = Tile::KROW, VROW = Tile::VROW;
+  constexpr int CPR = HD / 8;     // 16-byte chunks of a row
+  constexpr int NH = Tile::NH, KW = Tile::KW, KT = Tile::KT, NT = Tile::NT;
+  constexpr int NKB = KW / 16;  // 16-key blocks of a wave's keys
+  constexpr int NCH = (KT * CPR + NT - 1) / NT;  // chunks of a stage per thread
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  bf16_t* tiles = reinterpret_cast<bf16_t*>(smem_raw);  // [stage 2][K tile, V tile]
+  int* tbl = reinterpret_cast<int*>(smem_raw + Tile::BYTES);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = (threadIdx.x >> 6) & 3;  // the wave's row block
+  const int half = threadIdx.x >> 8;        // its share of a stage's keys
   const int c = lane & 15, s = lane >> 4;
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / p.n_chunks, chunk = blockIdx.y % p.n_chunks;
@@ -777,25 +813,26 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnParams p) {
   const int qlen = p.cu_q[req + 1] - q_begin;
   const int group = p.nh / p.nkv;
   const int pos0 = ctx - qlen + tok0;
-  // the pages of every key this workgroup may read -> LDS: no tile waits for a table entry
-  extern __shared__ int tbl[];
+  const int wg_last = pos0 + ntok - 1;
   const int wg_lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
-  const int page0 = cw_page_index<POW2>(wg_lo, p.block_size, p.bs_shift);
+  const int bs = p.block_size, sh = p.bs_shift;
+  // the pages of every key this workgroup may read -> LDS: no tile waits for a table entry
+  const int page0 = cw_page_index<POW2>(wg_lo, bs, sh);
   {
     const int* table = p.block_tables + (int64_t)req * p.table_stride;
-    const int n_pages = cw_page_index<POW2>(pos0 + ntok - 1, p.block_size, p.bs_shift) - page0 + 1;
-    for (int i = threadIdx.x; i < n_pages; i += 256) tbl[i] = table[page0 + i];
+    const int n_pages = cw_page_index<POW2>(wg_last, bs, sh) - page0 + 1;
+    for (int i = threadIdx.x; i < n_pages; i += NT) tbl[i] = table[page0 + i];
   }
   __syncthreads();
-  if (wave * tpw >= ntok) return;
+  const bf16_t* kc = (const bf16_t*)p.k_cache;
+  const bf16_t* vc = (const bf16_t*)p.v_cache;
+  const bf16_t* zrow = (const bf16_t*)p.zeros;
+
+  // ---- the wave's rows: block b, column c -> row b * 16 + c
+  const bool wave_on = wave * tpw < ntok;
   const int p_first = pos0 + wave * tpw;
   const int p_last = pos0 + min(ntok, (wave + 1) * tpw) - 1;
   const int lo = p.window > 0 ? max(0, p_first - p.window + 1) : 0;
-  const bf16_t* kc = (const bf16_t*)p.k_cache;
-  const bf16_t* vc = (const bf16_t*)p.v_cache;
-  const int bs = p.block_size, sh = p.bs_shift;
-
-  // ---- the wave's rows: block b, column c -> row b * 16 + c
   int row_pos[2];      // position of the row's token, -1 for an unused row
   int64_t row_off[2];  // offset of the row's head in q / out, in elements
   bf16x8_t qf[2][NF];
@@ -805,163 +842,196 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnParams p) {
     const int tl = row / gh, g = row - tl * gh;
     const int tokw = wave * tpw + tl;
     const int hig = chunk * gh + g;
-    const bool ok = tl < tpw && tokw < ntok && hig < group;
+    const bool ok = wave_on && tl < tpw && tokw < ntok && hig < group;
     row_pos[b] = ok ? pos0 + tokw : -1;
     row_off[b] = ok ? (int64_t)(kvh * group + hig) * HD : 0;
-    const bf16_t* qrow = (const bf16_t*)p.q + (int64_t)(q_begin + tok0 + (ok ? tokw : 0)) * p.q_stride + row_off[b];
+    const bf16_t* qrow = ok ? (const bf16_t*)p.q + (int64_t)(q_begin + tok0 + tokw) * p.q_stride + row_off[b] : zrow;
 #pragma unroll
-    for (int j = 0; j < NF; ++j) {
-      if (ok) qf[b][j] = *reinterpret_cast<const bf16x8_t*>(qrow + (j * 4 + s) * 8);
-      else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) qf[b][j][e] = (__bf16)0.0f;
-      }
-    }
+    for (int j = 0; j < NF; ++j) qf[b][j] = *reinterpret_cast<const bf16x8_t*>(qrow + (j * 4 + s) * 8);
   }
-  // identity as the B operand of the 16x16x16 product: element (k = 4s + e, n = c)
-  s16x4_t ident;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) ident[e] = (4 * s + e == c) ? (short)0x3F80 : (short)0;
 
   f32x4_t o[2][ND];
 #pragma unroll
   for (int b = 0; b < 2; ++b)
 #pragma unroll
     for (int db = 0; db < ND; ++db) o[b][db] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+  // running maximum in units of the raw score (the scale is positive) and the lane's share of the sum
   float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
+  const float sl2 = p.scale * 1.4426950408889634f;  // exp(x * scale) = exp2(x * sl2)
 
-  // Software pipeline over the key tiles: while tile t is being computed, the key and value
-  // fragments of tile t + 1 are already on their way, and the pages of tile t + 2 are looked up.
-  const int t_first = lo / 32, t_last = p_last / 32;
-  const bf16_t* zrow = (const bf16_t*)p.zeros;
-  // offset of the lane's key of tile t, block kb, in the caches; -1 when it is masked or its page is
-  // gone. A masked key is loaded from a row of zeros, so every load is issued unconditionally and
-  // the number of loads in flight is known at compile time.
-  auto lookup = [&](int t, int kb) -> int64_t {
-    const int kp = t * 32 + kb * 16 + c;
-    bool ok = t <= t_last && kp >= lo && kp <= p_last;
-    const int page = tbl[ok ? cw_page_index<POW2>(kp, bs, sh) - page0 : 0];
-    ok = ok && page >= 0;
-    return ok ? (((int64_t)page * bs + cw_page_offset<POW2>(kp, bs, sh)) * p.nkv + kvh) * HD : -1;
+  // ---- tile traffic: thread -> chunks idx = tid + i * NT of the KT x CPR chunks of K and of V
+  const int t_first = wg_lo / KT, t_last = wg_last / KT;
+  u32x4_t gk[NCH], gv[NCH];
+  auto fetch = [&](int t) __attribute__((always_inline)) {  // global -> registers; a masked key reads a row of zeros
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int idx = threadIdx.x + i * NT;
+      const int key = idx / CPR, ch = idx - key * CPR;
+      const int kp = t * KT + key;
+      bool ok = idx < KT * CPR && kp >= wg_lo && kp <= wg_last;
+      const int page = tbl[ok ? cw_page_index<POW2>(kp, bs, sh) - page0 : 0];
+      ok = ok && page >= 0;
+      const int64_t off = (((int64_t)page * bs + cw_page_offset<POW2>(kp, bs, sh)) * p.nkv + kvh) * HD + ch * 8;
+      gk[i] = *reinterpret_cast<const u32x4_t*>(ok ? kc + off : zrow);
+      gv[i] = *reinterpret_cast<const u32x4_t*>(ok ? vc + off : zrow);
+    }
   };
-  bf16x8_t kf[2][NF], kf_n[2][NF];
-  s16x4_t vf[2][ND], vf_n[2][ND];
-  int64_t off_nn[2];
-  bf16x8_t zero8;
+  auto stash = [&](int stage) __attribute__((always_inline)) {  // registers -> LDS
+    bf16_t* ks = tiles + stage * Tile::STAGE;
+    bf16_t* vs = ks + KT * KROW;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) zero8[e] = (__bf16)0.0f;
-  auto load_frags = [&](int64_t off, bf16x8_t* kf_, s16x4_t* vf_) {
-    const bf16_t* kr = off >= 0 ? kc + off : zrow;
-    const bf16_t* vr = off >= 0 ? vc + off : zrow;
-#pragma unroll
-    for (int j = 0; j < NF; ++j) kf_[j] = *reinterpret_cast<const bf16x8_t*>(kr + (j * 4 + s) * 8);
-#pragma unroll
-    for (int db = 0; db < ND; ++db) vf_[db] = *reinterpret_cast<const s16x4_t*>(vr + db * 16 + 4 * s);
+    for (int i = 0; i < NCH; ++i) {
+      const int idx = threadIdx.x + i * NT;
+      if (idx < KT * CPR) {
+        const int key = idx / CPR, ch = idx - key * CPR;
+        *reinterpret_cast<u32x4_t*>(ks + key * KROW + ch * 8) = gk[i];
+        *reinterpret_cast<u32x4_t*>(vs + key * VROW + ch * 8) = gv[i];
+      }
+    }
   };
-#pragma unroll
-  for (int kb = 0; kb < 2; ++kb) {
-    load_frags(lookup(t_first, kb), kf[kb], vf[kb]);
-    off_nn[kb] = lookup(t_first + 1, kb);
-  }
+  fetch(t_first);
+  stash(0);
+  __syncthreads();
 
   for (int t = t_first; t <= t_last; ++t) {
-    const int kv0 = t * 32;
-    // ---- issue the loads of tile t + 1 and the page lookups of tile t + 2
-    // (head sizes above 128 have no registers to spare for this: they load tile t + 1 late)
+    const int kv0 = t * KT + half * KW;  // the wave's keys of this stage
+    const int stage = (t - t_first) & 1;
+    if (t < t_last) fetch(t + 1);  // in flight while this tile is computed
+    const bool active = wave_on && kv0 <= p_last && kv0 + KW - 1 >= lo;
+    if (active) {
+      const bf16_t* ks = tiles + stage * Tile::STAGE + half * KW * KROW;
+      const bf16_t* vs = tiles + stage * Tile::STAGE + KT * KROW + half * KW * VROW;
+      // ---- S^T = K Q^T
+      f32x4_t sc[NKB][2];
 #pragma unroll
-    for (int kb = 0; kb < 2 && PIPE; ++kb) {
-      load_frags(off_nn[kb], kf_n[kb], vf_n[kb]);
-      off_nn[kb] = lookup(t + 2, kb);
-    }
-    // ---- S^T = K Q^T
-    f32x4_t sc[2][2];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        sc[kb][b] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+      for (int kb = 0; kb < NKB; ++kb) {
+        bf16x8_t kf[NF];
 #pragma unroll
         for (int j = 0; j < NF; ++j)
-          sc[kb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kb][j], qf[b][j], sc[kb][b], 0, 0, 0);
+          kf[j] = *reinterpret_cast<const bf16x8_t*>(ks + (kb * 16 + c) * KROW + (j * 4 + s) * 8);
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          sc[kb][b] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int j = 0; j < NF; ++j)
+            sc[kb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j], qf[b][j], sc[kb][b], 0, 0, 0);
+        }
       }
-    // ---- softmax per row; P^T packed as the B operand of the output product
-    bf16x8_t pf[2];
-    float alpha[2];
+      // ---- softmax per row; P^T packed as the B operand of the output product.
+      // A tile needs the position tests only if some row of the wave masks some key of it.
+      const bool masked = kv0 + KW - 1 > p_first || kv0 < wg_lo || (p.window > 0 && kv0 < p_last - p.window + 1);
+      if (masked) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const int rp = row_pos[b];
+          const int rlo = p.window > 0 ? rp - p.window + 1 : 0;
+#pragma unroll
+          for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int kp = kv0 + kb * 16 + 4 * s + i;
+              if (!(kp <= rp && kp >= rlo)) sc[kb][b][i] = -INFINITY;
+            }
+        }
+      }
+      float tmax[2];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        tmax[b] = fmaxf(fmaxf(sc[0][b][0], sc[0][b][1]), fmaxf(sc[0][b][2], sc[0][b][3]));
+#pragma unroll
+        for (int kb = 1; kb < NKB; ++kb)
+          tmax[b] = fmaxf(tmax[b], fmaxf(fmaxf(sc[kb][b][0], sc[kb][b][1]), fmaxf(sc[kb][b][2], sc[kb][b][3])));
+      }
+#pragma unroll
+      for (int b = 0; b < 2; ++b) tmax[b] = fmaxf(tmax[b], __shfl_xor(tmax[b], 16, 64));
+#pragma unroll
+      for (int b = 0; b < 2; ++b) tmax[b] = fmaxf(tmax[b], __shfl_xor(tmax[b], 32, 64));
+      bf16x8_t pf[2][NKB / 2];
+      float alpha[2];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const float m_new = fmaxf(m_run[b], tmax[b]);
+        // a row that has seen no key yet keeps m = -inf; its probabilities are zero
+        const float msc = m_new == -INFINITY ? 0.0f : m_new * sl2;
+        const float a = __builtin_amdgcn_exp2f(m_run[b] * sl2 - msc);
+        float psum = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float pe = __builtin_amdgcn_exp2f(fmaf(sc[kb][b][i], sl2, -msc));
+            psum += pe;
+            pf[b][kb / 2][(kb & 1) * 4 + i] = (__bf16)pe;
+          }
+        l_run[b] = l_run[b] * a + psum;
+        m_run[b] = m_new;
+        alpha[b] = a;
+      }
+      if (__any(alpha[0] != 1.0f || alpha[1] != 1.0f)) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int db = 0; db < ND; ++db) o[b][db] *= alpha[b];
+      }
+      // ---- O^T += V^T P^T, one 16-wide block of the head dimension at a time
+      const bf16_t* vlane = vs + (4 * s + (c >> 2)) * VROW + 4 * (c & 3);
+#pragma unroll
+      for (int k2 = 0; k2 < NKB / 2; ++k2)
+#pragma unroll
+        for (int db = 0; db < ND; ++db) {
+          const bf16_t* vp = vlane + k2 * 32 * VROW + db * 16;
+          const s16x4_t v0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)vp);
+          const s16x4_t v1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(vp + 16 * VROW));
+          const bf16x8_t vt = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+          for (int b = 0; b < 2; ++b) o[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pf[b][k2], o[b][db], 0, 0, 0);
+        }
+    }
+    if (t < t_last) stash(stage ^ 1);  // tile t + 1, read in the next round; nobody reads that buffer now
+    __syncthreads();
+  }
+
+  // ---- the waves of the second half hand their rows' state to the first half through LDS
+  // (the tiles are dead after the loop's last barrier): o, then m and l, lanes side by side
+  if constexpr (NH == 2) {
+    f32x4_t* xo = reinterpret_cast<f32x4_t*>(smem_raw);
+    float* xml = reinterpret_cast<float*>(smem_raw + (size_t)4 * 2 * ND * 64 * sizeof(f32x4_t));
+    if (half == 1) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+#pragma unroll
+        for (int db = 0; db < ND; ++db) xo[((wave * 2 + b) * ND + db) * 64 + lane] = o[b][db];
+        xml[((wave * 2 + b) * 2 + 0) * 64 + lane] = m_run[b];
+        xml[((wave * 2 + b) * 2 + 1) * 64 + lane] = l_run[b];
+      }
+    }
+    __syncthreads();
+    if (half == 1) return;
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      const int rp = row_pos[b];
-      const int rlo = p.window > 0 ? rp - p.window + 1 : 0;
-      float sv[8];
-      float tmax = -INFINITY;
+      const float m1 = xml[((wave * 2 + b) * 2 + 0) * 64 + lane];
+      const float l1 = xml[((wave * 2 + b) * 2 + 1) * 64 + lane];
+      const float m = fmaxf(m_run[b], m1);
+      const float msc = m == -INFINITY ? 0.0f : m * sl2;
+      const float a0 = __builtin_amdgcn_exp2f(m_run[b] * sl2 - msc);
+      const float a1 = __builtin_amdgcn_exp2f(m1 * sl2 - msc);
+      l_run[b] = l_run[b] * a0 + l1 * a1;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int kp = kv0 + kb * 16 + 4 * s + i;
-          const float v = (kp <= rp && kp >= rlo) ? sc[kb][b][i] * p.scale : -INFINITY;
-          sv[kb * 4 + i] = v;
-          tmax = fmaxf(tmax, v);
-        }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m_run[b], tmax);
-      float a = 1.0f, psum = 0.0f;
-      if (m_new != -INFINITY) {
-        a = __expf(m_run[b] - m_new);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float pe = __expf(sv[e] - m_new);
-          psum += pe;
-          pf[b][e] = (__bf16)pe;
-        }
-      } else {
-        pf[b] = zero8;
+      for (int db = 0; db < ND; ++db) {
+        const f32x4_t o1 = xo[((wave * 2 + b) * ND + db) * 64 + lane];
+        o[b][db] = o[b][db] * a0 + o1 * a1;
       }
-      psum += __shfl_xor(psum, 16, 64);
-      psum += __shfl_xor(psum, 32, 64);
-      l_run[b] = l_run[b] * a + psum;
-      m_run[b] = m_new;
-      alpha[b] = a;
-    }
-    if (__any(alpha[0] != 1.0f || alpha[1] != 1.0f)) {
-#pragma unroll
-      for (int b = 0; b < 2; ++b)
-#pragma unroll
-        for (int db = 0; db < ND; ++db) o[b][db] *= alpha[b];
-    }
-    // ---- O^T += V^T P^T, one 16-wide block of the head dimension at a time
-#pragma unroll
-    for (int db = 0; db < ND; ++db) {
-      bf16x8_t vt;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const f32x4_t tr = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[kb][db], ident, (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) vt[kb * 4 + i] = (__bf16)tr[i];
-      }
-#pragma unroll
-      for (int b = 0; b < 2; ++b) o[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pf[b], o[b][db], 0, 0, 0);
-    }
-    // ---- tile t + 1 becomes the current tile
-#pragma unroll
-    for (int kb = 0; kb < 2 && !PIPE; ++kb) {
-      load_frags(off_nn[kb], kf[kb], vf[kb]);
-      off_nn[kb] = lookup(t + 2, kb);
-    }
-#pragma unroll
-    for (int kb = 0; kb < 2 && PIPE; ++kb) {
-#pragma unroll
-      for (int j = 0; j < NF; ++j) kf[kb][j] = kf_n[kb][j];
-#pragma unroll
-      for (int db = 0; db < ND; ++db) vf[kb][db] = vf_n[kb][db];
     }
   }
 
   // ---- out[row][d]: lane (c, s) holds d = db * 16 + 4s .. + 3 of row (b, c)
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
+    float l = l_run[b];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
     if (row_pos[b] < 0) continue;
-    const float inv = 1.0f / l_run[b];
+    const float inv = 1.0f / l;
     bf16_t* orow = (bf16_t*)p.out + (int64_t)(q_begin + (row_pos[b] - (ctx - qlen))) * p.out_stride + row_off[b];
 #pragma unroll
     for (int db = 0; db < ND; ++db) {
@@ -1006,8 +1076,9 @@ CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* o
   p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = 1; p.window = window; p.scale = scale;
   p.part_o = nullptr; p.part_ml = nullptr; p.counters = nullptr; p.zeros = zeros;
   if ((int64_t)nkv * p.n_chunks > 65535) return CW_ERR_SIZE;
-  dim3 grid(n_items, nkv * p.n_chunks), block(256);
-  const size_t smem = sizeof(int) * ((size_t)table_stride + 2);  // a request's whole table fits
+  dim3 grid(n_items, nkv * p.n_chunks), block(PrefillTile<CW_HD>::NT);
+  // two stages of a 32-key K and V tile, then a request's whole table
+  const size_t smem = PrefillTile<CW_HD>::BYTES + sizeof(int) * ((size_t)table_stride + 2);
   if (smem > 160 * 1024) return CW_ERR_SIZE;
   if (p.bs_shift >= 0) {
     static size_t raised = 0;

@@ -16,7 +16,7 @@ from typing import Optional
 from clockwork_amd.cache.prefix import PrefixCache
 from clockwork_amd.config.engine import EngineConfig
 from clockwork_amd.engine.batch import StepEntry
-from clockwork_amd.engine.model_runner import ModelRunner
+from clockwork_amd.engine.model_runner import GRAPH_BATCH_SIZES, ModelRunner
 from clockwork_amd.engine.scheduler import Scheduler
 from clockwork_amd.engine.sequence import RequestOutput, SamplingParams, Sequence, SequenceStatus
 from clockwork_amd.sampling.sampler import Sampler
@@ -38,6 +38,11 @@ class LLMEngine:
         )
         self.tokenizer = tokenizer
         self.manager = self.runner.manager
+        if cfg.model.tune_products:
+            chunk = cfg.scheduler.max_num_batched_tokens
+            if cfg.scheduler.max_prefill_chunk > 0:
+                chunk = min(chunk, cfg.scheduler.max_prefill_chunk)
+            self.runner.tune_products([chunk, *GRAPH_BATCH_SIZES])
         self.prefix_cache = PrefixCache(
             cfg.cache.block_size,
             share=self.manager.share_handle,

@@ -103,6 +103,33 @@ class ModelRunner:
         if self.manager.has(seq_id):
             self.manager.free(seq_id)
 
+    # ------------------------------------------------------------------ library products
+    @torch.no_grad()
+    def tune_products(self, token_counts: Sequence[int]) -> list[int]:
+        """Let the matrix library choose its fastest kernel for the products of steps with these
+        token counts: each count runs once as a throwaway request while tuning is on. Counts the
+        hand-written narrow products serve, float32 models (no library product) and counts that
+        the cache cannot hold are skipped. Returns the counts that ran."""
+        done: list[int] = []
+        if self.dtype != torch.bfloat16:
+            return done
+        limit = min(self.cfg.model.max_model_len, self._table_width * self.manager.block_size)
+        for n in sorted({int(c) for c in token_counts}, reverse=True):
+            if n <= ops.SKINNY_MAX_ROWS or n > limit:
+                continue
+            seq_id = "__tune_products__"
+            if not self.manager.can_admit(n, n):
+                continue
+            self.reserve(seq_id, 0, n, total_len=n)
+            try:
+                with ops.library_tuning():
+                    self.step([StepEntry(seq_id, 0, [0] * n, [n - 1])])
+                torch.cuda.synchronize()
+                done.append(n)
+            finally:
+                self.release(seq_id)
+        return done
+
     # ------------------------------------------------------------------ decode steps as graphs
     def _graph_step(self, entries: Sequence[StepEntry]):
         """Replay the captured graph for this batch shape. The first step of a shape runs eagerly

@@ -9,7 +9,10 @@ loaded the call raises.
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
+import os
+import tempfile
 from ctypes import c_float, c_int, c_int64, c_void_p
 
 import torch
@@ -297,6 +300,25 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
 
 # above this many rows the library product is faster than the streaming kernel (measured)
 SKINNY_MAX_ROWS = 16
+
+
+@contextlib.contextmanager
+def library_tuning():
+    """While active, a library product of a shape not seen before is timed over the library's
+    candidate kernels and the fastest is remembered; afterwards the remembered choices stay in
+    use and unseen shapes take the library's own default again. The choices are kept in a file
+    in the temporary folder (or where PYTORCH_TUNABLEOP_FILENAME points), which later processes
+    of the same user read. Not to be left active during HIP-graph capture."""
+    import torch.cuda.tunable as tunable
+
+    if not os.environ.get("PYTORCH_TUNABLEOP_FILENAME"):
+        tunable.set_filename(os.path.join(tempfile.gettempdir(), f"clockwork_amd_products_{os.getuid()}.csv"), True)
+    tunable.enable(True)
+    tunable.tuning_enable(True)
+    try:
+        yield
+    finally:
+        tunable.tuning_enable(False)
 
 
 def qkv_rope_fused_supported(x: torch.Tensor, weight: torch.Tensor, rotary_dim: int, hd: int) -> bool:
