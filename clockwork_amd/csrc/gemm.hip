@@ -232,6 +232,194 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
   }
 }
 
+// The same product when a wave's share of the K loop is short (at most 8 steps of 32): the wave
+// keeps its x fragments (MT tiles of 16 tokens) in registers for good, so only weights move.
+// A workgroup walks over row tiles blockIdx.x, blockIdx.x + gridDim.x, ...; the weights of its
+// next tile are on their way while the current one is reduced through LDS (one barrier per tile
+// while the reduction buffer can be doubled, two for MT = 4). Loads are never conditional: a row
+// or k-step outside the matrix reads a valid address instead and meets zeros in x or is not
+// stored, which lets the compiler wait for exactly the loads a product needs. Wave w of k-split
+// blockIdx.y owns k-steps [(blockIdx.y * WAVES + w) * SPW, + SPW). Modes and layouts as in
+// gemm_skinny_bf16_kernel.
+template <int MODE, int WAVES, int SPW, int MT>
+__global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16_t* __restrict__ X, int64_t ldx,
+                                                               const bf16_t* __restrict__ W,
+                                                               void* __restrict__ C, int64_t ldc,
+                                                               int M, int N, int K, int n_tiles) {
+  constexpr int NBUF = MT <= 2 ? 2 : 1;
+  __shared__ float red[NBUF][WAVES][MT * 256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, s = lane >> 4;
+  const int I = N / 2;  // MODE 2 only
+
+  bf16x8_t xf[SPW][MT];
+  int koff[SPW];
+#pragma unroll
+  for (int u = 0; u < SPW; ++u) {
+    const int k = ((blockIdx.y * WAVES + wave) * SPW + u) * 32 + s * 8;
+    const bool kok = k + 8 <= K;
+    koff[u] = kok ? k : 0;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xf[u][mt][e] = (__bf16)0.0f;
+      if (kok && mt * 16 + r < M) xf[u][mt] = *reinterpret_cast<const bf16x8_t*>(X + (int64_t)(mt * 16 + r) * ldx + k);
+    }
+  }
+  auto wrow = [&](int tile) __attribute__((always_inline)) -> const bf16_t* {
+    int64_t n;
+    if (MODE == 2) {
+      const int64_t i = min((int64_t)tile * 8 + (r & 7), (int64_t)I - 1);
+      n = (r < 8) ? i : I + i;
+    } else {
+      n = min((int64_t)tile * 16 + r, (int64_t)N - 1);
+    }
+    return W + n * K;
+  };
+
+  int tile = blockIdx.x;
+  bf16x8_t cur[SPW], nxt[SPW];
+  {
+    const bf16_t* w = wrow(tile);
+#pragma unroll
+    for (int u = 0; u < SPW; ++u) cur[u] = *reinterpret_cast<const bf16x8_t*>(w + koff[u]);
+  }
+  int buf = 0;
+  for (; tile < n_tiles; tile += gridDim.x) {
+    {
+      const bf16_t* w = wrow(min(tile + (int)gridDim.x, n_tiles - 1));
+#pragma unroll
+      for (int u = 0; u < SPW; ++u) nxt[u] = *reinterpret_cast<const bf16x8_t*>(w + koff[u]);
+    }
+    f32x4_t acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int u = 0; u < SPW; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], xf[u][mt], acc[mt], 0, 0, 0);
+    // lane (r, s) holds weight rows 4s..4s+3 of token r of tile mt -> red[buf][wave][mt][row][token]
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[buf][wave][mt * 256 + (4 * s + i) * 16 + r] = acc[mt][i];
+    __syncthreads();
+    if (MODE == 2) {
+      if (threadIdx.x < MT * 128) {  // (token, j): 8 outputs of a token lie side by side
+        const int j = threadIdx.x & 7, m = threadIdx.x >> 3;
+        const int at = (m >> 4) * 256 + (m & 15);
+        float g = 0.0f, up = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+          g += red[buf][w][at + j * 16];
+          up += red[buf][w][at + (j + 8) * 16];
+        }
+        const int64_t i = (int64_t)tile * 8 + j;
+        if (m < M && i < I) ((bf16_t*)C)[(int64_t)m * ldc + i] = __float2bfloat16(g / (1.0f + __expf(-g)) * up);
+      }
+    } else {
+      for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {  // (token, j): 16 outputs side by side
+        const int j = idx & 15, m = idx >> 4;
+        const int at = (m >> 4) * 256 + (m & 15) + j * 16;
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) v += red[buf][w][at];
+        const int64_t n = (int64_t)tile * 16 + j;
+        if (m < M && n < N) {
+          if (MODE == 3) ((float*)C)[((int64_t)blockIdx.y * M + m) * ldc + n] = v;
+          else if (MODE == 1) ((float*)C)[(int64_t)m * ldc + n] = v;
+          else ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(v);
+        }
+      }
+    }
+    if (NBUF == 1) __syncthreads();
+#pragma unroll
+    for (int u = 0; u < SPW; ++u) cur[u] = nxt[u];
+    buf = (buf + 1) % NBUF;
+  }
+}
+
+static int cw_num_compute_units() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
+    cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }
+  return cus;
+}
+
+// Do a wave's x fragments, two sets of weight fragments and the accumulators fit its registers?
+constexpr bool cw_stream_fits(int waves, int spw, int mt) {
+  return spw * mt * 4 + spw * 8 + mt * 4 <= (waves == 16 ? 100 : 220);
+}
+
+template <int MODE, int WAVES, int SPW, int MT>
+static int launch_stream_one(dim3 grid, const bf16_t* X, int64_t ldx, const bf16_t* W, void* C, int64_t ldc,
+                             int M, int N, int K, int n_tiles, hipStream_t stream) {
+  if constexpr (cw_stream_fits(WAVES, SPW, MT)) {
+    hipLaunchKernelGGL((gemm_stream_bf16_kernel<MODE, WAVES, SPW, MT>), grid, dim3(WAVES * 64), 0, stream, X, ldx,
+                       W, C, ldc, M, N, K, n_tiles);
+    return cw_launch_status();
+  } else {
+    return CW_ERR_SIZE;
+  }
+}
+
+template <int MODE, int WAVES, int MT>
+static int launch_stream(int spw, dim3 grid, const bf16_t* X, int64_t ldx, const bf16_t* W, void* C, int64_t ldc,
+                         int M, int N, int K, int n_tiles, hipStream_t stream) {
+#define CW_STREAM(SPW_) \
+  case SPW_: return launch_stream_one<MODE, WAVES, SPW_, MT>(grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream)
+  switch (spw) {
+    CW_STREAM(1); CW_STREAM(2); CW_STREAM(3); CW_STREAM(4); CW_STREAM(5); CW_STREAM(6); CW_STREAM(7); CW_STREAM(8);
+    default: return CW_ERR_SIZE;
+  }
+#undef CW_STREAM
+}
+
+template <int MODE, int WAVES>
+static int launch_stream_mt(int mt, int spw, dim3 grid, const bf16_t* X, int64_t ldx, const bf16_t* W, void* C,
+                            int64_t ldc, int M, int N, int K, int n_tiles, hipStream_t stream) {
+  if (mt == 1) return launch_stream<MODE, WAVES, 1>(spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
+  if (mt == 2) return launch_stream<MODE, WAVES, 2>(spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
+  return launch_stream<MODE, WAVES, 4>(spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
+}
+
+// Shape of the streaming kernel's launch for this product, or false if it does not apply: a
+// wave's share of K must be short enough for its registers and there must be enough row tiles.
+static bool plan_stream(int mode, int M, int N, int K, int k_splits, int* mt, int* spw, dim3* grid, int* n_tiles) {
+  const int k_steps = (K + 31) / 32;
+  *n_tiles = mode == 2 ? (N / 2 + 7) / 8 : (N + 15) / 16;
+  const int waves = mode == 3 ? 8 : 16;
+  *mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  *spw = (k_steps + k_splits * waves - 1) / (k_splits * waves);
+  if (M > 64 || *spw > 8 || !cw_stream_fits(waves, *spw, *mt) || (mode != 3 && k_steps < 2 * waves)) return false;
+  // tiles per workgroup: one workgroup on every compute unit (a second round of these large
+  // workgroups costs more than it brings), each with the same share
+  // (up to 16 rows the one-tile kernels are as fast below two rounds; beyond, the alternative
+  // is a library product that is slower as soon as half the compute units have a tile)
+  const int slots = cw_num_compute_units();
+  if ((int64_t)*n_tiles * k_splits < (M <= 16 ? 2 * slots : slots / 2)) return false;
+  const int per = (*n_tiles * k_splits + slots - 1) / slots;
+  *grid = dim3((*n_tiles + per - 1) / per, k_splits);
+  return true;
+}
+
+static int try_stream(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W, void* C, int64_t ldc,
+                      int M, int N, int K, int k_splits, hipStream_t stream) {
+  int mt, spw, n_tiles;
+  dim3 grid;
+  if (!plan_stream(mode, M, N, K, k_splits, &mt, &spw, &grid, &n_tiles)) return CW_ERR_SIZE;
+  switch (mode) {
+    case 0: return launch_stream_mt<0, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
+    case 1: return launch_stream_mt<1, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
+    case 2: return launch_stream_mt<2, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
+    default: return launch_stream_mt<3, 8>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
+  }
+}
+
 #define CW_SKINNY_MAX_M 64
 
 template <int MT, int RT, int WAVES, int ROWS = 16>
@@ -252,11 +440,28 @@ static int launch_skinny(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W
 // (1: not worth it). The caller allocates [splits, M, N] float32 and passes mode 3.
 CW_EXPORT int cw_gemm_bf16_skinny_ksplits(int M, int N, int K) {
   const int tiles = (N + 15) / 16;
-  if (M > 16 || tiles > 128 || K < 4096) return 1;
+  if (M > 64 || tiles > 128 || K < 4096) return 1;
   int s = 512 / tiles;  // about two workgroups per compute unit
   if (s > 8) s = 8;
   while (s > 1 && K / s < 1024) --s;
-  return s < 1 ? 1 : s;
+  if (s < 1) s = 1;
+  if (M > 16) {  // only the streaming kernel takes partial sums of more than 16 rows
+    int mt, spw, n_tiles;
+    dim3 grid;
+    if (s == 1 || !plan_stream(3, M, N, K, s, &mt, &spw, &grid, &n_tiles)) return 1;
+  }
+  return s;
+}
+
+// 1 if cw_gemm_bf16_skinny streams the weights once for this shape at full speed: every shape
+// with M <= 16, and the shapes with 16 < M <= 64 that the streaming kernel takes (other shapes of
+// that range run, but a library product is faster). mode 3 is answered by ..._ksplits() > 1.
+CW_EXPORT int cw_gemm_bf16_skinny_fast(int mode, int M, int N, int K) {
+  if (M <= 16) return 1;
+  if (mode < 0 || mode > 2) return 0;
+  int mt, spw, n_tiles;
+  dim3 grid;
+  return plan_stream(mode, M, N, K, 1, &mt, &spw, &grid, &n_tiles) ? 1 : 0;
 }
 
 // y = x W^T for M <= 64 rows of bfloat16 x [M, K] (row stride ldx) and bfloat16 W [N, K].
@@ -277,8 +482,14 @@ CW_EXPORT int cw_gemm_bf16_skinny(int mode, const void* X, int64_t ldx, const vo
   const int tiles = (rows + (mode == 2 ? 7 : 15)) / (mode == 2 ? 8 : 16);
   if (mode == 3) {
     const int ks = cw_gemm_bf16_skinny_ksplits(M, N, K);
+    const int rc = try_stream(3, x, ldx, w, C, ldc, M, N, K, ks, stream);
+    if (rc != CW_ERR_SIZE) return rc;
     if (M > 16) return CW_ERR_SIZE;
     return launch_skinny<1, 1, 8>(3, x, ldx, w, C, ldc, M, N, K, ks, stream);
+  }
+  {
+    const int rc = try_stream(mode, x, ldx, w, C, ldc, M, N, K, 1, stream);
+    if (rc != CW_ERR_SIZE) return rc;
   }
   if (M <= 16) {
     // few tiles: many waves on each tile keep enough loads in flight

@@ -90,6 +90,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
             "cw_gemm_bf16_skinny": [I, P, L, P, P, L, I, I, I, P],
             "cw_gemm_bf16_skinny_ksplits": [I, I, I],
+            "cw_gemm_bf16_skinny_fast": [I, I, I, I],
             "cw_gemm_qkv_rope_bf16": [P, L, P, P, I, P, P, P, P, P, P, L, I, I, I, I, I, P],
         },
         "sampling": {
@@ -276,7 +277,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
         _check(_load("gemm").cw_gemm_f32(_ptr(x), K, _ptr(weight), _ptr(bias), _ptr(out), N, M, N, K, _stream()), "gemm_f32")
         return out
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "a bfloat16 product needs bfloat16 operands")
-    if M <= SKINNY_MAX_ROWS and K % 8 == 0 and bias is None:
+    if M <= STREAM_MAX_ROWS and K % 8 == 0 and bias is None:
         lib = _load("gemm")
         if partial_ok and out_dtype is None:
             splits = lib.cw_gemm_bf16_skinny_ksplits(M, N, K)
@@ -286,10 +287,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
                        "gemm_bf16_skinny(partial)")
                 return PartialSums(parts)
         want_f32 = out_dtype == torch.float32
-        out = torch.empty((M, N), dtype=torch.float32 if want_f32 else torch.bfloat16, device=x.device)
-        _check(_load("gemm").cw_gemm_bf16_skinny(1 if want_f32 else 0, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, _stream()),
-               "gemm_bf16_skinny")
-        return out
+        if lib.cw_gemm_bf16_skinny_fast(1 if want_f32 else 0, M, N, K):
+            out = torch.empty((M, N), dtype=torch.float32 if want_f32 else torch.bfloat16, device=x.device)
+            _check(lib.cw_gemm_bf16_skinny(1 if want_f32 else 0, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, _stream()),
+                   "gemm_bf16_skinny")
+            return out
     y = torch.mm(x, weight.t()) if bias is None else torch.addmm(bias, x, weight.t())
     if out_dtype == torch.float32:
         out = torch.empty((M, N), dtype=torch.float32, device=x.device)
@@ -298,8 +300,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
     return y
 
 
-# above this many rows the library product is faster than the streaming kernel (measured)
+# up to this many rows every product goes through the weight-streaming kernels
 SKINNY_MAX_ROWS = 16
+# up to this many rows the shapes that the persistent streaming kernel takes do (the library
+# product is faster for the others, measured)
+STREAM_MAX_ROWS = 64
 
 
 @contextlib.contextmanager
@@ -362,7 +367,8 @@ def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor
     two_i = gate_up_weight.shape[0]
     _need(gate_up_weight.shape[1] == K and two_i % 2 == 0, "gate_up weight must be [2 I, K]")
     out = torch.empty((M, two_i // 2), dtype=x.dtype, device=x.device)
-    if x.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and K % 8 == 0:
+    if (x.dtype == torch.bfloat16 and M <= STREAM_MAX_ROWS and K % 8 == 0
+            and _load("gemm").cw_gemm_bf16_skinny_fast(2, M, two_i, K)):
         _need(gate_up_weight.dtype == torch.bfloat16, "a bfloat16 product needs bfloat16 operands")
         _check(_load("gemm").cw_gemm_bf16_skinny(2, _ptr(x), K, _ptr(gate_up_weight), _ptr(out), two_i // 2, M, two_i, K, _stream()),
                "gemm_bf16_skinny(swiglu)")

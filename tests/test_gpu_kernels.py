@@ -272,6 +272,42 @@ def test_skinny_bf16_product(M, N, K):
         assert torch.equal(ops.linear(other, w, out_dtype=torch.float32)[M - 1], got32[M - 1])
 
 
+@pytest.mark.parametrize("M", [3, 16, 17, 32, 40, 64])
+def test_streaming_product_many_row_tiles(M):
+    """Shapes that the persistent streaming kernel takes (many row tiles, a short K per wave),
+    with up to 64 rows of x: plain, float32, gated and partial-sum outputs. The sizes are no
+    multiples of the tiles."""
+    from clockwork_amd import ops
+
+    lib = ops._load("gemm")
+    N, K = 8192 + 40, 1536
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV) / K ** 0.5).to(torch.bfloat16)
+    assert lib.cw_gemm_bf16_skinny_fast(0, M, N, K) == 1
+    want = x.float() @ w.float().t()
+    got32 = ops.linear(x, w, out_dtype=torch.float32)
+    torch.testing.assert_close(got32, want, rtol=1e-4, atol=1e-4)
+    got = ops.linear(x, w)
+    assert got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float(), want, rtol=1e-2, atol=1e-2)
+    alone = ops.linear(x[M - 1 :].contiguous(), w, out_dtype=torch.float32)[0]
+    torch.testing.assert_close(alone, got32[M - 1], rtol=1e-5, atol=1e-5)
+    # gated: I no multiple of 8
+    I = 4100 + 4
+    wg = (torch.randn(2 * I, K, device=DEV) / K ** 0.5).to(torch.bfloat16)
+    assert lib.cw_gemm_bf16_skinny_fast(2, M, 2 * I, K) == 1
+    y = x.float() @ wg.float().t()
+    torch.testing.assert_close(ops.linear_swiglu(x, wg).float(), torch.nn.functional.silu(y[:, :I]) * y[:, I:],
+                               rtol=2e-2, atol=2e-2)
+    # partial sums over a long K: K no multiple of 32 * waves * splits
+    N2, K2 = 1536 + 8, 8960 + 8
+    x2 = torch.randn(M, K2, device=DEV).to(torch.bfloat16)
+    w2 = (torch.randn(N2, K2, device=DEV) / K2 ** 0.5).to(torch.bfloat16)
+    parts = ops.linear(x2, w2, partial_ok=True)
+    assert isinstance(parts, ops.PartialSums) and parts.parts.shape[0] == lib.cw_gemm_bf16_skinny_ksplits(M, N2, K2) > 1
+    torch.testing.assert_close(parts.parts.sum(0), x2.float() @ w2.float().t(), rtol=1e-4, atol=2e-4)
+
+
 @pytest.mark.parametrize("M", [1, 8, 20, 64, 100])
 @pytest.mark.parametrize("I,K", [(176, 64), (8960, 1536), (100, 80), (52, 200)])
 def test_fused_swiglu_product(M, I, K):
