@@ -783,6 +783,7 @@ struct PrefillTile {
   static constexpr int NT = 256 * NH;           // threads of a workgroup
   static constexpr int STAGE = KT * (KROW + VROW);  // elements of one stage: a K tile, then a V tile
   static constexpr size_t BYTES = 2 * STAGE * sizeof(bf16_t);
+  static constexpr int TABLE = 2048;  // block-table entries held in LDS at a time
 };
 
 template <int HD, bool POW2>
@@ -816,13 +817,16 @@ __global__ __launch_bounds__(PrefillTile<HD>::NT, (HD <= 128 ? 2 : 1)) void attn
   const int wg_last = pos0 + ntok - 1;
   const int wg_lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
   const int bs = p.block_size, sh = p.bs_shift;
-  // the pages of every key this workgroup may read -> LDS: no tile waits for a table entry
-  const int page0 = cw_page_index<POW2>(wg_lo, bs, sh);
-  {
-    const int* table = p.block_tables + (int64_t)req * p.table_stride;
-    const int n_pages = cw_page_index<POW2>(wg_last, bs, sh) - page0 + 1;
+  // the pages of the keys this workgroup reads -> LDS, a window of Tile::TABLE entries at a time
+  // (32k keys with pages of 16): no tile waits for a table entry from memory
+  const int* table = p.block_tables + (int64_t)req * p.table_stride;
+  const int page_last = cw_page_index<POW2>(wg_last, bs, sh);
+  int page0 = cw_page_index<POW2>(wg_lo, bs, sh);  // the page of tbl[0]
+  auto load_table = [&]() __attribute__((always_inline)) {
+    const int n_pages = min(page_last - page0 + 1, Tile::TABLE);
     for (int i = threadIdx.x; i < n_pages; i += NT) tbl[i] = table[page0 + i];
-  }
+  };
+  load_table();
   __syncthreads();
   const bf16_t* kc = (const bf16_t*)p.k_cache;
   const bf16_t* vc = (const bf16_t*)p.v_cache;
@@ -896,7 +900,16 @@ __global__ __launch_bounds__(PrefillTile<HD>::NT, (HD <= 128 ? 2 : 1)) void attn
   for (int t = t_first; t <= t_last; ++t) {
     const int kv0 = t * KT + half * KW;  // the wave's keys of this stage
     const int stage = (t - t_first) & 1;
-    if (t < t_last) fetch(t + 1);  // in flight while this tile is computed
+    if (t < t_last) {
+      // the next stage's pages must lie in the table window; nobody reads the window right now
+      const int need = cw_page_index<POW2>(min((t + 1) * KT + KT - 1, wg_last), bs, sh);
+      if (need >= page0 + Tile::TABLE) {
+        page0 = cw_page_index<POW2>(max((t + 1) * KT, wg_lo), bs, sh);
+        load_table();
+        __syncthreads();
+      }
+      fetch(t + 1);  // in flight while this tile is computed
+    }
     const bool active = wave_on && kv0 <= p_last && kv0 + KW - 1 >= lo;
     if (active) {
       const bf16_t* ks = tiles + stage * Tile::STAGE + half * KW * KROW;
@@ -1077,8 +1090,10 @@ CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* o
   p.part_o = nullptr; p.part_ml = nullptr; p.counters = nullptr; p.zeros = zeros;
   if ((int64_t)nkv * p.n_chunks > 65535) return CW_ERR_SIZE;
   dim3 grid(n_items, nkv * p.n_chunks), block(PrefillTile<CW_HD>::NT);
-  // two stages of a 32-key K and V tile, then a request's whole table
-  const size_t smem = PrefillTile<CW_HD>::BYTES + sizeof(int) * ((size_t)table_stride + 2);
+  // two stages of K and V tiles, then the window of the block table
+  const size_t entries = (size_t)table_stride < (size_t)PrefillTile<CW_HD>::TABLE ? table_stride : PrefillTile<CW_HD>::TABLE;
+  if ((PrefillTile<CW_HD>::KT + block_size - 1) / block_size + 1 > PrefillTile<CW_HD>::TABLE) return CW_ERR_SIZE;
+  const size_t smem = PrefillTile<CW_HD>::BYTES + sizeof(int) * entries;
   if (smem > 160 * 1024) return CW_ERR_SIZE;
   if (p.bs_shift >= 0) {
     static size_t raised = 0;

@@ -399,9 +399,9 @@ static bool plan_stream(int mode, int M, int N, int K, int k_splits, int* mt, in
   // tiles per workgroup: one workgroup on every compute unit (a second round of these large
   // workgroups costs more than it brings), each with the same share
   // (up to 16 rows the one-tile kernels are as fast below two rounds; beyond, the alternative
-  // is a library product that is slower as soon as half the compute units have a tile)
+  // is a library product that is slower as soon as every compute unit has a tile)
   const int slots = cw_num_compute_units();
-  if ((int64_t)*n_tiles * k_splits < (M <= 16 ? 2 * slots : slots / 2)) return false;
+  if ((int64_t)*n_tiles * k_splits < (M <= 16 ? 2 * slots : slots)) return false;
   const int per = (*n_tiles * k_splits + slots - 1) / slots;
   *grid = dim3((*n_tiles + per - 1) / per, k_splits);
   return true;

@@ -572,6 +572,31 @@ def test_prefill_attention_kernel(nh, nkv, hd, bs, window):
         at += q_len
 
 
+@pytest.mark.parametrize("window", [0, 700])
+def test_prefill_attention_kernel_long_block_table(window):
+    """More pages than the kernel holds of a block table at a time (pages of one key): the table
+    window moves on while the keys are walked."""
+    dtype = torch.bfloat16
+    nh, nkv, hd, bs = 4, 2, 64, 1
+    ctx, q_len = 2500, 200
+    table = torch.randperm(ctx + 5).tolist()[:ctx]
+    kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, ctx + 5, [table], [ctx], poison=float("nan"))
+    q = torch.randn(q_len, nh, hd, device=DEV).to(dtype)
+    # one far key that every query of head 0 looks at
+    ks[0][37, 0] *= 0  # keep the reference tensors in step with the cache
+    kc[table[37], 0] = 0
+    kc[table[37], 0, :8] = 4.0
+    ks[0][37, 0, :8] = 4.0
+    q[:, 0, :8] = 4.0
+    tables_dev = [list(table)]
+    if window:
+        for b in range(max(0, (ctx - q_len) - window + 1)):
+            tables_dev[0][b] = -1
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables_dev, [ctx], [q_len], kc, vc, [q], window=window, prefill_kernel=True)
+    want = plain.attention_dense(q.float().cpu(), ks[0].float().cpu(), vs[0].float().cpu(), hd ** -0.5, window=window or None)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+
+
 def ops_decode_ok(hd):
     from clockwork_amd import ops
 
