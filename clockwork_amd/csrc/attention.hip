@@ -41,6 +41,9 @@ struct AttnParams {
   float* part_ml;         // [n_items, nkv * n_chunks, n_splits, ROWS, 2] running max, sum
   int* counters;          // decode kernel: one arrival counter per (item, head chunk), zero between launches
   const void* zeros;      // at least HD zero elements: what a masked key or value row is loaded from
+  // decode kernel only
+  int identity;           // 1: item i is request i and its one token is row i of the batch (items, cu_q unread)
+  int split_keys;         // > 0: split s takes keys [s * split_keys, (s + 1) * split_keys), a multiple of 32
 };
 
 // page of a position and the offset inside it; POW2: the page size is a power of two (shift given)
@@ -443,27 +446,45 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnParams p) {
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / p.n_chunks, chunk = blockIdx.y % p.n_chunks;
   const int split = blockIdx.z;
-  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1];
+  // Every trip to memory that depends on an earlier one costs about a microsecond, which is what
+  // a short context takes in all: with ``identity`` and fixed key ranges per split, the context
+  // length, the table entries and the query are fetched side by side, then keys and values.
+  const bool ident = p.identity != 0;
+  const int req = ident ? item : p.items[4 * item];
+  const int tok0 = ident ? 0 : p.items[4 * item + 1];
   const int ctx = p.ctx_lens[req];
-  const int q_begin = p.cu_q[req];
-  const int qlen = p.cu_q[req + 1] - q_begin;
+  const int q_begin = ident ? item : p.cu_q[req];
+  const int qlen = ident ? 1 : p.cu_q[req + 1] - q_begin;
   const int group = p.nh / p.nkv;
   const int gh = p.gh;
-  const int pos = ctx - qlen + tok0;
-  const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
-  const int tile0 = lo / 32;
-  const int n_tiles = pos / 32 + 1 - tile0;
-  const int tps = (n_tiles + p.n_splits - 1) / p.n_splits;
-  const int t_begin = tile0 + split * tps;
-  const int t_end = min(tile0 + n_tiles, t_begin + tps);
   const bf16_t* kc = (const bf16_t*)p.k_cache;
   const bf16_t* vc = (const bf16_t*)p.v_cache;
   const bf16_t* zrow = (const bf16_t*)p.zeros;
   const int bs = p.block_size, sh = p.bs_shift;
-  // the pages of this split's keys -> LDS, so that no tile waits for a table entry from memory
-  const int page0 = cw_page_index<POW2>(t_begin * 32, bs, sh);
-  {
-    const int* table = p.block_tables + (int64_t)req * p.table_stride;
+  const int* table = p.block_tables + (int64_t)req * p.table_stride;
+  int page0 = 0;
+  if (p.split_keys > 0) {
+    // the pages of this split's key range -> LDS, whatever the context length turns out to be
+    const int k_first = split * p.split_keys;
+    const int k_last = min(k_first + p.split_keys, p.table_stride * bs) - 1;
+    page0 = cw_page_index<POW2>(k_first, bs, sh);
+    const int n_pages = k_last >= k_first ? cw_page_index<POW2>(k_last, bs, sh) - page0 + 1 : 0;
+    for (int i = threadIdx.x; i < n_pages; i += 256) tbl[i] = table[page0 + i];
+  }
+  const int pos = ctx - qlen + tok0;
+  const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int tile0 = lo / 32;
+  const int n_tiles = pos / 32 + 1 - tile0;
+  int t_begin, t_end;
+  if (p.split_keys > 0) {
+    t_begin = max(tile0, split * (p.split_keys / 32));
+    t_end = min(tile0 + n_tiles, (split + 1) * (p.split_keys / 32));
+  } else {
+    const int tps = (n_tiles + p.n_splits - 1) / p.n_splits;
+    t_begin = tile0 + split * tps;
+    t_end = min(tile0 + n_tiles, t_begin + tps);
+    // the pages of this split's keys -> LDS, so that no tile waits for a table entry from memory
+    page0 = cw_page_index<POW2>(t_begin * 32, bs, sh);
     const int last_key = min(pos, t_end * 32 - 1);
     const int n_pages = t_end > t_begin ? cw_page_index<POW2>(last_key, bs, sh) - page0 + 1 : 0;
     for (int i = threadIdx.x; i < n_pages; i += 256) tbl[i] = table[page0 + i];
@@ -578,6 +599,8 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnParams p) {
       for (int j = 0; j < NF; ++j) { kf[kb][j] = kf_n[kb][j]; vf[kb][j] = vf_n[kb][j]; }
   }
 
+  // a context beyond the fixed key ranges (the caller promised there is none) must not pass for a result
+  if (p.split_keys > 0 && pos >= p.n_splits * p.split_keys) l_run = NAN;
   // ---- merge the waves: o_s[wave][head c][d], lane (c, s) holds d = db * 16 + 4s .. + 3
   if (s == 0) { M_s[wave][c] = m_run; L_s[wave][c] = l_run; }
 #pragma unroll
@@ -626,8 +649,9 @@ __global__ void attn_decode_merge_kernel(AttnParams p) {
   const int group = p.nh / p.nkv;
   const int hg = chunk * gh + g;
   if (hg >= group) return;
-  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1];
-  const int q_begin = p.cu_q[req];
+  const bool ident = p.identity != 0;
+  const int tok0 = ident ? 0 : p.items[4 * item + 1];
+  const int q_begin = ident ? item : p.cu_q[p.items[4 * item]];
   const int64_t base = ((int64_t)item * (p.nkv * p.n_chunks) + y) * p.n_splits;
   for (int sp = threadIdx.x; sp < p.n_splits; sp += blockDim.x) {
     const float2 ml = *reinterpret_cast<const float2*>(&p.part_ml[((base + sp) * gh + g) * 2]);
@@ -684,7 +708,7 @@ static int launch_decode(AttnParams& p, int n_items, hipStream_t stream) {
   constexpr int HD = CW_HD;
   // keys of a split: at most ceil(tiles / splits) tiles of 32; their pages go to LDS
   const int64_t max_tiles = ((int64_t)p.table_stride * p.block_size + 31) / 32;
-  const int64_t tiles_per_split = (max_tiles + p.n_splits - 1) / p.n_splits;
+  const int64_t tiles_per_split = p.split_keys > 0 ? p.split_keys / 32 : (max_tiles + p.n_splits - 1) / p.n_splits;
   const int64_t pages = (tiles_per_split * 32 + p.block_size - 1) / p.block_size + 2;
   const size_t smem = sizeof(float) * DEC_WAVES * 16 * HD + sizeof(int) * (size_t)pages;
   if (smem > 160 * 1024) return CW_ERR_SIZE;
@@ -707,12 +731,17 @@ static int launch_decode(AttnParams& p, int n_items, hipStream_t stream) {
 
 // Single-token items (every item: one token), bfloat16. Same arguments as cw_attention;
 // ``zeros``: at least CW_HD zero elements (16-byte aligned) that masked rows are read from.
+// ``identity``: item i is request i and its token is row i (a batch of single tokens only): items
+// and cu_q are not read. ``split_keys`` > 0 (a multiple of 32): split s takes keys
+// [s * split_keys, (s + 1) * split_keys) instead of a share of each request's own length, and
+// ``max_ctx``, the longest context among the requests, must not exceed n_splits * split_keys.
 CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride,
                                        const void* k_cache, const void* v_cache, const int* block_tables,
                                        int table_stride, const int* ctx_lens, const int* cu_q,
                                        const int* items, int n_items, int nh, int nkv, int block_size,
                                        int n_splits, int window, float scale, float* workspace,
-                                       int64_t workspace_floats, const void* zeros, hipStream_t stream) {
+                                       int64_t workspace_floats, const void* zeros, int identity,
+                                       int split_keys, int max_ctx, hipStream_t stream) {
 #if CW_HAS_DECODE
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || block_size <= 0 || table_stride <= 0)
     return CW_ERR_ARG;
@@ -720,6 +749,9 @@ CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* ou
   if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || (q_stride & 7))
     return CW_ERR_ARG;
   if (zeros == nullptr || ((uintptr_t)zeros & 15)) return CW_ERR_ARG;
+  // fixed key ranges must cover the longest context the caller will run
+  if (split_keys < 0 || (split_keys & 31) || max_ctx < 0) return CW_ERR_ARG;
+  if (split_keys > 0 && (int64_t)split_keys * n_splits < max_ctx) return CW_ERR_ARG;
   if (n_items == 0) return CW_OK;
   const int group = nh / nkv;
   AttnParams p;
@@ -727,6 +759,7 @@ CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* ou
   p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
   p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
   p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.bs_shift = cw_log2_or_minus1(block_size);
+  p.identity = identity ? 1 : 0; p.split_keys = split_keys;
   p.gh = cw_attention_decode_gh(group);
   p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = n_splits; p.window = window; p.scale = scale;
   if ((int64_t)nkv * p.n_chunks * p.gh > 65535) return CW_ERR_SIZE;

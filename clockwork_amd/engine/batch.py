@@ -43,6 +43,9 @@ class AttentionPlan:
     chunks_single: int = 1
     single_splits: int = 1
     decode_splits: int = 1   # splits of the bfloat16 decode kernel (finer: it walks 16-key tiles)
+    decode_split_keys: int = 0    # keys of each of those splits, at fixed places (a multiple of 32)
+    decode_max_ctx: int = 0       # the longest context the fixed places were planned for
+    single_identity: bool = False  # a batch of single tokens only: item i is request i, token row i
 
 
 class _Packer:
@@ -139,6 +142,11 @@ class StepContext:
             # unit are enough to keep memory busy
             base = plan.n_single * nkv * -(-group // min(group, 16))
             plan.decode_splits = max(1, min(-(-2 * self.num_compute_units // base), longest_single // 128, 64))
+            # fixed places for the splits: a workgroup then knows its pages before it knows the
+            # request's length, which saves it a trip to memory
+            plan.decode_split_keys = 32 * -(-(-(-longest_single // plan.decode_splits)) // 32)
+            plan.decode_max_ctx = longest_single
+            plan.single_identity = plan.n_single == len(self.h_q_lens)
         packer = _Packer()
         packer.add(wide)
         packer.add(single)

@@ -107,7 +107,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_attention_decode_supported": [],
             "cw_attention_decode_gh": [I],
             "cw_attention_decode_workspace_floats": [I, I, I, I],
-            "cw_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, P, P],
+            "cw_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, P, I, I, I, P],
         },
     }[name]
     for fn, argtypes in sigs.items():
@@ -424,9 +424,12 @@ def decode_attention_workspace_floats(hd: int, n_items: int, nh: int, nkv: int, 
 
 def attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
                      nh: int, nkv: int, hd: int, block_size: int, n_splits: int, window: int, scale: float,
-                     n_tokens: int, n_requests: int, workspace=None) -> None:
+                     n_tokens: int, n_requests: int, workspace=None, identity: bool = False,
+                     split_keys: int = 0, max_ctx: int = 0) -> None:
     """Single-token items through the bfloat16 decode kernel; arguments as for ``attention``.
-    With more than one split it needs a float32 ``workspace``."""
+    With more than one split it needs a float32 ``workspace``. ``identity``: item i is request i
+    with its token in row i (no other items). ``split_keys`` > 0: every split takes that many
+    keys at a fixed place; no context may then be longer than ``max_ctx`` <= n_splits * split_keys."""
     _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, workspace)
     _need(q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16, "the decode kernel is bfloat16")
     _need(out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd, "attention output must be [T, nh * hd]")
@@ -436,6 +439,10 @@ def attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_
     _i32(cu_q, n_requests + 1, "cu_q")
     _need(items.dtype == torch.int32 and items.numel() >= 4 * n_items, "items must be int32 [n_items, 4]")
     _need(tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape, "cache must be [..., nkv, hd]")
+    if identity:
+        _need(n_items == n_requests == n_tokens, "identity items: one single-token item per request, nothing else")
+    if split_keys:
+        _need(split_keys % 32 == 0 and split_keys * n_splits >= max_ctx > 0, "fixed key ranges do not cover the longest context")
     lib = _load("attention", hd)
     need = lib.cw_attention_decode_workspace_floats(n_items, nh, nkv, n_splits)
     ws_floats = 0
@@ -447,7 +454,8 @@ def attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_
         lib.cw_attention_decode_bf16(
             q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
             block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, nh, nkv, block_size, n_splits,
-            window, float(scale), _ptr(workspace), ws_floats, _zero_row(out.device), _stream()),
+            window, float(scale), _ptr(workspace), ws_floats, _zero_row(out.device), int(bool(identity)),
+            int(split_keys), int(max_ctx), _stream()),
         "attention_decode_bf16",
     )
 

@@ -88,7 +88,8 @@ class PagedAttention(Part):
                 need = ops.decode_attention_workspace_floats(hd, plan.n_single, nh, nkv, plan.decode_splits)
                 workspace = torch.empty(need, dtype=torch.float32, device=x.device)
             ops.attention_decode(items=plan.single_items, n_items=plan.n_single, n_splits=plan.decode_splits,
-                                 workspace=workspace, **common)
+                                 workspace=workspace, identity=plan.single_identity,
+                                 split_keys=plan.decode_split_keys, max_ctx=plan.decode_max_ctx, **common)
         elif plan.n_single:
             workspace = None
             if plan.single_splits > 1:

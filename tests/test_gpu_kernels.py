@@ -376,7 +376,7 @@ def _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens, poison=100.0)
 
 
 def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs, window=0, splits=None, scale=None,
-                   decode_kernel=False, prefill_kernel=False):
+                   decode_kernel=False, prefill_kernel=False, fixed_ranges=False):
     from clockwork_amd import ops
     from clockwork_amd.engine.batch import StepContext
 
@@ -414,7 +414,12 @@ def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs,
         if n_splits > 1:
             ws = torch.full((ops.decode_attention_workspace_floats(hd, plan.n_single, nh, nkv, n_splits),), float("nan"),
                             dtype=torch.float32, device=DEV)
-        ops.attention_decode(items=plan.single_items, n_items=plan.n_single, n_splits=n_splits, workspace=ws, **common)
+        extra = {}
+        if fixed_ranges:  # every split at a fixed place; a batch of single tokens needs no items
+            longest = max(c for c, q in zip(ctx_lens, q_lens) if q == 1)
+            extra = dict(identity=plan.single_identity, split_keys=32 * -(-(-(-longest // n_splits)) // 32), max_ctx=longest)
+        ops.attention_decode(items=plan.single_items, n_items=plan.n_single, n_splits=n_splits, workspace=ws, **common,
+                             **extra)
     elif plan.n_single:
         ws = None
         if plan.single_splits > 1:
@@ -519,7 +524,8 @@ DECODE_KERNEL_CASES = [
 
 @pytest.mark.parametrize("nh,nkv,hd,bs,ctx_lens", DECODE_KERNEL_CASES)
 @pytest.mark.parametrize("splits", [1, 2, 7])
-def test_decode_attention_kernel(nh, nkv, hd, bs, ctx_lens, splits):
+@pytest.mark.parametrize("fixed_ranges", [False, True])
+def test_decode_attention_kernel(nh, nkv, hd, bs, ctx_lens, splits, fixed_ranges):
     dtype = torch.bfloat16
     num_blocks = sum(-(-c // bs) for c in ctx_lens) + 5
     perm = torch.randperm(num_blocks).tolist()
@@ -531,7 +537,7 @@ def test_decode_attention_kernel(nh, nkv, hd, bs, ctx_lens, splits):
     kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens, poison=float("nan"))
     qs = [torch.randn(1, nh, hd, device=DEV).to(dtype) for _ in ctx_lens]
     out = _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, [1] * len(ctx_lens), kc, vc, qs, splits=splits,
-                         decode_kernel=True)
+                         decode_kernel=True, fixed_ranges=fixed_ranges)
     assert not torch.isnan(out.float()).any()
     for r in range(len(ctx_lens)):
         want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5)
@@ -617,7 +623,8 @@ def test_prefill_attention_kernel_sharp_scores():
 
 
 @pytest.mark.parametrize("window", [1, 5, 16, 40])
-def test_decode_attention_kernel_window_and_mixed_batch(window):
+@pytest.mark.parametrize("fixed_ranges", [False, True])
+def test_decode_attention_kernel_window_and_mixed_batch(window, fixed_ranges):
     """Single tokens beside a portion in one batch; pages behind the window are gone (-1)."""
     dtype = torch.bfloat16
     nh, nkv, hd, bs = 4, 2, 32, 8
@@ -629,7 +636,8 @@ def test_decode_attention_kernel_window_and_mixed_batch(window):
         for b in range(max(0, (c - q) - window + 1) // bs):
             tables_dev[r][b] = -1
     qs = [torch.randn(q, nh, hd, device=DEV).to(dtype) for q in q_lens]
-    out = _run_attention(dtype, nh, nkv, hd, bs, tables_dev, ctx_lens, q_lens, kc, vc, qs, window=window, decode_kernel=True)
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables_dev, ctx_lens, q_lens, kc, vc, qs, window=window, decode_kernel=True,
+                         splits=2 if fixed_ranges else None, fixed_ranges=fixed_ranges)
     at = 0
     for r, q_len in enumerate(q_lens):
         want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5, window=window)
@@ -646,7 +654,8 @@ def test_decode_attention_far_key_stands_out():
         q = torch.randn(1, nh, hd, device=DEV).to(torch.bfloat16)
         slot = tables[0][where // bs] * bs + where % bs
         kc[slot, 1] = (60.0 * q[0, 7].float() / q[0, 7].float().norm()).to(torch.bfloat16)
-        out = _run_attention(torch.bfloat16, nh, nkv, hd, bs, tables, [ctx], [1], kc, vc, [q], splits=3, decode_kernel=True)
+        out = _run_attention(torch.bfloat16, nh, nkv, hd, bs, tables, [ctx], [1], kc, vc, [q], splits=3, decode_kernel=True,
+                             fixed_ranges=where % 2 == 1)
         torch.testing.assert_close(out[0, 7].float(), vc[slot, 1].float(), rtol=2e-2, atol=2e-2)
 
 
