@@ -47,20 +47,23 @@ __device__ __forceinline__ float delta_at(const DT* dl, int64_t part_stride, int
 }
 
 template <typename T, typename WT, typename DT>
-__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const DT* __restrict__ delta, int parts,
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta0,
+                                   const DT* __restrict__ delta, int parts,
                                    int64_t part_stride, const WT* __restrict__ weight, float eps,
                                    T* __restrict__ out, const int* __restrict__ rows, int H) {
   __shared__ float partial[4];
   const int i = blockIdx.x;
   const int t = rows ? rows[i] : i;
   float* x = resid + (int64_t)t * H;
+  const T* d0 = delta0 ? delta0 + (int64_t)t * H : nullptr;
   const DT* dl = delta ? delta + (int64_t)t * H : nullptr;
   T* o = out + (int64_t)i * H;
-  const bool write_back = rows == nullptr && dl != nullptr;
+  const bool write_back = rows == nullptr && (dl != nullptr || d0 != nullptr);
 
   float ss = 0.0f;
   for (int j = threadIdx.x; j < H; j += 256) {
     float v = x[j];
+    if (d0) v += cw_to_float(d0[j]);
     if (dl) v += delta_at(dl, part_stride, parts, j);
     if (write_back) x[j] = v;
     ss += v * v;
@@ -73,6 +76,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const DT* __restri
   const float inv = 1.0f / sqrtf(total / (float)H + eps);
   for (int j = threadIdx.x; j < H; j += 256) {
     float v = x[j];
+    if (d0 && !write_back) v += cw_to_float(d0[j]);
     if (dl && !write_back) v += delta_at(dl, part_stride, parts, j);
     const T n = cw_from_float<T>(v * inv);
     o[j] = cw_from_float<T>(cw_to_float(weight[j]) * cw_to_float(n));
@@ -107,7 +111,8 @@ template <> struct Chunk4<bf16_t> {
 };
 
 template <typename T, typename WT, typename DT>
-__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const DT* __restrict__ delta,
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta0,
+                                                              const DT* __restrict__ delta,
                                                               int parts, int64_t part_stride,
                                                               const WT* __restrict__ weight, float eps,
                                                               T* __restrict__ out, const int* __restrict__ rows, int H) {
@@ -115,9 +120,10 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   const int i = blockIdx.x;
   const int t = rows ? rows[i] : i;
   float* x = resid + (int64_t)t * H;
+  const T* d0 = delta0 ? delta0 + (int64_t)t * H : nullptr;
   const DT* dl = delta ? delta + (int64_t)t * H : nullptr;
   T* o = out + (int64_t)i * H;
-  const bool write_back = rows == nullptr && dl != nullptr;
+  const bool write_back = rows == nullptr && (dl != nullptr || d0 != nullptr);
   const int n_chunks = H / 4;
   float v[4][4], w[4][4];
 #pragma unroll
@@ -128,6 +134,18 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
       Chunk4<WT>::load(weight + ch * 4, w[k]);
     } else {
       v[k][0] = v[k][1] = v[k][2] = v[k][3] = 0.0f;
+    }
+  }
+  if (d0) {  // an earlier branch's output that was not added yet: it comes first, as it would have
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int ch = threadIdx.x + k * 256;
+      if (ch < n_chunks) {
+        float d[4];
+        Chunk4<T>::load(d0 + ch * 4, d);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[k][e] += d[e];
+      }
     }
   }
   if (dl) {
@@ -178,24 +196,27 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
 }
 
 // delta: nullptr, or [T, H] in the activation type (delta_parts == 0), or float32 [delta_parts, T, H].
-CW_EXPORT int cw_add_rmsnorm(float* resid, const void* delta, int delta_parts, int T_rows,
+// delta0: nullptr, or [T, H] in the activation type, added to the residual before delta.
+CW_EXPORT int cw_add_rmsnorm(float* resid, const void* delta0, const void* delta, int delta_parts, int T_rows,
                              const void* weight, int w_dtype, float eps, void* out, int dtype,
                              const int* rows, int n, int H, hipStream_t stream) {
   if (n < 0 || H <= 0 || delta_parts < 0 || delta_parts > 64) return CW_ERR_ARG;
   if (n == 0) return CW_OK;
   dim3 grid(n), block(256);
   const bool vec = (H % 4 == 0) && H <= 4096 && !((uintptr_t)resid & 15) && !((uintptr_t)out & 15) &&
-                   !((uintptr_t)weight & 15) && !((uintptr_t)delta & 15);
+                   !((uintptr_t)weight & 15) && !((uintptr_t)delta & 15) && !((uintptr_t)delta0 & 15);
   const int parts = delta_parts > 0 ? delta_parts : 1;
   const int64_t part_stride = (int64_t)T_rows * H;
 #define CW_LAUNCH(T, WT, DT)                                                                           \
   do {                                                                                                 \
     if (vec)                                                                                           \
       hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, WT, DT>), grid, block, 0, stream, resid,           \
-                         (const DT*)delta, parts, part_stride, (const WT*)weight, eps, (T*)out, rows, H); \
+                         (const T*)delta0, (const DT*)delta, parts, part_stride, (const WT*)weight, eps, \
+                         (T*)out, rows, H);                                                            \
     else                                                                                               \
       hipLaunchKernelGGL((add_rmsnorm_kernel<T, WT, DT>), grid, block, 0, stream, resid,               \
-                         (const DT*)delta, parts, part_stride, (const WT*)weight, eps, (T*)out, rows, H); \
+                         (const T*)delta0, (const DT*)delta, parts, part_stride, (const WT*)weight, eps, \
+                         (T*)out, rows, H);                                                            \
   } while (0)
   if (delta_parts > 0) {
     if (dtype == CW_F32 && w_dtype == CW_F32) CW_LAUNCH(float, float, float);

@@ -241,30 +241,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
 // stored, which lets the compiler wait for exactly the loads a product needs. Wave w of k-split
 // blockIdx.y owns k-steps [(blockIdx.y * WAVES + w) * SPW, + SPW). Modes and layouts as in
 // gemm_skinny_bf16_kernel.
-template <int MODE, int WAVES, int SPW, int MT>
+// NORM (MT = 1, no k-split): x is not read but made here, x = rmsnorm(resid + delta) * weight over
+// the K elements of a row, with the rounding steps of the stand-alone norm kernel; every
+// workgroup does so for itself (the rows are few and come from L2), nothing is written back.
+struct StreamNormIn {
+  const float* resid;    // [M, K] float32
+  const bf16_t* delta;   // [M, K] bfloat16
+  const void* weight;    // [K] bfloat16 or float32
+  int weight_f32;
+  float eps;
+};
+
+template <int MODE, int WAVES, int SPW, int MT, bool NORM = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16_t* __restrict__ X, int64_t ldx,
                                                                const bf16_t* __restrict__ W,
                                                                void* __restrict__ C, int64_t ldc,
-                                                               int M, int N, int K, int n_tiles) {
+                                                               int M, int N, int K, int n_tiles, StreamNormIn nin) {
   constexpr int NBUF = MT <= 2 ? 2 : 1;
   __shared__ float red[NBUF][WAVES][MT * 256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, s = lane >> 4;
   const int I = N / 2;  // MODE 2 only
 
-  bf16x8_t xf[SPW][MT];
-  int koff[SPW];
+  int koff[SPW];  // the lane's 8 k-values of each step; a step outside K reads k = 0 and meets zeros in x
 #pragma unroll
   for (int u = 0; u < SPW; ++u) {
     const int k = ((blockIdx.y * WAVES + wave) * SPW + u) * 32 + s * 8;
-    const bool kok = k + 8 <= K;
-    koff[u] = kok ? k : 0;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) xf[u][mt][e] = (__bf16)0.0f;
-      if (kok && mt * 16 + r < M) xf[u][mt] = *reinterpret_cast<const bf16x8_t*>(X + (int64_t)(mt * 16 + r) * ldx + k);
-    }
+    koff[u] = k + 8 <= K ? k : 0;
   }
   auto wrow = [&](int tile) __attribute__((always_inline)) -> const bf16_t* {
     int64_t n;
@@ -276,13 +279,72 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
     }
     return W + n * K;
   };
-
+  // the first tile's weights are requested before anything else: x, and with NORM the norm's
+  // statistics, are fetched in their shadow
   int tile = blockIdx.x;
   bf16x8_t cur[SPW], nxt[SPW];
   {
     const bf16_t* w = wrow(tile);
 #pragma unroll
     for (int u = 0; u < SPW; ++u) cur[u] = *reinterpret_cast<const bf16x8_t*>(w + koff[u]);
+  }
+
+  bf16x8_t xf[SPW][MT];
+  if constexpr (NORM) {
+    static_assert(MT == 1, "the fused norm serves one tile of tokens");
+    __shared__ float ssq[WAVES][16];
+    float v[SPW][8], wv[SPW][8];
+    float ss = 0.0f;
+#pragma unroll
+    for (int u = 0; u < SPW; ++u) {
+      const int k = (wave * SPW + u) * 32 + s * 8;
+      const bool kok = k + 8 <= K;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[u][e] = wv[u][e] = 0.0f;
+      if (kok && r < M) {
+        const float4 a = *reinterpret_cast<const float4*>(nin.resid + (int64_t)r * K + k);
+        const float4 b = *reinterpret_cast<const float4*>(nin.resid + (int64_t)r * K + k + 4);
+        const bf16x8_t d = *reinterpret_cast<const bf16x8_t*>(nin.delta + (int64_t)r * K + k);
+        v[u][0] = a.x + (float)d[0]; v[u][1] = a.y + (float)d[1]; v[u][2] = a.z + (float)d[2]; v[u][3] = a.w + (float)d[3];
+        v[u][4] = b.x + (float)d[4]; v[u][5] = b.y + (float)d[5]; v[u][6] = b.z + (float)d[6]; v[u][7] = b.w + (float)d[7];
+        if (nin.weight_f32) {
+          const float4 w0 = *reinterpret_cast<const float4*>((const float*)nin.weight + k);
+          const float4 w1 = *reinterpret_cast<const float4*>((const float*)nin.weight + k + 4);
+          wv[u][0] = w0.x; wv[u][1] = w0.y; wv[u][2] = w0.z; wv[u][3] = w0.w;
+          wv[u][4] = w1.x; wv[u][5] = w1.y; wv[u][6] = w1.z; wv[u][7] = w1.w;
+        } else {
+          const bf16x8_t w8 = *reinterpret_cast<const bf16x8_t*>((const bf16_t*)nin.weight + k);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) wv[u][e] = (float)w8[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += v[u][e] * v[u][e];
+      }
+    }
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    if (s == 0) ssq[wave][r] = ss;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) total += ssq[w][r];
+    const float inv = 1.0f / sqrtf(total / (float)K + nin.eps);
+#pragma unroll
+    for (int u = 0; u < SPW; ++u)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xf[u][0][e] = (__bf16)(wv[u][e] * (float)(__bf16)(v[u][e] * inv));
+  } else {
+#pragma unroll
+    for (int u = 0; u < SPW; ++u) {
+      const int k = ((blockIdx.y * WAVES + wave) * SPW + u) * 32 + s * 8;
+      const bool kok = k + 8 <= K;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xf[u][mt][e] = (__bf16)0.0f;
+        if (kok && mt * 16 + r < M) xf[u][mt] = *reinterpret_cast<const bf16x8_t*>(X + (int64_t)(mt * 16 + r) * ldx + k);
+      }
+    }
   }
   int buf = 0;
   for (; tile < n_tiles; tile += gridDim.x) {
@@ -360,7 +422,7 @@ static int launch_stream_one(dim3 grid, const bf16_t* X, int64_t ldx, const bf16
                              int M, int N, int K, int n_tiles, hipStream_t stream) {
   if constexpr (cw_stream_fits(WAVES, SPW, MT)) {
     hipLaunchKernelGGL((gemm_stream_bf16_kernel<MODE, WAVES, SPW, MT>), grid, dim3(WAVES * 64), 0, stream, X, ldx,
-                       W, C, ldc, M, N, K, n_tiles);
+                       W, C, ldc, M, N, K, n_tiles, StreamNormIn{});
     return cw_launch_status();
   } else {
     return CW_ERR_SIZE;
@@ -462,6 +524,42 @@ CW_EXPORT int cw_gemm_bf16_skinny_fast(int mode, int M, int N, int K) {
   int mt, spw, n_tiles;
   dim3 grid;
   return plan_stream(mode, M, N, K, 1, &mt, &spw, &grid, &n_tiles) ? 1 : 0;
+}
+
+// 1 if cw_gemm_bf16_swiglu_normed takes this shape (the streaming kernel with one tile of tokens).
+CW_EXPORT int cw_gemm_bf16_swiglu_normed_ok(int M, int N, int K) {
+  int mt, spw, n_tiles;
+  dim3 grid;
+  return M >= 1 && M <= 16 && !(N & 1) && !(K & 7) && plan_stream(2, M, N, K, 1, &mt, &spw, &grid, &n_tiles) ? 1 : 0;
+}
+
+// y[m, i] = silu(gate_i . x_m) * (up_i . x_m) with x = rmsnorm(resid + delta) * norm_weight made
+// inside the product kernel: resid float32 [M, K], delta bfloat16 [M, K], norm_weight [K]
+// bfloat16 (norm_weight_f32 = 0) or float32, W [N = 2 I, K] with the gate rows first, y bfloat16
+// [M, I] with row stride ldc. resid is not changed: whoever adds delta to it must still do so.
+CW_EXPORT int cw_gemm_bf16_swiglu_normed(const float* resid, const void* delta, const void* norm_weight,
+                                         int norm_weight_f32, float eps, const void* W, void* C, int64_t ldc,
+                                         int M, int N, int K, hipStream_t stream) {
+  if (!cw_gemm_bf16_swiglu_normed_ok(M, N, K)) return CW_ERR_SIZE;
+  if (!resid || !delta || !norm_weight || !W || !C || ldc < N / 2) return CW_ERR_ARG;
+  if (((uintptr_t)resid & 15) || ((uintptr_t)delta & 15) || ((uintptr_t)norm_weight & 15) || ((uintptr_t)W & 15))
+    return CW_ERR_ARG;
+  int mt, spw, n_tiles;
+  dim3 grid;
+  plan_stream(2, M, N, K, 1, &mt, &spw, &grid, &n_tiles);
+  const StreamNormIn nin{resid, (const bf16_t*)delta, norm_weight, norm_weight_f32, eps};
+#define CW_NORMED(SPW_)                                                                                        \
+  case SPW_:                                                                                                   \
+    if constexpr (cw_stream_fits(16, SPW_, 1))                                                                 \
+      hipLaunchKernelGGL((gemm_stream_bf16_kernel<2, 16, SPW_, 1, true>), grid, dim3(16 * 64), 0, stream,      \
+                         (const bf16_t*)nullptr, (int64_t)K, (const bf16_t*)W, C, ldc, M, N, K, n_tiles, nin); \
+    break
+  switch (spw) {
+    CW_NORMED(1); CW_NORMED(2); CW_NORMED(3); CW_NORMED(4); CW_NORMED(5); CW_NORMED(6); CW_NORMED(7); CW_NORMED(8);
+    default: return CW_ERR_SIZE;
+  }
+#undef CW_NORMED
+  return cw_launch_status();
 }
 
 // y = x W^T for M <= 64 rows of bfloat16 x [M, K] (row stride ldx) and bfloat16 W [N, K].

@@ -80,7 +80,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
     sigs = {
         "core": {
             "cw_embedding": [P, I, P, P, I, I, I, P],
-            "cw_add_rmsnorm": [P, P, I, I, P, I, F, P, I, P, I, I, P],
+            "cw_add_rmsnorm": [P, P, P, I, I, P, I, F, P, I, P, I, I, P],
             "cw_rope_kv_write": [P, I, P, I, P, P, P, I, I, I, I, I, P, P, L, P],
             "cw_silu_mul": [P, P, I, I, I, P],
             "cw_copy_pages": [P, I, L, L, P, I, P],
@@ -91,6 +91,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_gemm_bf16_skinny": [I, P, L, P, P, L, I, I, I, P],
             "cw_gemm_bf16_skinny_ksplits": [I, I, I],
             "cw_gemm_bf16_skinny_fast": [I, I, I, I],
+            "cw_gemm_bf16_swiglu_normed_ok": [I, I, I],
+            "cw_gemm_bf16_swiglu_normed": [P, P, P, I, F, P, P, L, I, I, I, P],
             "cw_gemm_qkv_rope_bf16": [P, L, P, P, I, P, P, P, P, P, P, L, I, I, I, I, I, P],
         },
         "sampling": {
@@ -177,17 +179,68 @@ class PartialSums:
         return total if dtype is None else total.to(dtype)
 
 
-def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None) -> torch.Tensor:
+_row_indices: dict = {}
+
+
+def _all_rows(n: int, device) -> torch.Tensor:
+    """int32 [0, n) on ``device`` (kept: a HIP graph may hold its address)."""
+    t = _row_indices.get((n, device))
+    if t is None:
+        t = _row_indices[(n, device)] = torch.arange(n, dtype=torch.int32, device=device)
+    return t
+
+
+class PendingPair:
+    """Two branch outputs that are both still to be added to the residual stream, ``first``
+    before ``second``: what a block hands on when its second norm ran inside the feed-forward's
+    product kernel (which writes no residual). ``first`` is a tensor in the activation type,
+    ``second`` a tensor or :class:`PartialSums`."""
+
+    __slots__ = ("first", "second")
+
+    def __init__(self, first, second) -> None:
+        self.first = first
+        self.second = second
+
+
+class LazyAddNorm:
+    """rmsnorm(resid + delta) * weight, not computed yet: a consumer that can make it inside its
+    own kernel takes the pieces, any other calls :meth:`value`. The residual is not updated
+    either way: ``delta`` stays pending."""
+
+    __slots__ = ("resid", "delta", "weight", "eps", "dtype")
+
+    def __init__(self, resid, delta, weight, eps: float, dtype) -> None:
+        self.resid, self.delta, self.weight, self.eps, self.dtype = resid, delta, weight, eps, dtype
+
+    @property
+    def shape(self):
+        return self.resid.shape
+
+    def value(self) -> torch.Tensor:
+        out = torch.empty(tuple(self.resid.shape), dtype=self.dtype, device=self.resid.device)
+        return add_rmsnorm(self.resid, self.delta, self.weight, self.eps, out, write_back=False)
+
+
+def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_back: bool = True) -> torch.Tensor:
     """resid += delta (when given), out = rmsnorm(resid) * weight; with ``rows`` only those rows
-    are normed into out[i] and resid is left alone. resid float32 [T, H]; delta/out in the
-    activation type, or delta a :class:`PartialSums` of that shape."""
+    are normed into out[i] and resid is left alone, as it is with ``write_back`` off. resid
+    float32 [T, H]; delta/out in the activation type, or delta a :class:`PartialSums` of that
+    shape, or a :class:`PendingPair` (both are added, ``first`` first)."""
+    delta0 = None
+    if isinstance(delta, PendingPair):
+        delta0, delta = delta.first, delta.second
+    if not write_back and rows is None:
+        rows = _all_rows(resid.shape[0], resid.device)
     parts = 0
     if isinstance(delta, PartialSums):
         parts = delta.parts.shape[0]
         delta = delta.parts
-    _gpu(resid, delta, weight, out, rows)
+    _gpu(resid, delta, delta0, weight, out, rows)
     T, H = resid.shape
     _need(resid.dtype == torch.float32, "the residual stream is float32")
+    if delta0 is not None:
+        _need(tuple(delta0.shape) == (T, H) and delta0.dtype == out.dtype, "the first pending delta must be [T, H] in the activation type")
     n = T if rows is None else rows.numel()
     if rows is not None:
         _i32(rows, n, "rows")
@@ -199,7 +252,7 @@ def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None) -> torch.Tenso
         _need(tuple(delta.shape) == (T, H) and delta.dtype == out.dtype, "delta must be [T, H] in the activation type")
     _check(
         _load("core").cw_add_rmsnorm(
-            _ptr(resid), _ptr(delta), parts, T, _ptr(weight), dtype_code(weight.dtype), float(eps), _ptr(out),
+            _ptr(resid), _ptr(delta0), _ptr(delta), parts, T, _ptr(weight), dtype_code(weight.dtype), float(eps), _ptr(out),
             dtype_code(out.dtype), _ptr(rows), n, H, _stream()),
         "add_rmsnorm",
     )
@@ -357,11 +410,33 @@ def qkv_rope_fused(x, weight, bias, positions, slots, inv_freq, nh: int, nkv: in
     return q
 
 
-def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+def swiglu_norm_fusable(M: int, two_i: int, K: int, dtype, gate_up_weight, delta) -> bool:
+    """Can the gate/up product make its own input rmsnorm(resid + delta)? Few bfloat16 rows of a
+    shape the streaming kernel takes, the pending delta a plain bfloat16 tensor."""
+    return (dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and gate_up_weight.shape[1] == K
+            and isinstance(delta, torch.Tensor) and delta.dtype == torch.bfloat16 and delta.is_contiguous()
+            and bool(_load("gemm").cw_gemm_bf16_swiglu_normed_ok(M, two_i, K)))
+
+
+def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
     """silu(x @ gate.T) * (x @ up.T) for gate_up_weight = [gate; up] stacked along dim 0.
 
     Few bfloat16 rows: one kernel that streams the weights once and applies the gate in its
     epilogue. Otherwise the product followed by the gate kernel."""
+    if isinstance(x, LazyAddNorm):
+        M, K = x.shape
+        two_i = gate_up_weight.shape[0]
+        if swiglu_norm_fusable(M, two_i, K, x.dtype, gate_up_weight, x.delta):
+            _gpu(x.resid, x.delta, x.weight, gate_up_weight)
+            out = torch.empty((M, two_i // 2), dtype=x.dtype, device=x.resid.device)
+            _check(
+                _load("gemm").cw_gemm_bf16_swiglu_normed(
+                    _ptr(x.resid), _ptr(x.delta), _ptr(x.weight), int(x.weight.dtype == torch.float32), float(x.eps),
+                    _ptr(gate_up_weight), _ptr(out), two_i // 2, M, two_i, K, _stream()),
+                "gemm_bf16_swiglu_normed",
+            )
+            return out
+        x = x.value()
     _gpu(x, gate_up_weight)
     M, K = x.shape
     two_i = gate_up_weight.shape[0]

@@ -2,6 +2,8 @@
 
 from __future__ import annotations
 
+from clockwork_amd import ops
+
 
 class PreNormBlock:
     """x = x + mixer(norm(x)); x = x + ffn(norm(x)) (clockwork/engine/model.py:139-154).
@@ -28,5 +30,13 @@ class PreNormBlock:
     def forward(self, resid, delta, ctx, cache):
         x = self.mixer_norm.forward(resid, delta)
         a = self.mixer.forward(x, ctx, cache)
+        # Few rows: the second norm can run inside the feed-forward's first product, which saves a
+        # launch. That kernel writes no residual, so the mixer's output stays pending and is
+        # handed on together with the feed-forward's (the next norm must be able to take both).
+        fuses = getattr(self.feed_forward, "fuses_input_norm", None)
+        lazy = getattr(self.ffn_norm, "lazy", None)
+        if (fuses is not None and lazy is not None and getattr(ctx, "next_norm_accepts_pending", False)
+                and fuses(resid.shape[0], x.dtype, a)):
+            return ops.PendingPair(a, self.feed_forward.forward(lazy(resid, a), ctx))
         x = self.ffn_norm.forward(resid, a)
         return self.feed_forward.forward(x, ctx)

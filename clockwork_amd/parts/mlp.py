@@ -26,5 +26,11 @@ class SwiGLU(Part):
         self.gate_up = params["gate_up_weight"]
         self.down = params["down_weight"]
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+    def fuses_input_norm(self, n_tokens: int, dtype, delta) -> bool:
+        """True if ``forward`` can take an ``ops.LazyAddNorm`` of that many rows and make the
+        norm inside the gate/up product (decode: few rows)."""
+        H, I = self.spec.hidden_size, self.spec.intermediate_size
+        return ops.swiglu_norm_fusable(n_tokens, 2 * I, H, dtype, self.gate_up, delta)
+
+    def forward(self, x, ctx) -> torch.Tensor:
         return ops.linear(ops.linear_swiglu(x, self.gate_up), self.down, partial_ok=True)

@@ -132,7 +132,11 @@ class DecoderModel:
         resid = torch.empty((T, self.spec.hidden_size), dtype=torch.float32, device=self.device)
         ops.embedding(self.embed, ctx.token_ids, resid)
         delta = None
-        for i, entry in enumerate(self.spec.run):
+        run = self.spec.run
+        for i, entry in enumerate(run):
+            # may this block hand on two pending outputs? Only if the norm that comes next takes them
+            nxt = self.layers[run[i + 1].layer].parts().get("mixer_norm") if i + 1 < len(run) else self.final_norm
+            ctx.next_norm_accepts_pending = bool(getattr(nxt, "accepts_pending", False))
             delta = self.layers[entry.layer].forward(resid, delta, ctx, caches[i])
         if ctx.num_logit_rows == 0:
             return None

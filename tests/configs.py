@@ -24,3 +24,12 @@ TINY_C = dict(
 )
 # name -> (config, weight seed, cache block size)
 TINY_CONFIGS = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8), "C": (TINY_C, 5, 16)}
+
+# Layers wide enough for the decode kernels that only take large shapes (the persistent
+# weight-streaming product, the norm fused into the gate/up product): hidden >= 1024 and at least
+# 512 row tiles of 8 in the feed-forward. Two layers and a small vocabulary keep it quick.
+WIDE = dict(
+    model_type="qwen2", vocab_size=1203, hidden_size=1024, num_hidden_layers=2, num_attention_heads=8,
+    num_key_value_heads=2, intermediate_size=4360, rms_norm_eps=2e-6, rope_theta=300000.0,
+    tie_word_embeddings=False,
+)

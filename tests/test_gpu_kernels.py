@@ -308,6 +308,67 @@ def test_streaming_product_many_row_tiles(M):
     torch.testing.assert_close(parts.parts.sum(0), x2.float() @ w2.float().t(), rtol=1e-4, atol=2e-4)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H", [(3, 176), (9, 1536), (2, 5000)])
+def test_add_rmsnorm_two_pending_deltas(dtype, T, H):
+    """Two branch outputs still to be added: the result is that of adding them one after the
+    other, bit for bit, with and without a row selection."""
+    from clockwork_amd import ops
+
+    resid = torch.randn(T, H, device=DEV)
+    a = torch.randn(T, H, device=DEV).to(dtype)
+    b = torch.randn(T, H, device=DEV).to(dtype)
+    parts = torch.randn(3, T, H, device=DEV)
+    w = (1 + 0.1 * torch.randn(H, device=DEV)).to(dtype)
+    for second in (b, ops.PartialSums(parts)):
+        r1 = resid.clone()
+        ops.add_rmsnorm(r1, a, w, 1e-6, torch.empty(T, H, device=DEV, dtype=dtype))
+        o1 = ops.add_rmsnorm(r1, second, w, 1e-6, torch.empty(T, H, device=DEV, dtype=dtype))
+        r2 = resid.clone()
+        o2 = ops.add_rmsnorm(r2, ops.PendingPair(a, second), w, 1e-6, torch.empty(T, H, device=DEV, dtype=dtype))
+        assert torch.equal(r1, r2) and torch.equal(o1, o2)
+        r3 = resid.clone()
+        rows = torch.tensor([T - 1, 0], dtype=torch.int32, device=DEV)
+        o3 = ops.add_rmsnorm(r3, ops.PendingPair(a, second), w, 1e-6, torch.empty(2, H, device=DEV, dtype=dtype), rows)
+        assert torch.equal(r3, resid) and torch.equal(o3, o1[[T - 1, 0]])
+    # a lazy norm computes its value without touching the residual
+    r4 = resid.clone()
+    lazy = ops.LazyAddNorm(r4, a, w, 1e-6, dtype)
+    r5 = resid.clone()
+    o5 = ops.add_rmsnorm(r5, a, w, 1e-6, torch.empty(T, H, device=DEV, dtype=dtype))
+    assert torch.equal(lazy.value(), o5) and torch.equal(r4, resid)
+
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("norm_weight_dtype", [torch.bfloat16, torch.float32])
+def test_swiglu_product_with_the_norm_inside(M, norm_weight_dtype):
+    """gate/up product that makes its own input rmsnorm(resid + delta): against the two kernels
+    it replaces and against float32 arithmetic; the residual is left alone."""
+    from clockwork_amd import ops
+
+    K, I = 1536, 4360 + 4
+    resid = torch.randn(M, K, device=DEV)
+    delta = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    nw = (1 + 0.1 * torch.randn(K, device=DEV)).to(norm_weight_dtype)
+    w = (torch.randn(2 * I, K, device=DEV) / K ** 0.5).to(torch.bfloat16)
+    assert ops.swiglu_norm_fusable(M, 2 * I, K, torch.bfloat16, w, delta)
+    before = resid.clone()
+    got = ops.linear_swiglu(ops.LazyAddNorm(resid, delta, nw, 1e-6, torch.bfloat16), w)
+    assert torch.equal(resid, before)
+    x = ops.add_rmsnorm(resid.clone(), delta, nw, 1e-6, torch.empty(M, K, device=DEV, dtype=torch.bfloat16))
+    two_kernels = ops.linear_swiglu(x, w)
+    torch.testing.assert_close(got.float(), two_kernels.float(), rtol=2e-2, atol=2e-2)
+    v = resid + delta.float()
+    xn = (v * torch.rsqrt((v * v).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16).float() * nw.float()
+    y = xn.to(torch.bfloat16).float() @ w.float().t()
+    torch.testing.assert_close(got.float(), torch.nn.functional.silu(y[:, :I]) * y[:, I:], rtol=2e-2, atol=2e-2)
+    # a shape the fused kernel does not take falls back to the norm kernel and the plain product
+    small = (torch.randn(2 * 96, K, device=DEV) / K ** 0.5).to(torch.bfloat16)
+    assert not ops.swiglu_norm_fusable(M, 2 * 96, K, torch.bfloat16, small, delta)
+    torch.testing.assert_close(ops.linear_swiglu(ops.LazyAddNorm(resid, delta, nw, 1e-6, torch.bfloat16), small).float(),
+                               ops.linear_swiglu(x, small).float(), rtol=0, atol=0)
+
+
 @pytest.mark.parametrize("M", [1, 8, 20, 64, 100])
 @pytest.mark.parametrize("I,K", [(176, 64), (8960, 1536), (100, 80), (52, 200)])
 def test_fused_swiglu_product(M, I, K):

@@ -60,6 +60,42 @@ def test_replay_matches_plain(model_dirs, name, dtype, mode):
     assert runner.manager.min_free_blocks() == runner.manager.num_blocks
 
 
+@pytest.mark.parametrize("mode", ["prefill_then_decode", "mixed"])
+def test_wide_layers_take_the_streaming_and_fused_paths(tmp_path, mode):
+    """A model with layers as wide as real ones, so that decode steps run the kernels that tiny
+    layers never reach: the persistent streaming product and the second norm fused into the
+    gate/up product (eager and as replayed HIP graphs), against the plain implementation."""
+    from clockwork_amd import ops
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests.configs import WIDE
+
+    model_dir = write_random_model(tmp_path / "wide", WIDE, 3)
+    lib = ops._load("gemm")
+    assert lib.cw_gemm_bf16_swiglu_normed_ok(4, 2 * WIDE["intermediate_size"], WIDE["hidden_size"]) == 1
+    calls = {"fused": 0}
+    real = lib.cw_gemm_bf16_swiglu_normed
+
+    def counting(*args):
+        calls["fused"] += 1
+        return real(*args)
+
+    gen = torch.Generator().manual_seed(11)
+    requests = {f"w{i}": torch.randint(0, WIDE["vocab_size"], (n,), generator=gen).tolist() for i, n in enumerate([40, 70, 55])}
+    plain = PlainQwen2(model_dir)
+    want = {rid: plain.logits(toks) for rid, toks in requests.items()}
+    live = 3 if mode == "mixed" else 1
+    runner = replay.make_runner(model_dir, "bfloat16", 16, replay.pages_needed(requests, live, 16))
+    lib.cw_gemm_bf16_swiglu_normed = counting
+    try:
+        got = replay.run_trace(runner, getattr(replay, mode)(requests))
+    finally:
+        lib.cw_gemm_bf16_swiglu_normed = real
+    assert calls["fused"] > 0
+    worst = replay.compare(got, want, **TOL["bfloat16"])
+    print(f"wide bfloat16 {mode}: largest error {worst:.3e}, fused norm launches {calls['fused']}")
+    assert not runner.manager.live_requests()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_and_long_decoding(model_dirs, dtype):
     """The first tokens of a sequence (one-token prompt, then decoding from position 1) and a
