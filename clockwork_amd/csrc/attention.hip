@@ -828,7 +828,6 @@ __global__ __launch_bounds__(PrefillTile<HD>::NT, (HD <= 128 ? 2 : 1)) void attn
   constexpr int CPR = HD / 8;     // 16-byte chunks of a row
   constexpr int NH = Tile::NH, KW = Tile::KW, KT = Tile::KT, NT = Tile::NT;
   constexpr int NKB = KW / 16;  // 16-key blocks of a wave's keys
-  constexpr int NCH = (KT * CPR + NT - 1) / NT;  // chunks of a stage per thread
   extern __shared__ __align__(16) unsigned char smem_raw[];
   bf16_t* tiles = reinterpret_cast<bf16_t*>(smem_raw);  // [stage 2][K tile, V tile]
   int* tbl = reinterpret_cast<int*>(smem_raw + Tile::BYTES);
@@ -895,34 +894,43 @@ __global__ __launch_bounds__(PrefillTile<HD>::NT, (HD <= 128 ? 2 : 1)) void attn
   // running maximum in units of the raw score (the scale is positive) and the lane's share of the sum
   float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
   const float sl2 = p.scale * 1.4426950408889634f;  // exp(x * scale) = exp2(x * sl2)
+  const float rescale_step = 8.0f / sl2;            // 8 in the exponent, in units of the raw score
 
-  // ---- tile traffic: thread -> chunks idx = tid + i * NT of the KT x CPR chunks of K and of V
+  // ---- tile traffic: TPK threads share a key of the stage; thread j of them takes the 16-byte
+  // chunks j, j + TPK, ... of its K row and of its V row, so a thread looks up one page and
+  // builds one address per stage, and neighbouring lanes read neighbouring chunks (lanes spread
+  // over 16 different rows, which would suit the LDS banks better, cost more in memory coalescing
+  // than they saved: measured)
+  constexpr int TPK = NT / KT;                  // threads per key
+  constexpr int NCK = (CPR + TPK - 1) / TPK;    // chunks per thread and matrix
   const int t_first = wg_lo / KT, t_last = wg_last / KT;
-  u32x4_t gk[NCH], gv[NCH];
+  const int f_key = threadIdx.x / TPK, f_ch = threadIdx.x % TPK;
+  const int64_t row_elems = (int64_t)p.nkv * HD;
+  u32x4_t gk[NCK], gv[NCK];
   auto fetch = [&](int t) __attribute__((always_inline)) {  // global -> registers; a masked key reads a row of zeros
+    const int kp = t * KT + f_key;
+    bool ok = kp >= wg_lo && kp <= wg_last;
+    const int page = tbl[ok ? cw_page_index<POW2>(kp, bs, sh) - page0 : 0];
+    ok = ok && page >= 0;
+    const int64_t off = ((int64_t)page * bs + cw_page_offset<POW2>(kp, bs, sh)) * row_elems + kvh * HD + f_ch * 8;
+    const bf16_t* kr = ok ? kc + off : zrow;
+    const bf16_t* vr = ok ? vc + off : zrow;
+    const int step = ok ? TPK * 8 : 0;  // the row of zeros is short: every chunk reads its start
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int idx = threadIdx.x + i * NT;
-      const int key = idx / CPR, ch = idx - key * CPR;
-      const int kp = t * KT + key;
-      bool ok = idx < KT * CPR && kp >= wg_lo && kp <= wg_last;
-      const int page = tbl[ok ? cw_page_index<POW2>(kp, bs, sh) - page0 : 0];
-      ok = ok && page >= 0;
-      const int64_t off = (((int64_t)page * bs + cw_page_offset<POW2>(kp, bs, sh)) * p.nkv + kvh) * HD + ch * 8;
-      gk[i] = *reinterpret_cast<const u32x4_t*>(ok ? kc + off : zrow);
-      gv[i] = *reinterpret_cast<const u32x4_t*>(ok ? vc + off : zrow);
+    for (int i = 0; i < NCK; ++i) {
+      const bool in_row = CPR % TPK == 0 || f_ch + i * TPK < CPR;
+      gk[i] = *reinterpret_cast<const u32x4_t*>(kr + (in_row ? i * step : 0));
+      gv[i] = *reinterpret_cast<const u32x4_t*>(vr + (in_row ? i * step : 0));
     }
   };
   auto stash = [&](int stage) __attribute__((always_inline)) {  // registers -> LDS
-    bf16_t* ks = tiles + stage * Tile::STAGE;
-    bf16_t* vs = ks + KT * KROW;
+    bf16_t* ks = tiles + stage * Tile::STAGE + f_key * KROW + f_ch * 8;
+    bf16_t* vs = tiles + stage * Tile::STAGE + KT * KROW + f_key * VROW + f_ch * 8;
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int idx = threadIdx.x + i * NT;
-      if (idx < KT * CPR) {
-        const int key = idx / CPR, ch = idx - key * CPR;
-        *reinterpret_cast<u32x4_t*>(ks + key * KROW + ch * 8) = gk[i];
-        *reinterpret_cast<u32x4_t*>(vs + key * VROW + ch * 8) = gv[i];
+    for (int i = 0; i < NCK; ++i) {
+      if (CPR % TPK == 0 || f_ch + i * TPK < CPR) {
+        *reinterpret_cast<u32x4_t*>(ks + i * TPK * 8) = gk[i];
+        *reinterpret_cast<u32x4_t*>(vs + i * TPK * 8) = gv[i];
       }
     }
   };
@@ -996,7 +1004,11 @@ __global__ __launch_bounds__(PrefillTile<HD>::NT, (HD <= 128 ? 2 : 1)) void attn
       float alpha[2];
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
-        const float m_new = fmaxf(m_run[b], tmax[b]);
+        // The reference point of the exponentials moves only when the maximum has grown by more
+        // than 2^8 in the exponent (or is the row's first): probabilities then reach 256 at most,
+        // which float32 sums and bfloat16 products take without loss, and the accumulators are
+        // rescaled a few times per row instead of in most tiles. The result is the same quotient.
+        const float m_new = tmax[b] > m_run[b] + rescale_step ? tmax[b] : m_run[b];
         // a row that has seen no key yet keeps m = -inf; its probabilities are zero
         const float msc = m_new == -INFINITY ? 0.0f : m_new * sl2;
         const float a = __builtin_amdgcn_exp2f(m_run[b] * sl2 - msc);
