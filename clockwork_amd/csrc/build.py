@@ -37,7 +37,7 @@ FLAGS = [
 PLAIN_SOURCES = {"core": "core.hip", "gemm": "gemm.hip", "sampling": "sampling.hip"}
 ATTENTION_SOURCE = "attention.hip"
 # head sizes compiled by build_all: the tests' models, the kernel tests and the benchmark's
-DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 128)
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 160, 224, 256)
 
 
 def _log(msg: str) -> None:

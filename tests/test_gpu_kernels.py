@@ -580,6 +580,8 @@ DECODE_KERNEL_CASES = [
     (3, 3, 128, 32, [5, 1000]),
     (5, 1, 256, 16, [77, 300]),
     (14, 2, 128, 16, [2304]),
+    (4, 2, 160, 16, [130, 9]),
+    (3, 1, 224, 8, [400]),
 ]
 
 
@@ -606,7 +608,7 @@ def test_decode_attention_kernel(nh, nkv, hd, bs, ctx_lens, splits, fixed_ranges
 
 
 @pytest.mark.parametrize("nh,nkv,hd,bs", [(4, 2, 32, 4), (6, 1, 32, 8), (3, 3, 64, 16), (12, 2, 128, 16), (2, 1, 256, 16),
-                                          (40, 1, 64, 8), (7, 7, 96, 16)])
+                                          (40, 1, 64, 8), (7, 7, 96, 16), (4, 2, 160, 16), (2, 2, 224, 8)])
 @pytest.mark.parametrize("window", [0, 9, 40])
 def test_prefill_attention_kernel(nh, nkv, hd, bs, window):
     """The matrix-core kernel for portions: cached prefix + new tokens, ragged sizes, groups that
