@@ -19,7 +19,11 @@ from clockwork_amd.registry import build_part
 
 
 class PagedAttention(Part):
-    graph_safe = True
+    @property
+    def graph_safe(self) -> bool:
+        """A fixed sequence of launches if the position encoding is one too."""
+        return bool(getattr(self.position, "graph_safe", False))
+
     def __init__(self, spec: AttentionSpec) -> None:
         self.spec = spec
         self.position = build_part(spec.position) if spec.position is not None else NoPosition()

@@ -15,6 +15,8 @@ from clockwork_amd.parts.specs import RopeNeoxSpec
 
 
 class RopeNeox(Part):
+    graph_safe = True
+
     def __init__(self, spec: RopeNeoxSpec) -> None:
         if spec.rotary_dim % 2:
             raise ValueError(f"rotary_dim {spec.rotary_dim} must be even")
@@ -42,6 +44,8 @@ class RopeNeox(Part):
 
 class NoPosition(Part):
     """Stands in when a mixer has no position encoding: bias and cache write only."""
+
+    graph_safe = True
 
     def rotate_and_store(self, qkv, bias, positions, slots, nh, nkv, hd, k_cache, v_cache) -> None:
         ops.rope_kv_write(qkv, bias, positions, slots, None, 0, nh, nkv, hd, k_cache, v_cache)

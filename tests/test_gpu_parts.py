@@ -136,6 +136,81 @@ class EmaMixer:
 
 
 @dataclass(frozen=True)
+class RoutedFFNSpec:
+    """A feed-forward with routing: a float32 softmax over ``experts`` router logits, the best
+    ``top_k`` renormalised, each expert a two-layer ReLU network."""
+
+    hidden_size: int
+    inner_size: int
+    experts: int
+    top_k: int
+
+
+class RoutedFFN:
+    def __init__(self, spec):
+        self.spec = spec
+
+    def param_specs(self):
+        s = self.spec
+        return {
+            "router": ParamSpec((s.experts, s.hidden_size), init=("normal", 0.5)),
+            "w_in": ParamSpec((s.experts, s.inner_size, s.hidden_size), init=("normal", 0.1)),
+            "w_out": ParamSpec((s.experts, s.hidden_size, s.inner_size), init=("normal", 0.1)),
+        }
+
+    def bind(self, params, device, dtype):
+        self.router, self.w_in, self.w_out = params["router"], params["w_in"], params["w_out"]
+
+    def forward(self, x, ctx):
+        gates = torch.softmax(x.float() @ self.router.float().t(), dim=-1)
+        top, idx = gates.topk(self.spec.top_k, dim=-1)
+        top = top / top.sum(-1, keepdim=True)
+        out = torch.zeros(x.shape[0], self.spec.hidden_size, dtype=torch.float32, device=x.device)
+        for e in range(self.spec.experts):
+            weight = (top * (idx == e)).sum(-1, keepdim=True)  # zero for tokens that did not choose e
+            out += weight * (torch.relu(x.float() @ self.w_in[e].float().t()) @ self.w_out[e].float().t())
+        return out.to(x.dtype)
+
+
+@dataclass(frozen=True)
+class SinePositionSpec:
+    """A position encoding that is no rotation: scale * sin(pos / (i + 1)) is added to element i of
+    every query and key head."""
+
+    scale: float
+
+
+class SinePosition:
+    # no ``graph_safe``: the cache write below picks rows with a mask, so steps run eagerly
+
+    def __init__(self, spec):
+        self.spec = spec
+
+    def param_specs(self):
+        return {}
+
+    def bind(self, params, device, dtype):
+        pass
+
+    def rotate_and_store(self, qkv, bias, positions, slots, nh, nkv, hd, k_cache, v_cache):
+        T = qkv.shape[0]
+        if bias is not None:
+            qkv += bias.to(qkv.dtype)
+        i = torch.arange(hd, device=qkv.device, dtype=torch.float32)
+        enc = self.spec.scale * torch.sin(positions.float()[:, None, None] / (i + 1.0))
+        q = qkv[:, : nh * hd].view(T, nh, hd)
+        q.copy_((q.float() + enc).to(qkv.dtype))
+        if nkv:
+            k = qkv[:, nh * hd : (nh + nkv) * hd].view(T, nkv, hd)
+            v = qkv[:, (nh + nkv) * hd :].view(T, nkv, hd)
+            k.copy_((k.float() + enc).to(qkv.dtype))
+            keep = slots >= 0
+            rows = slots[keep].long()
+            k_cache.reshape(-1, nkv, hd)[rows] = k[keep]
+            v_cache.reshape(-1, nkv, hd)[rows] = v[keep]
+
+
+@dataclass(frozen=True)
 class ToyConfig:
     vocab: int
     hidden: int
@@ -149,8 +224,8 @@ def _toy_spec(cfg: ToyConfig) -> ModelSpec:
     ffn = SwiGLUSpec(cfg.hidden, 2 * cfg.hidden)
     rope = RopeNeoxSpec(rotary_dim=16, theta=1000.0)
 
-    def attn(window):
-        return AttentionSpec(cfg.hidden, 4, 2, 16, True, False, 0.25, window=window, position=rope)
+    def attn(window, position=rope):
+        return AttentionSpec(cfg.hidden, 4, 2, 16, True, False, 0.25, window=window, position=position)
 
     layers, run = [], []
     for kind in cfg.kinds:
@@ -160,6 +235,10 @@ def _toy_spec(cfg: ToyConfig) -> ModelSpec:
         if kind == "borrow":      # a layer that makes queries only and reads the first entry's keys
             layers.append(LayerSpec("prenorm", attn(None), ffn, norm, norm))
             run.append(RunEntry(layer=len(layers) - 1, cache_from=0))
+            continue
+        if kind == "routed":      # full attention with the sine encoding, then a routed feed-forward
+            layers.append(LayerSpec("prenorm", attn(None, SinePositionSpec(0.5)), RoutedFFNSpec(cfg.hidden, 40, 3, 2), norm, norm))
+            run.append(RunEntry(layer=len(layers) - 1))
             continue
         mixer = {"full": attn(None), "window": attn(cfg.window), "ema": EmaMixerSpec(cfg.hidden, 0.75)}[kind]
         layers.append(LayerSpec("prenorm", mixer, ffn, norm, norm))
@@ -182,6 +261,8 @@ def toy_dir(tmp_path_factory):
     from clockwork_amd.weights.random_init import write_random_model
 
     register_part(EmaMixerSpec, EmaMixer)
+    register_part(RoutedFFNSpec, RoutedFFN)
+    register_part(SinePositionSpec, SinePosition)
     register_architecture(
         ["ToyForCausalLM"],
         Architecture(
@@ -192,7 +273,7 @@ def toy_dir(tmp_path_factory):
         ),
     )
     config = {"architectures": ["ToyForCausalLM"], "vocab": 300, "hidden": 64, "window": 6, "eps": 1e-5,
-              "kinds": ["full", "window", "again", "ema", "borrow"]}
+              "kinds": ["full", "window", "again", "ema", "borrow", "routed"]}
     return write_random_model(tmp_path_factory.mktemp("toy") / "toy", config, seed=3)
 
 
@@ -226,9 +307,14 @@ def _toy_plain_logits(model_dir, tokens):
             a = torch.stack(rows)
         else:
             qkv = plain.linear(x, w[p + "mixer.qkv_weight"], w[p + "mixer.qkv_bias"])
-            q = plain.apply_rope(qkv[:, :64].view(T, 4, 16), cos, sin)
+            if kind == "routed":
+                enc = 0.5 * torch.sin(torch.arange(T).float()[:, None, None] / (torch.arange(16).float() + 1.0))
+                encode = lambda t: t + enc
+            else:
+                encode = lambda t: plain.apply_rope(t, cos, sin)
+            q = encode(qkv[:, :64].view(T, 4, 16))
             if borrow is None:
-                k = plain.apply_rope(qkv[:, 64:96].view(T, 2, 16), cos, sin)
+                k = encode(qkv[:, 64:96].view(T, 2, 16))
                 v = qkv[:, 96:].view(T, 2, 16)
                 kv_of[i] = (k, v)
             else:
@@ -237,6 +323,17 @@ def _toy_plain_logits(model_dir, tokens):
             a = plain.linear(plain.attention_dense(q, k, v, 0.25, window=window).reshape(T, 64), w[p + "mixer.out_weight"])
         h = h + a
         x = plain.rmsnorm(h, w[p + "ffn_norm.weight"], cfg["eps"])
+        if kind == "routed":
+            gates = torch.softmax(x @ w[p + "feed_forward.router"].t(), dim=-1)
+            y = torch.zeros(T, H)
+            for t in range(T):  # token by token, expert by expert
+                best = sorted(range(3), key=lambda e: -float(gates[t, e]))[:2]
+                total = sum(float(gates[t, e]) for e in best)
+                for e in best:
+                    hidden = torch.relu(w[p + "feed_forward.w_in"][e] @ x[t])
+                    y[t] += float(gates[t, e]) / total * (w[p + "feed_forward.w_out"][e] @ hidden)
+            h = h + y
+            continue
         gu = w[p + "feed_forward.gate_up_weight"]
         h = h + plain.swiglu(x, gu[: 2 * H], gu[2 * H :], w[p + "feed_forward.down_weight"])
     return plain.linear(plain.rmsnorm(h, w["final_norm.weight"], cfg["eps"]), w["embed.weight"])
@@ -248,8 +345,9 @@ def test_a_toy_architecture_registers_builds_and_steps(toy_dir, dtype, mode):
     gen = torch.Generator().manual_seed(5)
     requests = {f"t{i}": torch.randint(0, 300, (n,), generator=gen).tolist() for i, n in enumerate([50, 9, 77, 30, 64])}
     runner = replay.make_runner(toy_dir, dtype, 8, 64)
-    # three groups: all keys (two entries + a borrower), a window (two entries: the layer and its rerun), a state
-    assert [(g.is_kv, g.window, g.entries) for g in runner.manager.groups] == [(True, None, (0,)), (True, 6, (1, 2)), (False, None, (3,))]
+    # three groups: all keys (the first and the last entry; a borrower reads the first's), a window
+    # (two entries: the layer and its rerun), a state
+    assert [(g.is_kv, g.window, g.entries) for g in runner.manager.groups] == [(True, None, (0, 5)), (True, 6, (1, 2)), (False, None, (3,))]
     assert not runner.manager.supports_prefix_sharing
     got = replay.run_trace(runner, getattr(replay, mode)(requests))
     ref = {rid: _toy_plain_logits(toy_dir, toks) for rid, toks in requests.items()}
