@@ -67,6 +67,8 @@ class SchedulerConfig:
     preemption_mode: str = "recompute"
     enable_chunked_prefill: bool = True
     max_prefill_chunk: int = 0
+    # decide a decode-only step while the step before it still runs on the GPU
+    lookahead: bool = True
 
 
 _SECTIONS = ("model", "cache", "scheduler")

@@ -279,16 +279,20 @@ class StaticDecodeBatch:
             ctx.attention_plan(nh, nkv)
         self.ctx = ctx
 
-    def fill(self, entries: Sequence[StepEntry], manager) -> None:
+    def fill(self, entries: Sequence[StepEntry], manager, upload: bool = True) -> None:
         """Write this step's indices into the pinned buffer and send them to the device.
 
         Block-table rows are kept from step to step: a row is rewritten only when another request
         moves into it or one of its entries changed (the request's ``epoch`` says so); otherwise
-        just the newly taken pages are added."""
+        just the newly taken pages are added. With ``upload`` off the buffer is only prepared (an
+        entry's token may still be unknown: any placeholder): ``set_tokens`` and ``upload`` follow."""
         n = len(entries)
         size, width = self.size, self.table_width
         a = self._np
         bs = self.block_size
+        sent = getattr(self, "_sent", None)
+        if sent is not None:
+            sent.synchronize()  # the copy of the step before must have read the buffer
 
         def region(name):
             o, cnt = self._offsets[name]
@@ -337,5 +341,16 @@ class StaticDecodeBatch:
                     table[r, :] = -1
                     if g == len(manager.kv_groups) - 1:
                         rows[r][0], rows[r][1] = None, 0
-        self.device_buf.copy_(self.host, non_blocking=True)
         self.ctx.seq_ids = [e.seq_id for e in entries] + [""] * (size - n)
+        if upload:
+            self.upload()
+
+    def set_tokens(self, tokens: Sequence[int]) -> None:
+        """The tokens of the entries that ``fill`` prepared."""
+        o, _ = self._offsets["token_ids"]
+        self._np[o : o + len(tokens)] = tokens
+
+    def upload(self) -> None:
+        self.device_buf.copy_(self.host, non_blocking=True)
+        self._sent = torch.cuda.Event()
+        self._sent.record()

@@ -57,6 +57,18 @@ class LLMEngine:
         # arrival "times" are a counter, so order never depends on the clock (llm_engine.py:57-59)
         self._arrivals = itertools.count()
         self._generate_ids = itertools.count()
+        self._ahead = None          # (SchedulerOutput, runner handle) made one step ahead
+        self.lookahead_steps = 0    # steps that ran from such a schedule
+
+    def _look_ahead(self, out):
+        """(schedule, runner handle) of the step after ``out`` if it can be decided before
+        ``out``'s tokens are known (see Scheduler.schedule_ahead); the handle is None when the
+        runner has nothing to prepare for it."""
+        nxt = self.scheduler.schedule_ahead(out, self.cfg.model.max_model_len)
+        if nxt is None:
+            return None
+        self.runner.apply_copies(nxt.copies)
+        return nxt, self.runner.prepare_decode([(p.seq.seq_id, p.start) for p in nxt.portions])
 
     @classmethod
     def from_config(cls, cfg: EngineConfig) -> "LLMEngine":
@@ -117,29 +129,44 @@ class LLMEngine:
     def step(self) -> list[RequestOutput]:
         """Schedule, run one batch, sample, finish; an output per request that got a token
         (llm_engine.py:99-125)."""
-        out = self.scheduler.schedule()
-        if not out.portions:
-            if out.preempted or not self.scheduler.has_unfinished():
-                return []
-            # nothing runs and the head does not fit: give it everything the prefix cache
-            # holds idle, once, before calling the request unschedulable (llm_engine.py:102-113)
-            if self.prefix_cache.evict(self.manager.num_blocks) > 0:
-                out = self.scheduler.schedule()
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None and ahead[0].version == self.scheduler.version:
+            # decided (and mostly laid out) while the last step ran; nothing has changed since
+            out, handle = ahead
+            self.scheduler.commit_ahead(out)
+            self.lookahead_steps += 1
+        else:
+            handle = None
+            out = self.scheduler.schedule()
             if not out.portions:
-                raise RuntimeError("waiting request cannot be admitted even with an empty prefix cache")
-        self.runner.apply_copies(out.copies)
-        entries = [
-            StepEntry(
-                p.seq.seq_id,
-                p.start,
-                p.seq.tokens_in(p.start, p.start + p.num_tokens),
-                [p.num_tokens - 1] if p.samples else [],
-            )
-            for p in out.portions
-        ]
-        logits = self.runner.step(entries)
+                if out.preempted or not self.scheduler.has_unfinished():
+                    return []
+                # nothing runs and the head does not fit: give it everything the prefix cache
+                # holds idle, once, before calling the request unschedulable (llm_engine.py:102-113)
+                if self.prefix_cache.evict(self.manager.num_blocks) > 0:
+                    out = self.scheduler.schedule()
+                if not out.portions:
+                    raise RuntimeError("waiting request cannot be admitted even with an empty prefix cache")
+            self.runner.apply_copies(out.copies)
+        if handle is not None:
+            logits = self.runner.step_prepared(handle, [p.seq.output_token_ids[-1] for p in out.portions])
+        else:
+            entries = [
+                StepEntry(
+                    p.seq.seq_id,
+                    p.start,
+                    p.seq.tokens_in(p.start, p.start + p.num_tokens),
+                    [p.num_tokens - 1] if p.samples else [],
+                )
+                for p in out.portions
+            ]
+            logits = self.runner.step(entries)
         sampling = [p.seq for p in out.portions if p.samples]
-        tokens = self.sampler.sample(logits, sampling) if sampling else []
+        drawn_on_device = self.sampler.launch(logits, sampling) if sampling else None
+        # the GPU is busy with this step: decide the next one now if it is plain decoding
+        if self.cfg.scheduler.lookahead:
+            self._ahead = self._look_ahead(out)
+        tokens = drawn_on_device.tolist() if drawn_on_device is not None else []
         outputs: list[RequestOutput] = []
         drawn = iter(tokens)
         for p in out.portions:
@@ -197,6 +224,7 @@ class LLMEngine:
             "prefix_cache_prompt_tokens": cache.prompt_tokens,
             "prefix_cache_hit_rate": cache.hit_rate,
             "num_free_blocks": self.manager.min_free_blocks(),
+            "lookahead_steps": self.lookahead_steps,
         }
 
     # ------------------------------------------------------------------ text and finishing

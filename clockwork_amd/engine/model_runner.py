@@ -174,6 +174,44 @@ class ModelRunner:
             return out[:n]
         return out[torch.tensor(rows, device=self.device)]
 
+    def prepare_decode(self, positions: Sequence[tuple[str, int]]):
+        """Get a decode-only step ready before its tokens are known: ``positions`` names each
+        request and the position of its next token (pages reserved). Returns a handle for
+        ``step_prepared``, or None when the step cannot simply replay a captured graph (then
+        ``step`` runs it as usual). Everything but the tokens is written to the pinned buffer."""
+        n = len(positions)
+        if not (self.use_graphs and not self.manager.state_groups and 0 < n <= GRAPH_BATCH_SIZES[-1]):
+            return None
+        size = next(b for b in GRAPH_BATCH_SIZES if b >= n)
+        longest = max(start + 1 for _, start in positions)
+        if longest > self._table_width * self.manager.block_size:
+            return None
+        key = (size, GRAPH_KEY_BUCKET * -(-longest // GRAPH_KEY_BUCKET))
+        state = self._graphs.get(key)
+        if not isinstance(state, tuple):
+            return None
+        entries = [StepEntry(seq_id, start, (0,), (0,)) for seq_id, start in positions]
+        state[0].fill(entries, self.manager, upload=False)
+        return key, entries
+
+    @torch.no_grad()
+    def step_prepared(self, handle, tokens: Sequence[int]) -> torch.Tensor:
+        """Run the step that ``prepare_decode`` got ready, now that its tokens are known; every
+        entry's logits are returned, float32 [entries, vocab]."""
+        key, entries = handle
+        if len(tokens) != len(entries):
+            raise ValueError(f"{len(tokens)} tokens for {len(entries)} prepared entries")
+        for e, tok in zip(entries, tokens):
+            if not 0 <= int(tok) < self.spec.vocab_size:
+                raise ValueError(f"request {e.seq_id}: token id {tok} outside the vocabulary")
+        batch, graph, out = self._graphs[key]
+        batch.set_tokens(tokens)
+        batch.upload()
+        graph.replay()
+        for e in entries:
+            self.manager.release_behind_window(e.seq_id, e.start + 1)
+        return out[: len(entries)]
+
     # ------------------------------------------------------------------ the step
     @torch.no_grad()
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:

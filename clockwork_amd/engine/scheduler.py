@@ -54,6 +54,7 @@ class SchedulerOutput:
     preempted: list[Sequence] = field(default_factory=list)
     copies: list[tuple[int, int, int]] = field(default_factory=list)  # (group, src, dst) page copies
     num_batched_tokens: int = 0
+    version: int = -1  # of the scheduler's queues, for an output made ahead of time (``schedule_ahead``)
 
     def is_empty(self) -> bool:
         return not (self.portions or self.preempted)
@@ -81,6 +82,9 @@ class Scheduler:
         self._matches: dict[str, PrefixMatch] = {}
         self._order: dict[str, int] = {}
         self._counter = 0
+        # grows whenever a request arrives, leaves, is preempted or aborted: an output made ahead
+        # of time is good only while it has not moved
+        self.version = 0
 
     # ------------------------------------------------------------------ queue
     def _priority(self, seq: Sequence) -> tuple[float, int]:
@@ -91,6 +95,7 @@ class Scheduler:
         self._counter += 1
         seq.status = SequenceStatus.WAITING
         self.waiting.append(seq)
+        self.version += 1
         self._refresh()
 
     def has_unfinished(self) -> bool:
@@ -119,6 +124,7 @@ class Scheduler:
             i += 1
         self.waiting.insert(i, seq)
         self.stats.num_preempted_total += 1
+        self.version += 1
 
     def _evict_for(self, pages: int) -> bool:
         """Try to free ``pages`` pages from idle prefix-cache blocks; True if any went."""
@@ -221,12 +227,51 @@ class Scheduler:
         self._refresh()
         return out
 
+    # ------------------------------------------------------------------ one step ahead
+    def schedule_ahead(self, prev: SchedulerOutput, max_len: Optional[int] = None) -> Optional[SchedulerOutput]:
+        """The step after ``prev``, decided while ``prev`` still runs on the GPU and its tokens
+        are unknown, for the common case that nothing changes: nobody waits, every running
+        request decoded one token in ``prev`` and none of them ends by length (``max_tokens``, the
+        model length, ``max_len`` if the caller has a tighter one) with that token.
+        The pages of the next positions are taken now; nothing is evicted or preempted ahead of
+        time. Returns None when the ordinary ``schedule`` has to decide. The caller may use the
+        result only if ``version`` still equals the scheduler's when the tokens have arrived (no
+        request stopped, arrived or was aborted), and then calls ``commit_ahead``; a result
+        that is dropped leaves the pages with their requests, which ask for them again anyway."""
+        if self.waiting or prev.preempted or not prev.portions or len(prev.portions) != len(self.running):
+            return None
+        limit = self.cfg.max_model_len if max_len is None else min(self.cfg.max_model_len, max_len)
+        for p in prev.portions:
+            seq = p.seq
+            if p.num_tokens != 1 or not p.samples or seq.status is not SequenceStatus.RUNNING:
+                return None
+            if (len(seq.output_token_ids) + 1 >= seq.sampling_params.max_tokens
+                    or len(seq) + 1 >= limit):
+                return None  # its last token is being made right now
+        for p in prev.portions:
+            if not self.manager.can_extend(p.seq.seq_id, p.start + 1, p.start + 2):
+                return None
+        out = SchedulerOutput(version=self.version)
+        for p in prev.portions:
+            out.copies += self.manager.extend(p.seq.seq_id, p.start + 1, p.start + 2)
+            out.portions.append(ScheduledPortion(p.seq, p.start + 1, 1, True))
+            out.decode_seqs.append(p.seq)
+            out.num_batched_tokens += 1
+        return out
+
+    def commit_ahead(self, out: SchedulerOutput) -> None:
+        """``out`` of ``schedule_ahead`` is run as this step's schedule."""
+        if out.version != self.version:
+            raise RuntimeError("the schedule made ahead of time is out of date")
+        self.stats.num_scheduled_batches += 1
+
     # ------------------------------------------------------------------ finishing
     def free_finished(self) -> None:
         for seq in self.running:
             if seq.is_finished():
                 self._release(seq)
                 self._order.pop(seq.seq_id, None)
+                self.version += 1
         self.running = [seq for seq in self.running if not seq.is_finished()]
         self._refresh()
 
@@ -241,5 +286,6 @@ class Scheduler:
                     queue.pop(i)
                     seq.status = SequenceStatus.FINISHED_ABORTED
                     self._order.pop(seq_id, None)
+                    self.version += 1
                     self._refresh()
                     return

@@ -25,14 +25,20 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, seqs: Seq[Sequence]) -> list[int]:
         """One token per row of ``logits`` (float32 [n, vocab]); row i belongs to ``seqs[i]``."""
+        drawn = self.launch(logits, seqs)
+        return [] if drawn is None else drawn.tolist()
+
+    def launch(self, logits: torch.Tensor, seqs: Seq[Sequence]):
+        """Start the kernels of ``sample`` and return the tokens as a device tensor (int32 [n]),
+        without waiting for them; None for no sequences."""
         n = len(seqs)
         if n == 0:
-            return []
+            return None
         if logits.shape[0] != n:
             raise ValueError(f"{logits.shape[0]} logits rows for {n} sequences")
         params = [s.sampling_params for s in seqs]
         if all(p.greedy for p in params):
-            return ops.argmax(logits).tolist()
+            return ops.argmax(logits)
         vocab = logits.shape[1]
         temperature = torch.tensor([p.temperature for p in params], dtype=torch.float32)
         top_k = torch.tensor([p.top_k if 0 < p.top_k < vocab else -1 for p in params], dtype=torch.int32)
@@ -44,4 +50,4 @@ class Sampler:
         dev = self.device
         return ops.sample(
             logits, temperature.to(dev), top_k.to(dev), top_p.to(dev), seeds.to(dev), draws.to(dev)
-        ).tolist()
+        )

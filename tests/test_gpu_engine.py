@@ -57,6 +57,60 @@ def test_bfloat16_generation_follows_the_plain_implementation(model_dirs):
                 break
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_decided_one_step_ahead_change_nothing(model_dirs, dtype):
+    """Requests that end at different times (lengths, an end-of-sequence token), one arriving in
+    the middle and one aborted: with and without looking ahead the same tokens come out, and the
+    plain decode stretches do run from schedules made ahead."""
+    from clockwork_amd.engine.llm_engine import LLMEngine
+
+    name = "A"
+    prompts = prompts_for(name, [6, 11, 3, 20, 8], seed=4)
+    lengths = [30, 7, 19, 12, 25]
+
+    def session(lookahead: bool):
+        eng = LLMEngine(EngineConfig.defaults(str(model_dirs[name]), dtype=dtype, block_size=4, num_blocks=256,
+                                              watermark=0.0, lookahead=lookahead, enable_prefix_cache=False))
+        finals = {}
+        for i in range(3):
+            eng.add_request(f"r{i}", prompt_token_ids=prompts[i], sampling_params=greedy(lengths[i]))
+        step = 0
+        while eng.has_unfinished_requests():
+            if step == 9:
+                eng.add_request("r3", prompt_token_ids=prompts[3], sampling_params=greedy(lengths[3]))
+                eng.add_request("r4", prompt_token_ids=prompts[4], sampling_params=greedy(lengths[4]))
+            if step == 15:
+                eng.abort_request("r4")
+            for out in eng.step():
+                if out.finished:
+                    finals[out.request_id] = out.token_ids
+            step += 1
+        assert eng.manager.min_free_blocks() == eng.manager.num_blocks
+        return finals, eng.stats()["lookahead_steps"], step
+
+    with_ahead, used, steps_a = session(True)
+    without, unused, steps_b = session(False)
+    assert with_ahead == without and steps_a == steps_b
+    assert unused == 0 and used >= 10
+    assert sorted(with_ahead) == ["r0", "r1", "r2", "r3"] and [len(with_ahead[f"r{i}"]) for i in range(4)] == lengths[:4]
+    # a stop token ends a request in the middle of a stretch: the step made ahead is dropped
+    stop = with_ahead["r0"][10]
+    eng = LLMEngine(EngineConfig.defaults(str(model_dirs[name]), dtype=dtype, block_size=4, num_blocks=256, watermark=0.0,
+                                          enable_prefix_cache=False))
+    eng.add_request("s", prompt_token_ids=prompts[0],
+                    sampling_params=SamplingParams(max_tokens=30, temperature=0.0, ignore_eos=True, stop_token_ids=[stop]))
+    eng.add_request("t", prompt_token_ids=prompts[1], sampling_params=greedy(20))
+    finals = {}
+    while eng.has_unfinished_requests():
+        for out in eng.step():
+            if out.finished:
+                finals[out.request_id] = (out.token_ids, out.finish_reason)
+    first = with_ahead["r0"].index(stop)
+    assert finals["s"] == (with_ahead["r0"][: first + 1], "stop")
+    assert len(finals["t"][0]) == 20 and eng.stats()["lookahead_steps"] > 0
+    assert eng.manager.min_free_blocks() == eng.manager.num_blocks
+
+
 def test_eight_staggered_requests_equal_each_alone(model_dirs):
     # tests/test_llm_engine.py:94-131: a budget of 32 tokens forces portions and mixed steps
     name = "A"

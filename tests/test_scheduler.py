@@ -346,3 +346,103 @@ def test_stats_count_admissions_and_batches():
     assert (sched.stats.num_waiting, sched.stats.num_running, sched.stats.total_prompt_tokens) == (0, 1, 5)
     engine_step(sched)
     assert sched.stats.num_scheduled_batches == 2 and sched.stats.num_running == 0
+
+
+# ------------------------------------------------------------------ one step ahead
+def portions_of(out):
+    return [(p.seq.seq_id, p.start, p.num_tokens, p.samples) for p in out.portions]
+
+
+def run_session(use_ahead: bool):
+    """Three requests of different lengths, one arriving late; returns each step's portions."""
+    sched, manager, _ = make_env(num_blocks=64, budget=16, chunked=True)
+    sched.add_seq(make_seq("a", range(5), 0.0, max_tokens=9))
+    sched.add_seq(make_seq("b", range(11), 1.0, max_tokens=4))
+    late = make_seq("c", range(3), 2.0, max_tokens=6)
+    history, ahead, used = [], None, 0
+    for step in range(40):
+        if step == 7:
+            sched.add_seq(late)
+        if ahead is not None and ahead.version == sched.version:
+            out = ahead
+            sched.commit_ahead(out)
+            used += 1
+        else:
+            out = sched.schedule()
+        if not out.portions:
+            break
+        history.append(portions_of(out))
+        # the engine looks ahead while the step runs, before its tokens are known
+        ahead = sched.schedule_ahead(out) if use_ahead else None
+        apply(sched, out)
+    assert not sched.has_unfinished()
+    assert manager.min_free_blocks() == manager.num_blocks
+    return history, used, sched.stats.num_scheduled_batches
+
+
+def test_schedule_ahead_decides_what_schedule_would():
+    plain_history, _, plain_batches = run_session(False)
+    ahead_history, used, ahead_batches = run_session(True)
+    assert ahead_history == plain_history
+    assert ahead_batches == plain_batches
+    assert used >= 5  # the plain decode stretches ran from schedules made ahead
+
+
+def test_schedule_ahead_leaves_the_hard_cases_to_schedule():
+    sched, manager, _ = make_env(num_blocks=8, budget=16, chunked=True)
+    a = make_seq("a", range(6), 0.0, max_tokens=3)
+    sched.add_seq(a)
+    out = sched.schedule()                      # the prompt: a portion, not a decode step
+    assert sched.schedule_ahead(out) is None
+    apply(sched, out)
+    out = sched.schedule()                      # first decode step; the token after it is the last (3 of 3)
+    assert portions_of(out) == [("a", 6, 1, True)]
+    ahead = sched.schedule_ahead(out)
+    assert ahead is not None and portions_of(ahead) == [("a", 7, 1, True)]
+    apply(sched, out)
+    sched.commit_ahead(ahead)
+    assert sched.schedule_ahead(ahead) is None  # max_tokens: this token ends the request
+    # somebody waits: the ordinary schedule has to look at admission
+    sched2, _, _ = make_env(num_blocks=8, budget=16, chunked=True)
+    sched2.add_seq(make_seq("x", range(4), 0.0))
+    apply(sched2, sched2.schedule())
+    out = sched2.schedule()
+    sched2.add_seq(make_seq("y", range(4), 1.0))
+    assert sched2.schedule_ahead(out) is None
+    # a schedule made ahead goes stale when a request is aborted
+    sched3, _, _ = make_env(num_blocks=8, budget=16, chunked=True)
+    sched3.add_seq(make_seq("p", range(4), 0.0))
+    sched3.add_seq(make_seq("q", range(4), 1.0))
+    apply(sched3, sched3.schedule())
+    out = sched3.schedule()
+    ahead = sched3.schedule_ahead(out)
+    assert ahead is not None
+    apply(sched3, out)
+    sched3.abort("q")
+    assert ahead.version != sched3.version
+    with pytest.raises(RuntimeError):
+        sched3.commit_ahead(ahead)
+
+
+def test_schedule_ahead_never_preempts_or_evicts():
+    # 3 pages of 4: two requests of 5 tokens hold 2 pages each? no: one page is free for one of them only
+    sched, manager, _ = make_env(num_blocks=4, budget=16, chunked=True)
+    a, b = make_seq("a", range(4), 0.0), make_seq("b", range(4), 1.0)
+    sched.add_seq(a)
+    sched.add_seq(b)
+    apply(sched, sched.schedule())              # both prompts; each holds one full page
+    out = sched.schedule()                      # decode at position 4: a second page each
+    assert len(out.portions) == 2 and manager.min_free_blocks() == 0
+    ahead = sched.schedule_ahead(out)           # position 5 lies in the pages they hold
+    assert ahead is not None
+    apply(sched, out)
+    sched.commit_ahead(ahead)
+    apply(sched, ahead)
+    for _ in range(2):                          # positions 6 and 7
+        out = sched.schedule()
+        apply(sched, out)
+    before = sched.stats.num_preempted_total
+    assert sched.schedule_ahead(out) is None    # position 8 needs a page that is not there
+    assert sched.stats.num_preempted_total == before and len(sched.running) == 2
+    out = sched.schedule()                      # the ordinary schedule preempts the later request
+    assert ids(out.preempted) == ["b"]
