@@ -39,7 +39,6 @@ struct AttnParams {
   float scale;
   float* part_o;          // [n_items, nkv * n_chunks, n_splits, ROWS, HD] unnormalised outputs
   float* part_ml;         // [n_items, nkv * n_chunks, n_splits, ROWS, 2] running max, sum
-  int* counters;          // decode kernel: one arrival counter per (item, head chunk), zero between launches
   const void* zeros;      // at least HD zero elements: what a masked key or value row is loaded from
   // decode kernel only
   int identity;           // 1: item i is request i and its one token is row i of the batch (items, cu_q unread)
@@ -386,7 +385,7 @@ CW_EXPORT int cw_attention(int rows, int dtype, const void* q, int64_t q_stride,
   const int group = nh / nkv;
   if (gh < 1 || gh > group || gh > rows || n_splits < 1 || n_splits > 65535 || window < 0) return CW_ERR_ARG;
   if (n_items == 0) return CW_OK;
-  AttnParams p;
+  AttnParams p{};
   p.q = q; p.q_stride = q_stride; p.out = out; p.out_stride = out_stride;
   p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
   p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
@@ -398,7 +397,6 @@ CW_EXPORT int cw_attention(int rows, int dtype, const void* q, int64_t q_stride,
   const int64_t n_o = need / (CW_HD + 2) * CW_HD;
   p.part_o = workspace;
   p.part_ml = workspace ? workspace + n_o : nullptr;
-  p.counters = nullptr;
   p.zeros = nullptr;
   constexpr int BN = CW_HD <= 128 ? 64 : 32;
   if (dtype == CW_F32) {
@@ -754,7 +752,7 @@ CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* ou
   if (split_keys > 0 && (int64_t)split_keys * n_splits < max_ctx) return CW_ERR_ARG;
   if (n_items == 0) return CW_OK;
   const int group = nh / nkv;
-  AttnParams p;
+  AttnParams p{};
   p.q = q; p.q_stride = q_stride; p.out = out; p.out_stride = out_stride;
   p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
   p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
@@ -768,7 +766,6 @@ CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* ou
   if ((uintptr_t)workspace & 7) return CW_ERR_ARG;
   p.part_o = workspace;
   p.part_ml = workspace ? workspace + need / (CW_HD + 2) * CW_HD : nullptr;
-  p.counters = nullptr;
   p.zeros = zeros;
   return p.bs_shift >= 0 ? launch_decode<true>(p, n_items, stream) : launch_decode<false>(p, n_items, stream);
 #else
@@ -1126,13 +1123,13 @@ CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* o
     return CW_ERR_ARG;
   if (n_items == 0) return CW_OK;
   const int group = nh / nkv;
-  AttnParams p;
+  AttnParams p{};
   p.q = q; p.q_stride = q_stride; p.out = out; p.out_stride = out_stride;
   p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
   p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
   p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.bs_shift = cw_log2_or_minus1(block_size); p.gh = group < 32 ? group : 32;
   p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = 1; p.window = window; p.scale = scale;
-  p.part_o = nullptr; p.part_ml = nullptr; p.counters = nullptr; p.zeros = zeros;
+  p.part_o = nullptr; p.part_ml = nullptr; p.zeros = zeros;
   if ((int64_t)nkv * p.n_chunks > 65535) return CW_ERR_SIZE;
   dim3 grid(n_items, nkv * p.n_chunks), block(PrefillTile<CW_HD>::NT);
   // two stages of K and V tiles, then the window of the block table
