@@ -502,17 +502,25 @@ static int launch_skinny(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W
 // (1: not worth it). The caller allocates [splits, M, N] float32 and passes mode 3.
 CW_EXPORT int cw_gemm_bf16_skinny_ksplits(int M, int N, int K) {
   const int tiles = (N + 15) / 16;
-  if (M > 64 || tiles > 128 || K < 4096) return 1;
+  if (M > 64 || tiles > 128) return 1;
+  if (M > 16) {
+    // Only the streaming kernel takes partial sums of more than 16 rows, and the alternative is a
+    // library product that leaves most compute units idle on so narrow an output: split K just
+    // far enough that every compute unit gets a tile, down to 8 steps of 32 per split.
+    int s = (cw_num_compute_units() + tiles - 1) / tiles;
+    if (K >= 4096 && s < 512 / tiles) s = 512 / tiles;
+    if (s > 8) s = 8;
+    while (s > 1 && K / s < 256) --s;
+    int mt, spw, n_tiles;
+    dim3 grid;
+    if (s <= 1 || !plan_stream(3, M, N, K, s, &mt, &spw, &grid, &n_tiles)) return 1;
+    return s;
+  }
+  if (K < 4096) return 1;
   int s = 512 / tiles;  // about two workgroups per compute unit
   if (s > 8) s = 8;
   while (s > 1 && K / s < 1024) --s;
-  if (s < 1) s = 1;
-  if (M > 16) {  // only the streaming kernel takes partial sums of more than 16 rows
-    int mt, spw, n_tiles;
-    dim3 grid;
-    if (s == 1 || !plan_stream(3, M, N, K, s, &mt, &spw, &grid, &n_tiles)) return 1;
-  }
-  return s;
+  return s < 1 ? 1 : s;
 }
 
 // 1 if cw_gemm_bf16_skinny streams the weights once for this shape at full speed: every shape
@@ -614,13 +622,13 @@ CW_EXPORT int cw_gemm_bf16_skinny(int mode, const void* X, int64_t ldx, const vo
 // every rotary pair (half-split pairing, full rotary dimension) end up in one workgroup. The
 // epilogue adds the bias, rotates by float32(pos) * inv_freq[i] and writes q to ``q_out``
 // [M, nh * hd], rotated k and plain v to their cache rows ``slots[m]`` ([rows, nkv, hd]).
-template <int WAVES>
+template <int WAVES, int MT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_qkv_rope_bf16_kernel(
     const bf16_t* __restrict__ X, int64_t ldx, const bf16_t* __restrict__ W, const void* __restrict__ bias,
     int bias_f32, const int* __restrict__ positions, const int* __restrict__ slots,
     const float* __restrict__ inv_freq, bf16_t* __restrict__ q_out, bf16_t* __restrict__ k_cache,
     bf16_t* __restrict__ v_cache, int64_t cache_rows, int M, int K, int nh, int nkv, int hd) {
-  __shared__ float red[WAVES][256];
+  __shared__ float red[WAVES][MT * 256];  // [wave][token tile][tile row][token]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, s = lane >> 4;
   const int half = hd / 2;
@@ -631,64 +639,75 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_qkv_rope_bf16_kernel(
   // weight row of this lane inside the head
   const int row_in_head = is_v ? tile * 16 + r : (r < 8 ? tile * 8 + r : half + tile * 8 + (r - 8));
   const bf16_t* wrow = W + ((int64_t)head * hd + row_in_head) * K;
-  const bool xok = r < M;
-  const bf16_t* xrow = X + (int64_t)(xok ? r : 0) * ldx;
+  bool xok[MT];
+  const bf16_t* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    xok[mt] = mt * 16 + r < M;
+    xrow[mt] = X + (int64_t)(xok[mt] ? mt * 16 + r : 0) * ldx;
+  }
 
-  f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
   bf16x8_t zero;
 #pragma unroll
   for (int e = 0; e < 8; ++e) zero[e] = (__bf16)0.0f;
   const int k_steps = (K + 31) / 32;
-  constexpr int U = 4;
+  constexpr int U = MT == 1 ? 4 : 2;
   for (int ks0 = wave * U; ks0 < k_steps; ks0 += WAVES * U) {
-    bf16x8_t wf[U], xf[U];
+    bf16x8_t wf[U], xf[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k = (ks0 + u) * 32 + s * 8;
       const bool kok = (ks0 + u) < k_steps && k + 8 <= K;
       wf[u] = kok ? *reinterpret_cast<const bf16x8_t*>(wrow + k) : zero;
-      xf[u] = (kok && xok) ? *reinterpret_cast<const bf16x8_t*>(xrow + k) : zero;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        xf[u][mt] = (kok && xok[mt]) ? *reinterpret_cast<const bf16x8_t*>(xrow[mt] + k) : zero;
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u], acc, 0, 0, 0);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u][mt], acc[mt], 0, 0, 0);
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) red[wave][(4 * s + i) * 16 + r] = acc[i];
-  __syncthreads();
-  // 256 values [tile row][token]; thread t < 256 sums value t over the waves
-  {
-    const int idx = threadIdx.x;
-    if (idx < 256) {
-      float sum = red[0][idx];
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int w = 1; w < WAVES; ++w) sum += red[w][idx];
-      red[0][idx] = sum;
-    }
+    for (int i = 0; i < 4; ++i) red[wave][mt * 256 + (4 * s + i) * 16 + r] = acc[mt][i];
+  __syncthreads();
+  // MT * 256 values [token tile][tile row][token]; each is summed over the waves by one thread
+  for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {
+    float sum = red[0][idx];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) sum += red[w][idx];
+    red[0][idx] = sum;
   }
   __syncthreads();
   auto bias_at = [&](int col) -> float {
     if (bias == nullptr) return 0.0f;
     return bias_f32 ? ((const float*)bias)[col] : __bfloat162float(((const bf16_t*)bias)[col]);
   };
+  auto summed = [&](int row, int m) -> float { return red[0][(m >> 4) * 256 + row * 16 + (m & 15)]; };
   if (is_v) {
     // idx -> (token m, row j), j fastest: 16 consecutive elements of a cache row
-    for (int idx = threadIdx.x; idx < 256; idx += WAVES * 64) {
+    for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {
       const int j = idx & 15, m = idx >> 4;
       if (m >= M) continue;
       const int64_t slot = slots[m];
       if (slot < 0 || slot >= cache_rows) continue;
       const int d = tile * 16 + j;
-      const float v = red[0][j * 16 + m] + bias_at(head * hd + d);
+      const float v = summed(j, m) + bias_at(head * hd + d);
       v_cache[(slot * nkv + (head - nh - nkv)) * hd + d] = __float2bfloat16(v);
     }
   } else {
     // idx -> (token m, pair p): elements i = tile * 8 + p and i + half
-    for (int idx = threadIdx.x; idx < 128; idx += WAVES * 64) {
+    for (int idx = threadIdx.x; idx < MT * 128; idx += WAVES * 64) {
       const int p = idx & 7, m = idx >> 3;
       if (m >= M) continue;
       const int i = tile * 8 + p;
-      const float a = red[0][p * 16 + m] + bias_at(head * hd + i);
-      const float b = red[0][(p + 8) * 16 + m] + bias_at(head * hd + half + i);
+      const float a = summed(p, m) + bias_at(head * hd + i);
+      const float b = summed(p + 8, m) + bias_at(head * hd + half + i);
       float sn, cs;
       sincosf((float)positions[m] * inv_freq[i], &sn, &cs);
       const bf16_t oa = __float2bfloat16(a * cs - b * sn), ob = __float2bfloat16(b * cs + a * sn);
@@ -707,14 +726,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_qkv_rope_bf16_kernel(
   }
 }
 
-// x [M <= 16, K] bfloat16, W [(nh + 2 nkv) * hd, K] bfloat16 (q heads, k heads, v heads), hd a
+// x [M <= 64, K] bfloat16, W [(nh + 2 nkv) * hd, K] bfloat16 (q heads, k heads, v heads), hd a
 // multiple of 16, rotary dimension == hd. bias: nullptr, bfloat16 or float32 [(nh + 2 nkv) * hd].
 CW_EXPORT int cw_gemm_qkv_rope_bf16(const void* X, int64_t ldx, const void* W, const void* bias,
                                     int bias_f32, const int* positions, const int* slots,
                                     const float* inv_freq, void* q_out, void* k_cache, void* v_cache,
                                     int64_t cache_rows, int M, int K, int nh, int nkv, int hd,
                                     hipStream_t stream) {
-  if (M < 0 || M > 16 || K <= 0 || nh <= 0 || nkv <= 0 || hd <= 0 || (hd & 15)) return CW_ERR_ARG;
+  if (M < 0 || M > 64 || K <= 0 || nh <= 0 || nkv <= 0 || hd <= 0 || (hd & 15)) return CW_ERR_ARG;
   if ((K & 7) || (ldx & 7) || ldx < K || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return CW_ERR_ARG;
   if (!positions || !slots || !inv_freq || !q_out || !k_cache || !v_cache) return CW_ERR_ARG;
   if (M == 0) return CW_OK;
@@ -722,13 +741,22 @@ CW_EXPORT int cw_gemm_qkv_rope_bf16(const void* X, int64_t ldx, const void* W, c
   dim3 grid(tiles);
   const bf16_t* x = (const bf16_t*)X;
   const bf16_t* w = (const bf16_t*)W;
-#define CW_QKV(WAVES_)                                                                              \
-  hipLaunchKernelGGL((gemm_qkv_rope_bf16_kernel<WAVES_>), grid, dim3(WAVES_ * 64), 0, stream, x, ldx, \
-                     w, bias, bias_f32, positions, slots, inv_freq, (bf16_t*)q_out, (bf16_t*)k_cache, \
+#define CW_QKV(WAVES_, MT_)                                                                              \
+  hipLaunchKernelGGL((gemm_qkv_rope_bf16_kernel<WAVES_, MT_>), grid, dim3(WAVES_ * 64), 0, stream, x, ldx, \
+                     w, bias, bias_f32, positions, slots, inv_freq, (bf16_t*)q_out, (bf16_t*)k_cache,    \
                      (bf16_t*)v_cache, cache_rows, M, K, nh, nkv, hd)
-  if (tiles <= 256 && K >= 1024) CW_QKV(16);
-  else if (K >= 512) CW_QKV(8);
-  else CW_QKV(4);
+  if (M > 32) {  // the reduction buffer is WAVES * MT KB
+    if (K >= 512) CW_QKV(8, 4);
+    else CW_QKV(4, 4);
+  } else if (M > 16) {
+    if (tiles <= 256 && K >= 1024) CW_QKV(16, 2);
+    else if (K >= 512) CW_QKV(8, 2);
+    else CW_QKV(4, 2);
+  } else {
+    if (tiles <= 256 && K >= 1024) CW_QKV(16, 1);
+    else if (K >= 512) CW_QKV(8, 1);
+    else CW_QKV(4, 1);
+  }
 #undef CW_QKV
   return cw_launch_status();
 }

@@ -381,7 +381,7 @@ def library_tuning():
 
 def qkv_rope_fused_supported(x: torch.Tensor, weight: torch.Tensor, rotary_dim: int, hd: int) -> bool:
     """The fused q/k/v product + rotary + cache write takes few bfloat16 rows and a full rotary dimension."""
-    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[0] <= STREAM_MAX_ROWS
             and x.shape[1] % 8 == 0 and rotary_dim == hd and hd % 16 == 0)
 
 

@@ -147,7 +147,7 @@ def test_rope_kv_write(dtype, nh, nkv, hd, rotary, theta):
             assert torch.all(kc[s] == 100.0) and torch.all(vc[s] == 100.0)
 
 
-@pytest.mark.parametrize("M", [1, 8, 16])
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
 @pytest.mark.parametrize("nh,nkv,hd,K,theta,bias_dtype", [(12, 2, 128, 1536, 1e6, torch.bfloat16), (6, 1, 32, 192, 1e6, torch.float32),
                                                          (4, 2, 16, 64, 1e4, torch.bfloat16), (3, 3, 48, 80, 5e4, None)])
 def test_fused_qkv_rope_cache_write(M, nh, nkv, hd, K, theta, bias_dtype):
@@ -159,11 +159,11 @@ def test_fused_qkv_rope_cache_write(M, nh, nkv, hd, K, theta, bias_dtype):
     w = (torch.randn(width, K, device=DEV) / K ** 0.5).to(torch.bfloat16)
     bias = None if bias_dtype is None else (0.5 * torch.randn(width, device=DEV)).to(bias_dtype)
     positions = torch.randint(0, 5000, (M,), dtype=torch.int32, device=DEV)
-    slots = torch.randperm(40, device=DEV)[:M].to(torch.int32)
+    slots = torch.randperm(80, device=DEV)[:M].to(torch.int32)
     if M > 2:
         slots[1] = -1  # a padding row of a captured decode batch: no cache row
-    kc = torch.full((40, nkv, hd), 100.0, device=DEV, dtype=torch.bfloat16)
-    vc = torch.full((40, nkv, hd), 100.0, device=DEV, dtype=torch.bfloat16)
+    kc = torch.full((80, nkv, hd), 100.0, device=DEV, dtype=torch.bfloat16)
+    vc = torch.full((80, nkv, hd), 100.0, device=DEV, dtype=torch.bfloat16)
     inv_freq = plain.inv_frequencies(hd, theta).to(DEV)
     q = ops.qkv_rope_fused(x, w, bias, positions, slots, inv_freq, nh, nkv, hd, kc, vc)
 
@@ -183,7 +183,7 @@ def test_fused_qkv_rope_cache_write(M, nh, nkv, hd, K, theta, bias_dtype):
         written.add(sl)
         torch.testing.assert_close(kc[sl].float().cpu(), k_ref[i], **t)
         torch.testing.assert_close(vc[sl].float().cpu(), v_ref[i], **t)
-    for sl in range(40):
+    for sl in range(80):
         if sl not in written:
             assert torch.all(kc[sl] == 100.0) and torch.all(vc[sl] == 100.0)
 
