@@ -33,3 +33,17 @@ WIDE = dict(
     num_key_value_heads=2, intermediate_size=4360, rms_norm_eps=2e-6, rope_theta=300000.0,
     tie_word_embeddings=False,
 )
+
+# One layer each of the larger models the engine is meant for (Qwen2.5-7B and -32B layer sizes, a
+# small vocabulary): products whose K does not fit the streaming kernel's registers, groups of 7
+# and 5 query heads per key head, 18944 / 27648-wide feed-forwards.
+LAYER_7B = dict(
+    model_type="qwen2", vocab_size=1501, hidden_size=3584, num_hidden_layers=1, num_attention_heads=28,
+    num_key_value_heads=4, intermediate_size=18944, rms_norm_eps=1e-6, rope_theta=1000000.0,
+    tie_word_embeddings=False,
+)
+LAYER_32B = dict(
+    model_type="qwen2", vocab_size=1302, hidden_size=5120, num_hidden_layers=1, num_attention_heads=40,
+    num_key_value_heads=8, intermediate_size=27648, rms_norm_eps=1e-6, rope_theta=1000000.0,
+    tie_word_embeddings=False,
+)

@@ -96,6 +96,50 @@ def test_wide_layers_take_the_streaming_and_fused_paths(tmp_path, mode):
     assert not runner.manager.live_requests()
 
 
+@pytest.mark.parametrize("which", ["LAYER_7B", "LAYER_32B"])
+def test_layers_of_the_larger_models(tmp_path, which):
+    """One layer of the 7B and of the 32B shape, bfloat16: a prompt in two portions, then tokens
+    one by one beside a second request's prompt, against the plain implementation."""
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests import configs
+
+    config = getattr(configs, which)
+    model_dir = write_random_model(tmp_path / which, config, 7)
+    gen = torch.Generator().manual_seed(13)
+    requests = {f"m{i}": torch.randint(0, config["vocab_size"], (n,), generator=gen).tolist() for i, n in enumerate([45, 21])}
+    plain = PlainQwen2(model_dir)
+    want = {rid: plain.logits(toks) for rid, toks in requests.items()}
+    a, b = requests["m0"], requests["m1"]
+    steps = [
+        {"entries": [{"id": "m0", "tokens": a[:30], "want": list(range(30))}], "end": []},
+        {"entries": [{"id": "m0", "tokens": a[30:37], "want": list(range(7))}], "end": []},
+    ]
+    for p in range(37, 45):
+        entry = [{"id": "m0", "tokens": a[p : p + 1], "want": [0]}]
+        if p == 39:
+            entry.append({"id": "m1", "tokens": b[:17], "want": list(range(17))})
+        if p > 39 and 17 + (p - 40) < len(b):
+            q = 17 + (p - 40)
+            entry.append({"id": "m1", "tokens": b[q : q + 1], "want": [0]})
+        steps.append({"entries": entry, "end": []})
+    steps[-1]["end"] = ["m0", "m1"]
+    runner = replay.make_runner(model_dir, "bfloat16", 16, 16)
+    got = replay.run_trace(runner, steps)
+    assert len(got) == 45 + 17 + 4
+    # Rounding every activation to 8 bits gives each logit an error of about a hundredth of the
+    # logits' own scale (measured: 0.95% and 1.0% for the two shapes, the same at every position
+    # and in every kind of step), and that scale grows with the width (1.2 and 1.4 here, 0.15 for
+    # the tiny models, whose bound is absolute). So the bound is relative to the scale: the root
+    # mean square of the errors within 2% of it, the largest of the 100,000 within 10%. A wrong
+    # key, mask or weight row moves logits by the scale itself.
+    scale = torch.cat([w.flatten() for w in want.values()]).square().mean().sqrt().item()
+    errors = torch.stack([row - want[rid][pos] for (rid, pos), row in sorted(got.items())])
+    assert not torch.isnan(errors).any()
+    rms, worst = errors.square().mean().sqrt().item(), errors.abs().max().item()
+    print(f"{which} bfloat16: logits' scale {scale:.3f}, rms error {rms:.3e}, largest {worst:.3e}")
+    assert rms < 2e-2 * scale and worst < 1e-1 * scale
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_and_long_decoding(model_dirs, dtype):
     """The first tokens of a sequence (one-token prompt, then decoding from position 1) and a
