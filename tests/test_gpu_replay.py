@@ -60,6 +60,23 @@ def test_replay_matches_plain(model_dirs, name, dtype, mode):
     assert runner.manager.min_free_blocks() == runner.manager.num_blocks
 
 
+def test_wide_layers_in_float32(tmp_path):
+    """The same wide model in true float32, mixed batches: the 1e-5 bar at layer sizes that the
+    tiny models do not reach (a feed-forward 4360 wide, 1024-element rows, head size 128)."""
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests.configs import WIDE
+
+    model_dir = write_random_model(tmp_path / "wide", WIDE, 3)
+    gen = torch.Generator().manual_seed(11)
+    requests = {f"w{i}": torch.randint(0, WIDE["vocab_size"], (n,), generator=gen).tolist() for i, n in enumerate([40, 70, 55])}
+    plain = PlainQwen2(model_dir)
+    want = {rid: plain.logits(toks) for rid, toks in requests.items()}
+    runner = replay.make_runner(model_dir, "float32", 16, replay.pages_needed(requests, 3, 16))
+    got = replay.run_trace(runner, replay.mixed(requests))
+    worst = replay.compare(got, want, **TOL["float32"])
+    print(f"wide float32 mixed: largest error {worst:.3e}")
+
+
 @pytest.mark.parametrize("mode", ["prefill_then_decode", "mixed"])
 def test_wide_layers_take_the_streaming_and_fused_paths(tmp_path, mode):
     """A model with layers as wide as real ones, so that decode steps run the kernels that tiny
