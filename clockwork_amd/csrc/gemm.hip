@@ -232,8 +232,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
   }
 }
 
-// The same product when a wave's share of the K loop is short (at most 8 steps of 32): the wave
-// keeps its x fragments (MT tiles of 16 tokens) in registers for good, so only weights move.
+// The same product with the x fragments of a wave's whole share of the K loop (up to 24 steps of
+// 32, as many as its registers hold beside MT tiles of 16 tokens) kept in registers for good, so
+// that only weights move.
 // A workgroup walks over row tiles blockIdx.x, blockIdx.x + gridDim.x, ...; the weights of its
 // next tile are on their way while the current one is reduced through LDS (one barrier per tile
 // while the reduction buffer can be doubled, two for MT = 4). Loads are never conditional: a row
@@ -252,12 +253,18 @@ struct StreamNormIn {
   float eps;
 };
 
+// Weight fragments of a tile are fetched CH steps at a time (two sets in flight), while the x
+// fragments of all SPW steps stay in registers: a long K costs registers for x only.
+constexpr int cw_stream_chunk(int spw) { return spw <= 8 ? spw : (spw <= 12 ? spw / 2 : spw / 4); }
+
 template <int MODE, int WAVES, int SPW, int MT, bool NORM = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16_t* __restrict__ X, int64_t ldx,
                                                                const bf16_t* __restrict__ W,
                                                                void* __restrict__ C, int64_t ldc,
                                                                int M, int N, int K, int n_tiles, StreamNormIn nin) {
   constexpr int NBUF = MT <= 2 ? 2 : 1;
+  constexpr int CH = cw_stream_chunk(SPW), NC = SPW / CH;
+  static_assert(SPW % CH == 0, "the steps of a wave are whole chunks");
   __shared__ float red[NBUF][WAVES][MT * 256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, s = lane >> 4;
@@ -282,26 +289,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
   // the first tile's weights are requested before anything else: x, and with NORM the norm's
   // statistics, are fetched in their shadow
   int tile = blockIdx.x;
-  bf16x8_t cur[SPW], nxt[SPW];
-  {
-    const bf16_t* w = wrow(tile);
+  bf16x8_t cur[CH], nxt[CH];
+  const bf16_t* w_tile = wrow(tile);
 #pragma unroll
-    for (int u = 0; u < SPW; ++u) cur[u] = *reinterpret_cast<const bf16x8_t*>(w + koff[u]);
-  }
+  for (int u = 0; u < CH; ++u) cur[u] = *reinterpret_cast<const bf16x8_t*>(w_tile + koff[u]);
 
   bf16x8_t xf[SPW][MT];
   if constexpr (NORM) {
-    static_assert(MT == 1, "the fused norm serves one tile of tokens");
+    static_assert(MT == 1 && SPW <= 4, "the fused norm serves one tile of tokens and rows of up to 2048 elements");
     __shared__ float ssq[WAVES][16];
-    float v[SPW][8], wv[SPW][8];
+    float v[SPW][8], wv[SPW][8];  // resid + delta and the norm weight at the lane's elements
     float ss = 0.0f;
 #pragma unroll
     for (int u = 0; u < SPW; ++u) {
       const int k = (wave * SPW + u) * 32 + s * 8;
-      const bool kok = k + 8 <= K;
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[u][e] = wv[u][e] = 0.0f;
-      if (kok && r < M) {
+      if (k + 8 <= K && r < M) {
         const float4 a = *reinterpret_cast<const float4*>(nin.resid + (int64_t)r * K + k);
         const float4 b = *reinterpret_cast<const float4*>(nin.resid + (int64_t)r * K + k + 4);
         const bf16x8_t d = *reinterpret_cast<const bf16x8_t*>(nin.delta + (int64_t)r * K + k);
@@ -348,18 +352,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
   }
   int buf = 0;
   for (; tile < n_tiles; tile += gridDim.x) {
-    {
-      const bf16_t* w = wrow(min(tile + (int)gridDim.x, n_tiles - 1));
-#pragma unroll
-      for (int u = 0; u < SPW; ++u) nxt[u] = *reinterpret_cast<const bf16x8_t*>(w + koff[u]);
-    }
+    const bf16_t* w_next = wrow(min(tile + (int)gridDim.x, n_tiles - 1));
     f32x4_t acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int u = 0; u < SPW; ++u)
+    for (int c = 0; c < NC; ++c) {
+      // the chunk after this one: of this tile, or the first of the workgroup's next tile
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], xf[u][mt], acc[mt], 0, 0, 0);
+      for (int u = 0; u < CH; ++u)
+        nxt[u] = *reinterpret_cast<const bf16x8_t*>((c + 1 < NC ? w_tile + koff[(c + 1) * CH + u] : w_next + koff[u]));
+#pragma unroll
+      for (int u = 0; u < CH; ++u)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], xf[c * CH + u][mt], acc[mt], 0, 0, 0);
+#pragma unroll
+      for (int u = 0; u < CH; ++u) cur[u] = nxt[u];
+    }
+    w_tile = w_next;
     // lane (r, s) holds weight rows 4s..4s+3 of token r of tile mt -> red[buf][wave][mt][row][token]
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -395,8 +406,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
       }
     }
     if (NBUF == 1) __syncthreads();
-#pragma unroll
-    for (int u = 0; u < SPW; ++u) cur[u] = nxt[u];
     buf = (buf + 1) % NBUF;
   }
 }
@@ -414,7 +423,12 @@ static int cw_num_compute_units() {
 
 // Do a wave's x fragments, two sets of weight fragments and the accumulators fit its registers?
 constexpr bool cw_stream_fits(int waves, int spw, int mt) {
-  return spw * mt * 4 + spw * 8 + mt * 4 <= (waves == 16 ? 100 : 220);
+  return spw * mt * 4 + cw_stream_chunk(spw) * 8 + mt * 4 <= (waves == 16 ? 100 : 220);
+}
+
+// Steps per wave the kernel is built for: every count up to 8, then even counts, then multiples of 4.
+constexpr int cw_stream_round_spw(int spw) {
+  return spw <= 8 ? spw : (spw <= 12 ? (spw + 1) / 2 * 2 : (spw + 3) / 4 * 4);
 }
 
 template <int MODE, int WAVES, int SPW, int MT>
@@ -436,6 +450,7 @@ static int launch_stream(int spw, dim3 grid, const bf16_t* X, int64_t ldx, const
   case SPW_: return launch_stream_one<MODE, WAVES, SPW_, MT>(grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream)
   switch (spw) {
     CW_STREAM(1); CW_STREAM(2); CW_STREAM(3); CW_STREAM(4); CW_STREAM(5); CW_STREAM(6); CW_STREAM(7); CW_STREAM(8);
+    CW_STREAM(10); CW_STREAM(12); CW_STREAM(16); CW_STREAM(20); CW_STREAM(24);
     default: return CW_ERR_SIZE;
   }
 #undef CW_STREAM
@@ -456,8 +471,8 @@ static bool plan_stream(int mode, int M, int N, int K, int k_splits, int* mt, in
   *n_tiles = mode == 2 ? (N / 2 + 7) / 8 : (N + 15) / 16;
   const int waves = mode == 3 ? 8 : 16;
   *mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  *spw = (k_steps + k_splits * waves - 1) / (k_splits * waves);
-  if (M > 64 || *spw > 8 || !cw_stream_fits(waves, *spw, *mt) || (mode != 3 && k_steps < 2 * waves)) return false;
+  *spw = cw_stream_round_spw((k_steps + k_splits * waves - 1) / (k_splits * waves));
+  if (M > 64 || *spw > 24 || !cw_stream_fits(waves, *spw, *mt) || (mode != 3 && k_steps < 2 * waves)) return false;
   // tiles per workgroup: one workgroup on every compute unit (a second round of these large
   // workgroups costs more than it brings), each with the same share
   // (up to 16 rows the one-tile kernels are as fast below two rounds; beyond, the alternative
@@ -502,8 +517,10 @@ static int launch_skinny(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W
 // (1: not worth it). The caller allocates [splits, M, N] float32 and passes mode 3.
 CW_EXPORT int cw_gemm_bf16_skinny_ksplits(int M, int N, int K) {
   const int tiles = (N + 15) / 16;
-  if (M > 64 || tiles > 128) return 1;
+  const int k_steps = (K + 31) / 32;
+  if (M > 64 || tiles > 512) return 1;
   if (M > 16) {
+    if (tiles > 128) return 1;
     // Only the streaming kernel takes partial sums of more than 16 rows, and the alternative is a
     // library product that leaves most compute units idle on so narrow an output: split K just
     // far enough that every compute unit gets a tile, down to 8 steps of 32 per split.
@@ -517,8 +534,11 @@ CW_EXPORT int cw_gemm_bf16_skinny_ksplits(int M, int N, int K) {
     return s;
   }
   if (K < 4096) return 1;
-  int s = 512 / tiles;  // about two workgroups per compute unit
+  int s = 512 / tiles;  // about two workgroups per compute unit,
   if (s > 8) s = 8;
+  const int for_registers = (k_steps + 8 * 16 - 1) / (8 * 16);  // and at most 16 steps for each of 8 waves
+  if (s < for_registers) s = for_registers;
+  if (s > 16) s = 16;
   while (s > 1 && K / s < 1024) --s;
   return s < 1 ? 1 : s;
 }
@@ -538,7 +558,11 @@ CW_EXPORT int cw_gemm_bf16_skinny_fast(int mode, int M, int N, int K) {
 CW_EXPORT int cw_gemm_bf16_swiglu_normed_ok(int M, int N, int K) {
   int mt, spw, n_tiles;
   dim3 grid;
-  return M >= 1 && M <= 16 && !(N & 1) && !(K & 7) && plan_stream(2, M, N, K, 1, &mt, &spw, &grid, &n_tiles) ? 1 : 0;
+  // rows of up to 2048 elements: a lane holds its share of a row in registers over the statistics
+  return M >= 1 && M <= 16 && !(N & 1) && !(K & 7) && plan_stream(2, M, N, K, 1, &mt, &spw, &grid, &n_tiles) &&
+                 spw <= 4
+             ? 1
+             : 0;
 }
 
 // y[m, i] = silu(gate_i . x_m) * (up_i . x_m) with x = rmsnorm(resid + delta) * norm_weight made
@@ -563,7 +587,7 @@ CW_EXPORT int cw_gemm_bf16_swiglu_normed(const float* resid, const void* delta, 
                          (const bf16_t*)nullptr, (int64_t)K, (const bf16_t*)W, C, ldc, M, N, K, n_tiles, nin); \
     break
   switch (spw) {
-    CW_NORMED(1); CW_NORMED(2); CW_NORMED(3); CW_NORMED(4); CW_NORMED(5); CW_NORMED(6); CW_NORMED(7); CW_NORMED(8);
+    CW_NORMED(1); CW_NORMED(2); CW_NORMED(3); CW_NORMED(4);
     default: return CW_ERR_SIZE;
   }
 #undef CW_NORMED
