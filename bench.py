@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16] [--shape 1.5b]
 
 Default workload: the layer sizes of Qwen2.5-1.5B with random weights (seed 2), bfloat16,
 8 requests that each hold a 2048-token prompt, context limit 4096, pages of 16 tokens. A
@@ -26,7 +26,13 @@ QWEN25_1P5B = dict(
     rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True, hidden_act="silu",
     use_sliding_window=False, max_position_embeddings=32768,
 )
-FULL_LAYERS = QWEN25_1P5B["num_hidden_layers"]
+# the other layer shapes the engine is meant for (``--shape``); the default run and the recorded
+# numbers are the 1.5B shape
+QWEN25_7B = dict(QWEN25_1P5B, vocab_size=152064, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+                 intermediate_size=18944, tie_word_embeddings=False)
+QWEN25_32B = dict(QWEN25_1P5B, vocab_size=152064, hidden_size=5120, num_hidden_layers=64, num_attention_heads=40,
+                  num_key_value_heads=8, intermediate_size=27648, tie_word_embeddings=False)
+SHAPES = {"1.5b": ("Qwen2.5-1.5B", QWEN25_1P5B), "7b": ("Qwen2.5-7B", QWEN25_7B), "32b": ("Qwen2.5-32B", QWEN25_32B)}
 PROMPT_LEN = 2048
 CONTEXT = 4096
 BLOCK = 16
@@ -45,7 +51,10 @@ def build_runner(args):
     from clockwork_amd.registry import resolve_architecture
     from clockwork_amd.weights.random_init import RandomSource
 
-    config = dict(QWEN25_1P5B, num_hidden_layers=args.layers)
+    config = dict(SHAPES[args.shape][1])
+    if args.layers is not None:
+        config["num_hidden_layers"] = args.layers
+    args.layers = config["num_hidden_layers"]
     arch = resolve_architecture(config)
     mcfg = arch.parse_config(config)
     spec = arch.build_spec(mcfg)
@@ -137,7 +146,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (both numbers are recorded)")
+    ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes: the 1.5B shape is the recorded benchmark")
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--no-tune", action="store_true", help="leave the matrix library's kernel choice at its default")
@@ -161,7 +171,7 @@ def main() -> int:
     achieved = step_bytes / (elapsed / args.steps) / 1e9
 
     record = {
-        "metric": "decode tok/s, Qwen2.5-1.5B shape, batch 8, 2048-token prompts",
+        "metric": f"decode tok/s, {SHAPES[args.shape][0]} shape, batch {args.batch}, 2048-token prompts",
         "value": round(value, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -174,9 +184,9 @@ def main() -> int:
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: uniform random token ids, random weights (seed 2)",
         "config": {
-            "model": "Qwen2.5-1.5B shape (random weights)",
+            "model": f"{SHAPES[args.shape][0]} shape (random weights)",
             "layers": args.layers,
-            "layers_of_full_model": FULL_LAYERS,
+            "layers_of_full_model": SHAPES[args.shape][1]["num_hidden_layers"],
             "hidden": runner.spec.info["hidden"],
             "heads": runner.spec.info["heads"],
             "kv_heads": runner.spec.info["kv_heads"],
