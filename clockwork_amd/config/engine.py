@@ -28,6 +28,9 @@ class ModelConfig:
     # at start-up, let the matrix library time its kernels for the products of a full prefill
     # portion and of the wide decode batches and keep the fastest (bfloat16 only)
     tune_products: bool = False
+    # run the large bfloat16 products on this package's own tiled kernel instead of the matrix
+    # library (slower; for runs that must not depend on the library). Process-wide.
+    hip_products: bool = False
 
     def torch_dtype(self):
         import torch

@@ -34,7 +34,7 @@ FLAGS = [
     # hipcc -O3 forms packed float32 instructions by itself; they are kept out of these kernels
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
-PLAIN_SOURCES = {"core": "core.hip", "gemm": "gemm.hip", "sampling": "sampling.hip"}
+PLAIN_SOURCES = {"core": "core.hip", "gemm": "gemm.hip", "gemm_tile": "gemm_tile.hip", "sampling": "sampling.hip"}
 ATTENTION_SOURCE = "attention.hip"
 # head sizes compiled by build_all: the tests' models, the kernel tests and the benchmark's
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 160, 224, 256)

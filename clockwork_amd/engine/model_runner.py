@@ -47,6 +47,7 @@ class ModelRunner:
             raise ValueError(f"device {cfg.model.device!r}: this engine runs on the GPU only")
         self.device = require_gpu()
         self.dtype = cfg.model.torch_dtype()
+        ops.use_hip_products(cfg.model.hip_products)  # process-wide: the runner made last decides
         self.config_dict = config_dict if config_dict is not None else read_config_json(cfg.model.model)
         self.arch = resolve_architecture(self.config_dict)
         self.model_config = self.arch.parse_config(self.config_dict)

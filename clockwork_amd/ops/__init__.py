@@ -64,7 +64,7 @@ def _load(name: str, head_dim: int | None = None) -> ctypes.CDLL:
 
 def preload(head_dims) -> None:
     """Build (side by side, if several are missing) and load what a model with these head sizes runs."""
-    jobs = [("core", None), ("gemm", None), ("sampling", None)]
+    jobs = [("core", None), ("gemm", None), ("gemm_tile", None), ("sampling", None)]
     jobs += [("attention", int(hd)) for hd in sorted(set(head_dims))]
     build.ensure_many(jobs)
     for name, hd in jobs:
@@ -94,6 +94,9 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_gemm_bf16_swiglu_normed_ok": [I, I, I],
             "cw_gemm_bf16_swiglu_normed": [P, P, P, I, F, P, P, L, I, I, I, P],
             "cw_gemm_qkv_rope_bf16": [P, L, P, P, I, P, P, P, P, P, P, L, I, I, I, I, I, P],
+        },
+        "gemm_tile": {
+            "cw_gemm_bf16_tiled": [I, P, L, P, P, I, P, L, I, I, I, P],
         },
         "sampling": {
             "cw_argmax_chunks": [I],
@@ -345,7 +348,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
             _check(lib.cw_gemm_bf16_skinny(1 if want_f32 else 0, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, _stream()),
                    "gemm_bf16_skinny")
             return out
-    y = torch.mm(x, weight.t()) if bias is None else torch.addmm(bias, x, weight.t())
+    if HIP_PRODUCTS and K % 8 == 0 and x.is_contiguous():
+        y = linear_tiled(x, weight, bias)
+    else:
+        y = torch.mm(x, weight.t()) if bias is None else torch.addmm(bias, x, weight.t())
     if out_dtype == torch.float32:
         out = torch.empty((M, N), dtype=torch.float32, device=x.device)
         _check(_load("core").cw_bf16_to_f32(_ptr(y), _ptr(out), M * N, _stream()), "bf16_to_f32")
@@ -353,11 +359,45 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
     return y
 
 
+# True: products of many bfloat16 rows go through this package's own LDS-tiled kernel instead of
+# the library (about half as fast on an MI355X; for a run that must not depend on the library).
+# Set through ``use_hip_products`` / the model section's ``hip_products``.
+HIP_PRODUCTS = False
+
+
+def use_hip_products(on: bool) -> None:
+    global HIP_PRODUCTS
+    HIP_PRODUCTS = bool(on)
+
+
 # up to this many rows every product goes through the weight-streaming kernels
 SKINNY_MAX_ROWS = 16
 # up to this many rows the shapes that the persistent streaming kernel takes do (the library
 # product is faster for the others, measured)
 STREAM_MAX_ROWS = 64
+
+
+def linear_tiled(x: torch.Tensor, weight: torch.Tensor, bias=None, swiglu: bool = False) -> torch.Tensor:
+    """y = x @ weight.T (+ bias), or with ``swiglu`` silu(x @ gate.T) * (x @ up.T) for weight =
+    [gate; up], through the LDS-tiled matrix-core kernel for many bfloat16 rows (csrc/gemm_tile.hip).
+    The rows of x may have a stride (a slice of a wider buffer)."""
+    _gpu(weight, bias)
+    _need(x.is_cuda and x.dim() == 2, "x must be a 2-d tensor on the GPU")
+    M, K = x.shape
+    N = weight.shape[0]
+    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "the tiled product is bfloat16")
+    _need(weight.shape[1] == K and K % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0, "rows of 16-byte multiples")
+    _need(not swiglu or (N % 2 == 0 and bias is None), "gate_up weight must be [2 I, K], without bias")
+    if bias is not None:
+        _need(bias.numel() == N and bias.dtype in (torch.bfloat16, torch.float32), "bias must be [N] bfloat16 or float32")
+    out = torch.empty((M, N // 2 if swiglu else N), dtype=torch.bfloat16, device=x.device)
+    _check(
+        _load("gemm_tile").cw_gemm_bf16_tiled(
+            2 if swiglu else 0, _ptr(x), x.stride(0), _ptr(weight), _ptr(bias),
+            int(bias is not None and bias.dtype == torch.float32), _ptr(out), out.shape[1], M, N, K, _stream()),
+        "gemm_bf16_tiled",
+    )
+    return out
 
 
 @contextlib.contextmanager
@@ -448,6 +488,8 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
         _check(_load("gemm").cw_gemm_bf16_skinny(2, _ptr(x), K, _ptr(gate_up_weight), _ptr(out), two_i // 2, M, two_i, K, _stream()),
                "gemm_bf16_skinny(swiglu)")
         return out
+    if HIP_PRODUCTS and x.dtype == torch.bfloat16 and K % 8 == 0 and x.is_contiguous():
+        return linear_tiled(x, gate_up_weight, swiglu=True)
     return silu_mul(linear(x, gate_up_weight), out)
 
 

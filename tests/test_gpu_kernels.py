@@ -382,6 +382,52 @@ def test_fused_swiglu_product(M, I, K):
     torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 1000, 200), (2048, 1536, 1536), (129, 130, 72), (64, 256, 8), (1000, 52, 2048)])
+def test_tiled_product(M, N, K):
+    """The LDS-tiled matrix-core product: plain with a bias of either type, and gated; sizes that
+    are no multiples of the 128 x 128 x 64 tile; rows of x with a stride."""
+    from clockwork_amd import ops
+
+    wide = torch.randn(M, K + 16, device=DEV).to(torch.bfloat16)
+    x = wide[:, :K]  # row stride K + 16
+    w = (torch.randn(N, K, device=DEV) / K ** 0.5).to(torch.bfloat16)
+    want = x.float() @ w.float().t()
+    torch.testing.assert_close(ops.linear_tiled(x, w).float(), want, rtol=1e-2, atol=1e-2)
+    for bias_dtype in (torch.bfloat16, torch.float32):
+        b = torch.randn(N, device=DEV).to(bias_dtype)
+        torch.testing.assert_close(ops.linear_tiled(x, w, b).float(), want + b.float(), rtol=1e-2, atol=2e-2)
+    if N % 2 == 0:
+        I = N // 2
+        got = ops.linear_tiled(x, w, swiglu=True)
+        assert tuple(got.shape) == (M, I)
+        torch.testing.assert_close(got.float(), torch.nn.functional.silu(want[:, :I]) * want[:, I:], rtol=2e-2, atol=2e-2)
+    # a row does not depend on the other rows of the batch
+    alone = ops.linear_tiled(x[M - 1 :], w)
+    assert torch.equal(alone[0], ops.linear_tiled(x, w)[M - 1])
+
+
+def test_hip_products_switch_routes_large_products_to_the_tiled_kernel():
+    from clockwork_amd import ops
+
+    x = torch.randn(200, 96, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(2 * 70, 96, device=DEV) / 10).to(torch.bfloat16)
+    b = torch.randn(140, device=DEV).to(torch.bfloat16)
+    lib_y, lib_g = ops.linear(x, w, b), ops.linear_swiglu(x, w)
+    calls = []
+    real = ops.linear_tiled
+    ops.linear_tiled = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+    ops.use_hip_products(True)
+    try:
+        own_y, own_g = ops.linear(x, w, b), ops.linear_swiglu(x, w)
+        logits = ops.linear(x, w, out_dtype=torch.float32)
+    finally:
+        ops.use_hip_products(False)
+        ops.linear_tiled = real
+    assert len(calls) == 3 and logits.dtype == torch.float32
+    torch.testing.assert_close(own_y.float(), lib_y.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(own_g.float(), lib_g.float(), rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_linear_library_path_and_float32_logits(dtype):
     from clockwork_amd import ops

@@ -157,6 +157,30 @@ def test_layers_of_the_larger_models(tmp_path, which):
     assert rms < 2e-2 * scale and worst < 1e-1 * scale
 
 
+def test_replay_with_the_tiled_products_instead_of_the_library(model_dirs):
+    """``hip_products``: the large bfloat16 products run on the package's own tiled kernel."""
+    from clockwork_amd import ops
+    from clockwork_amd.config.engine import EngineConfig
+    from clockwork_amd.engine.model_runner import ModelRunner
+
+    name = "B"
+    requests = _requests(name)
+    cfg = EngineConfig.defaults(str(model_dirs[name]), dtype="bfloat16", block_size=8, enable_prefix_cache=False,
+                                watermark=0.0, max_model_len=512, hip_products=True,
+                                num_blocks=replay.pages_needed(requests, 4, 8))
+    calls = []
+    real = ops.linear_tiled
+    ops.linear_tiled = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+    try:
+        runner = ModelRunner(cfg, cache_fill=float("nan"))
+        got = replay.run_trace(runner, replay.mixed(requests))
+    finally:
+        ops.linear_tiled = real
+        ops.use_hip_products(False)
+    assert calls
+    replay.compare(got, _plain(name, model_dirs), **TOL["bfloat16"])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_and_long_decoding(model_dirs, dtype):
     """The first tokens of a sequence (one-token prompt, then decoding from position 1) and a
