@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16] [--shape 1.5b]
+    python bench.py --workload mixed [--shape 7b] [--requests 64]
 
 Default workload: the layer sizes of Qwen2.5-1.5B with random weights (seed 2), bfloat16,
 8 requests that each hold a 2048-token prompt, context limit 4096, pages of 16 tokens. A
@@ -44,7 +45,7 @@ def _sync():
     torch.cuda.synchronize()
 
 
-def build_runner(args):
+def build_runner(args, prefix_cache: bool = False, max_batch: int = 0):
     from clockwork_amd.config.engine import EngineConfig
     from clockwork_amd.engine.model_runner import GRAPH_BATCH_SIZES, ModelRunner
     from clockwork_amd.parts.model import model_param_specs
@@ -59,10 +60,10 @@ def build_runner(args):
     mcfg = arch.parse_config(config)
     spec = arch.build_spec(mcfg)
     source = RandomSource(arch.weight_plan(mcfg, spec), model_param_specs(spec), seed=2, device="cuda")
-    max_batch = max(args.batch, 64)
+    max_batch = max(args.batch, 64, max_batch)
     cfg = EngineConfig.defaults(
         "random:qwen2.5-1.5b", dtype=args.dtype, max_model_len=CONTEXT, block_size=BLOCK,
-        num_blocks=max_batch * CONTEXT // BLOCK, enable_prefix_cache=False, watermark=0.0,
+        num_blocks=max_batch * CONTEXT // BLOCK, enable_prefix_cache=prefix_cache, watermark=0.0,
         max_num_seqs=max_batch, max_num_batched_tokens=max(PROMPT_LEN, max_batch),
     )
     runner = ModelRunner(cfg, weight_source=source, config_dict=config)
@@ -128,6 +129,126 @@ def time_prefill(cfg, runner, repeats: int = 3):
     return best
 
 
+def run_mixed(args) -> dict:
+    """A continuous batch through the whole engine: ``args.requests`` requests arrive at once,
+    prompt lengths uniform in [128, 2048], half of them opening with the same 1024 tokens (the
+    prefix cache serves those), prompts cut into portions under a budget of 2048 tokens a step
+    beside the decoding requests, 128 greedy tokens each."""
+    import torch
+
+    from clockwork_amd.engine.llm_engine import LLMEngine
+    from clockwork_amd.engine.sequence import SamplingParams
+
+    n_req, out_len, shared = args.requests, 128, 1024
+    cfg, runner = build_runner(args, prefix_cache=True, max_batch=n_req)
+    vocab = runner.spec.vocab_size
+    gen = torch.Generator().manual_seed(7)
+    common = torch.randint(0, vocab, (shared,), generator=gen).tolist()
+    prompts = []
+    for i in range(n_req):
+        n = int(torch.randint(128, PROMPT_LEN + 1, (1,), generator=gen))
+        ids = torch.randint(0, vocab, (n,), generator=gen).tolist()
+        if i % 2 == 1 and n > shared:
+            ids[:shared] = common
+        prompts.append(ids)
+    params = SamplingParams(max_tokens=out_len, temperature=0.0, ignore_eos=True)
+
+    engine = LLMEngine(cfg, runner=runner)
+
+    def once(tag):
+        engine.prefix_cache.reset()  # a cold prefix cache: only prefixes shared within the run hit
+        _sync()
+        before = engine.stats()
+        t0 = time.perf_counter()
+        for i, ids in enumerate(prompts):
+            engine.add_request(f"{tag}-{i}", prompt_token_ids=ids, sampling_params=params)
+        first, done, steps = {}, 0, 0
+        while engine.has_unfinished_requests():
+            outs = engine.step()
+            steps += 1
+            now = time.perf_counter() - t0
+            for o in outs:
+                if o.num_generated_tokens >= 1 and o.request_id not in first:
+                    first[o.request_id] = now
+                done += bool(o.finished)
+        _sync()
+        elapsed = time.perf_counter() - t0
+        assert done == n_req
+        after = engine.stats()
+        return elapsed, steps, first, {k: after[k] - before[k] for k in ("total_cached_tokens", "num_preempted_total")}
+
+    once("warm")  # graphs captured, library kernels chosen, prefix cache filled as in a running server
+    elapsed, steps, first, stats = once("run")
+    n_prompt = sum(len(p) for p in prompts)
+    ttft = sorted(first.values())
+    return {
+        "metric": f"output tok/s, {SHAPES[args.shape][0]} shape, continuous batch of {n_req} requests",
+        "value": round(n_req * out_len / elapsed, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": 0,
+        "ms_per_step": round(1e3 * elapsed / steps, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: uniform random token ids, random weights (seed 2)",
+        "seconds": round(elapsed, 4),
+        "prompt_tokens": n_prompt,
+        "prompt_tokens_from_prefix_cache": stats["total_cached_tokens"],
+        "all_tokens_per_s": round((n_prompt + n_req * out_len) / elapsed, 1),
+        "first_token_ms": {"p50": round(1e3 * ttft[len(ttft) // 2], 2), "max": round(1e3 * ttft[-1], 2)},
+        "preempted": stats["num_preempted_total"],
+        "config": {
+            "model": f"{SHAPES[args.shape][0]} shape (random weights)",
+            "layers": args.layers,
+            "layers_of_full_model": SHAPES[args.shape][1]["num_hidden_layers"],
+            "requests": n_req,
+            "prompt_len": "uniform 128..2048, every second one shares its first 1024 tokens",
+            "output_len": out_len,
+            "token_budget": PROMPT_LEN,
+            "seq_len": CONTEXT,
+            "block_size": BLOCK,
+            "sampling": "greedy",
+            "parallelism": "single GPU",
+        },
+    }
+
+
+def measure_peaks() -> dict:
+    """What this card reaches on the two plainest workloads, beside the published peaks the
+    fractions are priced against: a device-to-device copy of 2 GiB (bytes read + written) and the
+    library's bfloat16 product of 8192 x 8192 x 8192."""
+    import torch
+
+    def best_of(fn, n=5):
+        fn()
+        best = None
+        for _ in range(n):
+            _sync()
+            t0 = time.perf_counter()
+            fn()
+            _sync()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        return best
+
+    src = torch.empty(1 << 30, dtype=torch.int16, device="cuda").zero_()
+    dst = torch.empty_like(src)
+    t_copy = best_of(lambda: dst.copy_(src))
+    n = 8192
+    a = torch.randn(n, n, device="cuda", dtype=torch.bfloat16)
+    b = torch.randn(n, n, device="cuda", dtype=torch.bfloat16)
+    t_mm = best_of(lambda: torch.mm(a, b.t()))
+    return {
+        "copy_GBps": round(2 * src.numel() * 2 / t_copy / 1e9, 1),
+        "copy_frac_of_hbm_peak": round(2 * src.numel() * 2 / t_copy / 1e9 / PEAK_HBM_GBS, 4),
+        "bf16_product_TFLOPs": round(2 * n ** 3 / t_mm / 1e12, 1),
+        "bf16_product_frac_of_mfma_peak": round(2 * n ** 3 / t_mm / PEAK_FLOPS["bfloat16"], 4),
+    }
+
+
 def prefill_flops(spec, model, T: int) -> float:
     """2 * T * (matrix parameters of the layers) + causal attention + one row of the output head."""
     layer_params = 0
@@ -152,6 +273,10 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--no-tune", action="store_true", help="leave the matrix library's kernel choice at its default")
     ap.add_argument("--only-prefill", action="store_true", help="run the 2048-token prefill alone (for profiling)")
+    ap.add_argument("--workload", default="decode", choices=("decode", "mixed"),
+                    help="decode: the recorded benchmark; mixed: a continuous batch of --requests prompts of mixed lengths")
+    ap.add_argument("--requests", type=int, default=64)
+    ap.add_argument("--peaks", action="store_true", help="measure a device copy and a large library product instead")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
@@ -159,6 +284,12 @@ def main() -> int:
 
     import torch
 
+    if args.peaks:
+        print(json.dumps(measure_peaks()))
+        return 0
+    if args.workload == "mixed":
+        print(json.dumps(run_mixed(args)))
+        return 0
     cfg, runner = build_runner(args)
     if args.only_prefill:
         t = time_prefill(cfg, runner)
