@@ -265,7 +265,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
   constexpr int NBUF = MT <= 2 ? 2 : 1;
   constexpr int CH = cw_stream_chunk(SPW), NC = SPW / CH;
   static_assert(SPW % CH == 0, "the steps of a wave are whole chunks");
-  __shared__ float red[NBUF][WAVES][MT * 256];
+  __shared__ __align__(16) float red[NBUF][WAVES][MT * 256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, s = lane >> 4;
   const int I = N / 2;  // MODE 2 only
@@ -278,9 +278,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
   }
   auto wrow = [&](int tile) __attribute__((always_inline)) -> const bf16_t* {
     int64_t n;
-    if (MODE == 2) {
-      const int64_t i = min((int64_t)tile * 8 + (r & 7), (int64_t)I - 1);
-      n = (r < 8) ? i : I + i;
+    if (MODE == 2) {  // gate and up rows alternate, so that a pair lies side by side in the tile
+      const int64_t i = min((int64_t)tile * 8 + (r >> 1), (int64_t)I - 1);
+      n = (r & 1) ? I + i : i;
     } else {
       n = min((int64_t)tile * 16 + r, (int64_t)N - 1);
     }
@@ -371,21 +371,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
       for (int u = 0; u < CH; ++u) cur[u] = nxt[u];
     }
     w_tile = w_next;
-    // lane (r, s) holds weight rows 4s..4s+3 of token r of tile mt -> red[buf][wave][mt][row][token]
+    // lane (r, s) holds weight rows 4s..4s+3 of token r of tile mt -> red[buf][wave][mt][token][row]:
+    // one 16-byte store a lane, the lanes of a wave side by side (no bank is hit twice)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) red[buf][wave][mt * 256 + (4 * s + i) * 16 + r] = acc[mt][i];
+      *reinterpret_cast<f32x4_t*>(&red[buf][wave][mt * 256 + r * 16 + 4 * s]) = acc[mt];
     __syncthreads();
     if (MODE == 2) {
-      if (threadIdx.x < MT * 128) {  // (token, j): 8 outputs of a token lie side by side
+      if (threadIdx.x < MT * 128) {  // (token, j): the gate and the up value of output j are neighbours
         const int j = threadIdx.x & 7, m = threadIdx.x >> 3;
-        const int at = (m >> 4) * 256 + (m & 15);
         float g = 0.0f, up = 0.0f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
-          g += red[buf][w][at + j * 16];
-          up += red[buf][w][at + (j + 8) * 16];
+          const float2 gu = *reinterpret_cast<const float2*>(&red[buf][w][m * 16 + 2 * j]);
+          g += gu.x;
+          up += gu.y;
         }
         const int64_t i = (int64_t)tile * 8 + j;
         if (m < M && i < I) ((bf16_t*)C)[(int64_t)m * ldc + i] = __float2bfloat16(g / (1.0f + __expf(-g)) * up);
@@ -393,10 +393,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
     } else {
       for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {  // (token, j): 16 outputs side by side
         const int j = idx & 15, m = idx >> 4;
-        const int at = (m >> 4) * 256 + (m & 15) + j * 16;
         float v = 0.0f;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) v += red[buf][w][at];
+        for (int w = 0; w < WAVES; ++w) v += red[buf][w][idx];
         const int64_t n = (int64_t)tile * 16 + j;
         if (m < M && n < N) {
           if (MODE == 3) ((float*)C)[((int64_t)blockIdx.y * M + m) * ldc + n] = v;
@@ -520,17 +519,21 @@ CW_EXPORT int cw_gemm_bf16_skinny_ksplits(int M, int N, int K) {
   const int k_steps = (K + 31) / 32;
   if (M > 64 || tiles > 512) return 1;
   if (M > 16) {
-    if (tiles > 128) return 1;
     // Only the streaming kernel takes partial sums of more than 16 rows, and the alternative is a
-    // library product that leaves most compute units idle on so narrow an output: split K just
-    // far enough that every compute unit gets a tile, down to 8 steps of 32 per split.
+    // library product that leaves most compute units idle on so narrow an output. Split K far
+    // enough that every compute unit gets a tile (two for a long K) and that a wave's share of x
+    // fits its registers, down to 8 steps of 32 per split.
+    // (an output wide enough for half the compute units is split only if K is much longer still)
+    if (tiles > 128 && K < 2 * N) return 1;
+    const int mt = M <= 32 ? 2 : 4;
     int s = (cw_num_compute_units() + tiles - 1) / tiles;
     if (K >= 4096 && s < 512 / tiles) s = 512 / tiles;
     if (s > 8) s = 8;
+    while (s < 16 && !cw_stream_fits(8, cw_stream_round_spw((k_steps + s * 8 - 1) / (s * 8)), mt)) ++s;
     while (s > 1 && K / s < 256) --s;
-    int mt, spw, n_tiles;
+    int mt_, spw, n_tiles;
     dim3 grid;
-    if (s <= 1 || !plan_stream(3, M, N, K, s, &mt, &spw, &grid, &n_tiles)) return 1;
+    if (s <= 1 || !plan_stream(3, M, N, K, s, &mt_, &spw, &grid, &n_tiles)) return 1;
     return s;
   }
   if (K < 4096) return 1;
@@ -652,7 +655,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_qkv_rope_bf16_kernel(
     int bias_f32, const int* __restrict__ positions, const int* __restrict__ slots,
     const float* __restrict__ inv_freq, bf16_t* __restrict__ q_out, bf16_t* __restrict__ k_cache,
     bf16_t* __restrict__ v_cache, int64_t cache_rows, int M, int K, int nh, int nkv, int hd) {
-  __shared__ float red[WAVES][MT * 256];  // [wave][token tile][tile row][token]
+  __shared__ __align__(16) float red[WAVES][MT * 256];  // [wave][token tile][token][tile row]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, s = lane >> 4;
   const int half = hd / 2;
@@ -695,12 +698,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_qkv_rope_bf16_kernel(
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u][mt], acc[mt], 0, 0, 0);
   }
+  // lane (r, s) holds tile rows 4s..4s+3 of token r: one 16-byte store, no bank hit twice
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][mt * 256 + (4 * s + i) * 16 + r] = acc[mt][i];
+  for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<f32x4_t*>(&red[wave][mt * 256 + r * 16 + 4 * s]) = acc[mt];
   __syncthreads();
-  // MT * 256 values [token tile][tile row][token]; each is summed over the waves by one thread
+  // MT * 256 values [token tile][token][tile row]; each is summed over the waves by one thread
   for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {
     float sum = red[0][idx];
 #pragma unroll
@@ -712,7 +714,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_qkv_rope_bf16_kernel(
     if (bias == nullptr) return 0.0f;
     return bias_f32 ? ((const float*)bias)[col] : __bfloat162float(((const bf16_t*)bias)[col]);
   };
-  auto summed = [&](int row, int m) -> float { return red[0][(m >> 4) * 256 + row * 16 + (m & 15)]; };
+  auto summed = [&](int row, int m) -> float { return red[0][m * 16 + row]; };
   if (is_v) {
     // idx -> (token m, row j), j fastest: 16 consecutive elements of a cache row
     for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {

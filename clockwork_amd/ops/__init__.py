@@ -383,6 +383,8 @@ SKINNY_MAX_ROWS = 16
 # up to this many rows the shapes that the persistent streaming kernel takes do (the library
 # product is faster for the others, measured)
 STREAM_MAX_ROWS = 64
+# the fused q/k/v kernel takes more than SKINNY_MAX_ROWS rows for weight matrices up to this many elements
+FUSED_QKV_MAX_WEIGHTS = 8 << 20
 
 
 def linear_tiled(x: torch.Tensor, weight: torch.Tensor, bias=None, swiglu: bool = False) -> torch.Tensor:
@@ -428,8 +430,12 @@ def library_tuning():
 
 
 def qkv_rope_fused_supported(x: torch.Tensor, weight: torch.Tensor, rotary_dim: int, hd: int) -> bool:
-    """The fused q/k/v product + rotary + cache write takes few bfloat16 rows and a full rotary dimension."""
-    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[0] <= STREAM_MAX_ROWS
+    """The fused q/k/v product + rotary + cache write takes few bfloat16 rows and a full rotary
+    dimension. Beyond 16 rows it serves small weight matrices only: a large one is faster as a
+    product and a rotation kernel (measured: 33 MB at 24 rows and more)."""
+    rows = x.shape[0]
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+            and (rows <= SKINNY_MAX_ROWS or (rows <= STREAM_MAX_ROWS and weight.numel() <= FUSED_QKV_MAX_WEIGHTS))
             and x.shape[1] % 8 == 0 and rotary_dim == hd and hd % 16 == 0)
 
 
