@@ -110,7 +110,8 @@ template <> struct Chunk4<bf16_t> {
   }
 };
 
-template <typename T, typename WT, typename DT>
+// KC: chunks of 4 elements a thread holds (rows of up to 1024 * KC elements)
+template <typename T, typename WT, typename DT, int KC>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta0,
                                                               const DT* __restrict__ delta,
                                                               int parts, int64_t part_stride,
@@ -125,9 +126,9 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   T* o = out + (int64_t)i * H;
   const bool write_back = rows == nullptr && (dl != nullptr || d0 != nullptr);
   const int n_chunks = H / 4;
-  float v[4][4], w[4][4];
+  float v[KC][4], w[KC][4];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < KC; ++k) {
     const int ch = threadIdx.x + k * 256;
     if (ch < n_chunks) {
       Chunk4<float>::load(x + ch * 4, v[k]);
@@ -138,7 +139,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   }
   if (d0) {  // an earlier branch's output that was not added yet: it comes first, as it would have
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < KC; ++k) {
       const int ch = threadIdx.x + k * 256;
       if (ch < n_chunks) {
         float d[4];
@@ -149,28 +150,28 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     }
   }
   if (dl) {
-    float acc[4][4];
+    float acc[KC][4];
     for (int q = 0; q < parts; ++q) {
-      float d[4][4];
+      float d[KC][4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
+      for (int k = 0; k < KC; ++k) {
         const int ch = threadIdx.x + k * 256;
         if (ch < n_chunks) Chunk4<DT>::load(dl + q * part_stride + ch * 4, d[k]);
         else d[k][0] = d[k][1] = d[k][2] = d[k][3] = 0.0f;
       }
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
+      for (int k = 0; k < KC; ++k)
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[k][e] = q == 0 ? d[k][e] : acc[k][e] + d[k][e];
     }
 #pragma unroll
-    for (int k = 0; k < 4; ++k)
+    for (int k = 0; k < KC; ++k)
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[k][e] += acc[k][e];
   }
   float ss = 0.0f;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < KC; ++k) {
     const int ch = threadIdx.x + k * 256;
     if (ch < n_chunks) {
       if (write_back) Chunk4<float>::store(x + ch * 4, v[k]);
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   const float total = (partial[0] + partial[1]) + (partial[2] + partial[3]);
   const float inv = 1.0f / sqrtf(total / (float)H + eps);
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < KC; ++k) {
     const int ch = threadIdx.x + k * 256;
     if (ch < n_chunks) {
       float r[4];
@@ -203,14 +204,18 @@ CW_EXPORT int cw_add_rmsnorm(float* resid, const void* delta0, const void* delta
   if (n < 0 || H <= 0 || delta_parts < 0 || delta_parts > 64) return CW_ERR_ARG;
   if (n == 0) return CW_OK;
   dim3 grid(n), block(256);
-  const bool vec = (H % 4 == 0) && H <= 4096 && !((uintptr_t)resid & 15) && !((uintptr_t)out & 15) &&
+  const bool vec = (H % 4 == 0) && H <= 8192 && !((uintptr_t)resid & 15) && !((uintptr_t)out & 15) &&
                    !((uintptr_t)weight & 15) && !((uintptr_t)delta & 15) && !((uintptr_t)delta0 & 15);
   const int parts = delta_parts > 0 ? delta_parts : 1;
   const int64_t part_stride = (int64_t)T_rows * H;
 #define CW_LAUNCH(T, WT, DT)                                                                           \
   do {                                                                                                 \
-    if (vec)                                                                                           \
-      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, WT, DT>), grid, block, 0, stream, resid,           \
+    if (vec && H <= 4096)                                                                              \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, WT, DT, 4>), grid, block, 0, stream, resid,        \
+                         (const T*)delta0, (const DT*)delta, parts, part_stride, (const WT*)weight, eps, \
+                         (T*)out, rows, H);                                                            \
+    else if (vec)                                                                                      \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, WT, DT, 8>), grid, block, 0, stream, resid,        \
                          (const T*)delta0, (const DT*)delta, parts, part_stride, (const WT*)weight, eps, \
                          (T*)out, rows, H);                                                            \
     else                                                                                               \

@@ -36,7 +36,7 @@ def test_embedding(dtype, V, H, T):
 
 
 @pytest.mark.parametrize("dtype,wdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32)])
-@pytest.mark.parametrize("T,H,eps", [(5, 100, 1e-5), (3, 1536, 1e-6), (2, 7, 3e-6), (1, 4100, 1e-6)])
+@pytest.mark.parametrize("T,H,eps", [(5, 100, 1e-5), (3, 1536, 1e-6), (2, 7, 3e-6), (1, 4100, 1e-6), (2, 8192, 1e-6), (1, 8196, 1e-5)])
 def test_add_rmsnorm(dtype, wdtype, T, H, eps):
     from clockwork_amd import ops
 
