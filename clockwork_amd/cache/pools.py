@@ -17,6 +17,35 @@ from clockwork_amd.cache.manager import GroupLayout
 from clockwork_amd.parts.base import EntryCache
 
 
+def page_bytes(groups: list[GroupLayout], block_size: int, dtype: torch.dtype) -> int:
+    """Bytes one page number occupies: its keys and values in every entry of every paged group
+    (each group has a pool of ``num_blocks`` pages of its own)."""
+    elem = torch.empty((), dtype=dtype).element_size()
+    total = 0
+    for group in groups:
+        if group.is_kv:
+            total += len(group.entries) * 2 * block_size * group.need.num_kv_heads * group.need.head_dim * elem
+    return total
+
+
+def pages_that_fit(groups: list[GroupLayout], block_size: int, dtype: torch.dtype, free_bytes: int,
+                   fraction: float, most: int) -> int:
+    """How many pages per group to make when the configuration leaves it open: ``fraction`` of
+    the free device memory, but no more than ``most`` (what the scheduler can ever hold live,
+    with room for cached prefixes) and at least one page."""
+    per_page = page_bytes(groups, block_size, dtype)
+    if per_page == 0:
+        return 1
+    if not 0.0 < fraction <= 1.0:
+        raise ValueError(f"memory_fraction must be in (0, 1], got {fraction}")
+    fit = int(free_bytes * fraction) // per_page
+    if fit < 1:
+        raise RuntimeError(
+            f"no room for the cache: one page takes {per_page} bytes, {free_bytes} bytes of device memory are free"
+        )
+    return max(1, min(fit, most))
+
+
 class CachePools:
     def __init__(self, groups: list[GroupLayout], block_size: int, num_blocks: int,
                  max_num_seqs: int, dtype: torch.dtype, device, fill: float = 0.0) -> None:

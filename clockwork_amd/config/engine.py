@@ -46,10 +46,14 @@ class ModelConfig:
 
 @dataclass
 class CacheConfig:
-    """Paged cache sizing (clockwork/config.py:34-39). ``num_blocks`` is pages per layer group."""
+    """Paged cache sizing (clockwork/config.py:34-39). ``num_blocks`` is pages per layer group;
+    0 leaves it to the engine: ``memory_fraction`` of the device memory that is free once the
+    weights are loaded, capped at twice what ``max_num_seqs`` requests of ``max_model_len``
+    tokens can hold (the second half is room for cached prefixes)."""
 
     block_size: int = 16
     num_blocks: int = 512
+    memory_fraction: float = 0.8
     enable_prefix_cache: bool = True
     watermark: float = 0.01
 

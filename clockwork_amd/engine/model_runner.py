@@ -17,7 +17,7 @@ import torch
 
 from clockwork_amd import ops
 from clockwork_amd.cache.manager import CacheManager, cache_needs_of, plan_groups
-from clockwork_amd.cache.pools import CachePools
+from clockwork_amd.cache.pools import CachePools, pages_that_fit
 from clockwork_amd.config.engine import EngineConfig
 from clockwork_amd.engine.batch import StaticDecodeBatch, StepContext, StepEntry, build_context
 from clockwork_amd.parts.model import DecoderModel
@@ -61,15 +61,22 @@ class ModelRunner:
         self.model.bind(params, self.device, self.dtype)
 
         groups = plan_groups(cache_needs_of(self.spec, self.model.mixers()))
+        num_blocks = cfg.cache.num_blocks
+        if num_blocks <= 0:
+            # left open: what fits beside the weights, up to what the scheduler can ever use
+            most = 2 * cfg.scheduler.max_num_seqs * -(-cfg.model.max_model_len // cfg.cache.block_size)
+            num_blocks = pages_that_fit(groups, cfg.cache.block_size, self.dtype,
+                                        torch.cuda.mem_get_info(self.device)[0], cfg.cache.memory_fraction, most)
+        self.num_blocks = num_blocks
         self.manager = CacheManager(
             groups,
             block_size=cfg.cache.block_size,
-            num_blocks=cfg.cache.num_blocks,
+            num_blocks=num_blocks,
             max_num_seqs=cfg.scheduler.max_num_seqs,
             watermark=cfg.cache.watermark,
         )
         self.pools = CachePools(
-            groups, cfg.cache.block_size, cfg.cache.num_blocks, cfg.scheduler.max_num_seqs,
+            groups, cfg.cache.block_size, num_blocks, cfg.scheduler.max_num_seqs,
             self.dtype, self.device, fill=cache_fill,
         )
         self.caches = [self.pools.entry_cache(i, e.cache_from) for i, e in enumerate(self.spec.run)]

@@ -286,3 +286,29 @@ def test_random_request_orders_never_lose_or_duplicate_a_page(seed):
     for sid in list(live):
         m.free(sid)
     assert all(p.num_free == 24 for p in m.pools)
+
+
+# ------------------------------------------------------------------ sizing the pools
+def test_pages_that_fit_follows_the_reference_arithmetic_and_its_caps():
+    import torch
+
+    from clockwork_amd.cache.pools import page_bytes, pages_that_fit
+
+    # 28 layers, block 16, 2 kv heads of 128, 2 bytes: 458,752 bytes a page
+    # (configs/qwen2.5-1.5b-instruct-cuda.yaml:24-34)
+    groups = plan_groups([KVPagesSpec(2, 128)] * 28)
+    assert page_bytes(groups, 16, torch.bfloat16) == 458752
+    assert page_bytes(groups, 16, torch.float32) == 2 * 458752
+    free = 100 * 458752 + 17
+    assert pages_that_fit(groups, 16, torch.bfloat16, free, 1.0, most=10 ** 9) == 100
+    assert pages_that_fit(groups, 16, torch.bfloat16, free, 0.5, most=10 ** 9) == 50
+    assert pages_that_fit(groups, 16, torch.bfloat16, free, 1.0, most=64) == 64
+    with pytest.raises(RuntimeError, match="no room"):
+        pages_that_fit(groups, 16, torch.bfloat16, 1000, 1.0, most=64)
+    with pytest.raises(ValueError, match="memory_fraction"):
+        pages_that_fit(groups, 16, torch.bfloat16, free, 0.0, most=64)
+    # two groups (all keys / a window) each have a pool: a page number costs both
+    two = plan_groups([KVPagesSpec(2, 16), KVPagesSpec(2, 16, window=8), KVPagesSpec(2, 16)])
+    assert page_bytes(two, 4, torch.float32) == 3 * 2 * 4 * 2 * 16 * 4
+    # a model without paged state needs no pages
+    assert pages_that_fit(plan_groups([StateSpec((4,), "float32")]), 16, torch.float32, 10, 1.0, most=5) == 1

@@ -16,7 +16,9 @@ def test_engine_defaults_match_the_reference():
     cfg = EngineConfig.defaults("some/dir")
     # clockwork/config.py:17-47
     assert (cfg.model.dtype, cfg.model.max_model_len, cfg.model.seed) == ("float32", 4096, 0)
-    assert dataclasses.asdict(cfg.cache) == dict(block_size=16, num_blocks=512, enable_prefix_cache=True, watermark=0.01)
+    cache = dataclasses.asdict(cfg.cache)
+    assert cache.pop("memory_fraction") == 0.8  # this engine's own: sizes the pools when num_blocks is 0
+    assert cache == dict(block_size=16, num_blocks=512, enable_prefix_cache=True, watermark=0.01)
     assert (cfg.scheduler.max_num_seqs, cfg.scheduler.max_num_batched_tokens) == (64, 2048)
     assert cfg.scheduler.enable_chunked_prefill and cfg.scheduler.max_prefill_chunk == 0
 
@@ -50,6 +52,15 @@ def test_yaml_sections(tmp_path):
     bad.write_text("cache:\n  block_size: 8\n")
     with pytest.raises(ValueError, match="top-level 'model' section"):
         EngineConfig.from_yaml(bad)
+
+
+def test_the_example_configuration_loads():
+    from pathlib import Path
+
+    cfg = EngineConfig.from_yaml(Path(__file__).resolve().parent.parent / "configs" / "qwen2.5-1.5b-instruct.yaml")
+    assert cfg.model.dtype == "bfloat16" and cfg.model.tune_products is True
+    assert cfg.cache.num_blocks == 0 and cfg.cache.memory_fraction == 0.8 and cfg.cache.block_size == 16
+    assert cfg.scheduler.max_num_batched_tokens == 2048 and cfg.scheduler.max_model_len == cfg.model.max_model_len
 
 
 def test_dtype_whitelist():

@@ -283,3 +283,13 @@ def test_command_line(model_dirs, tmp_path, capsys):
     assert line["token_ids"] == PlainQwen2(model_dirs[name]).greedy(prompt, 5)
     with pytest.raises(SystemExit):
         cli.main(["--config", str(yaml_path), "--set", "nonsense=1", "--prompt-ids", "1"])
+
+
+def test_cache_size_left_open_is_what_the_scheduler_can_use(model_dirs):
+    # a tiny model on a large card: the cap (twice max_num_seqs requests of max_model_len tokens) decides
+    eng = engine(model_dirs["A"], num_blocks=0, max_num_seqs=4, max_model_len=64)
+    assert eng.runner.num_blocks == 2 * 4 * (64 // 4) == eng.manager.num_blocks
+    prompts = prompts_for("A", [9, 17])
+    plain = PlainQwen2(model_dirs["A"])
+    for prompt, out in zip(prompts, eng.generate(prompts, greedy(6))):
+        assert out.token_ids == plain.greedy(prompt, 6)
