@@ -803,22 +803,31 @@ typedef __attribute__((address_space(3))) s16x4_t lds_s16x4_t;
 
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 
-template <int HD>
+// RB: row blocks (waves that own 32 query rows each) of a workgroup, 4 or 2. With 2 the same eight
+// waves cut a stage's keys four ways instead of two: half the rows per workgroup and half the
+// time per stage, for launches whose portions would otherwise leave compute units without work
+// and wait for the workgroups with the longest key ranges.
+template <int HD, int RB>
 struct PrefillTile {
+  static_assert(RB == 4 || (RB == 2 && HD <= 128), "two row blocks only with the eight-wave workgroup");
   static constexpr int KROW = HD + 8;   // K rows: 16 bytes of padding spread the 16-byte reads over the banks
   static constexpr int VROW = HD + 16;  // V rows: 32 bytes, for the 8-byte transposing reads
-  static constexpr int NH = HD <= 128 ? 2 : 1;  // waves that share a row block and split its keys
-  static constexpr int KW = HD <= 128 ? 64 : 32;  // keys a wave takes from a stage
+  static constexpr int NH = HD <= 128 ? 8 / RB : 1;  // waves that share a row block and split its keys
+  static constexpr int KW = HD <= 128 ? 128 / NH : 32;  // keys a wave takes from a stage
   static constexpr int KT = KW * NH;            // keys of one stage
-  static constexpr int NT = 256 * NH;           // threads of a workgroup
+  static constexpr int NT = 64 * RB * NH;       // threads of a workgroup
   static constexpr int STAGE = KT * (KROW + VROW);  // elements of one stage: a K tile, then a V tile
   static constexpr size_t BYTES = 2 * STAGE * sizeof(bf16_t);
   static constexpr int TABLE = 2048;  // block-table entries held in LDS at a time
+  // what the sets of waves exchange at the end: accumulators, then maxima and sums
+  static constexpr size_t XO_BYTES = (size_t)(NH - 1) * RB * 2 * (HD / 16) * 64 * 16;
+  static constexpr size_t XCHG_BYTES = XO_BYTES + (size_t)(NH - 1) * RB * 2 * 2 * 64 * 4;
+  static_assert(XCHG_BYTES <= BYTES, "the exchange reuses the tiles' memory");
 };
 
-template <int HD, bool POW2>
-__global__ __launch_bounds__(PrefillTile<HD>::NT, (HD <= 128 ? 2 : 1)) void attn_prefill_bf16_kernel(AttnParams p) {
-  using Tile = PrefillTile<HD>;
+template <int HD, bool POW2, int RB>
+__global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) void attn_prefill_bf16_kernel(AttnParams p) {
+  using Tile = PrefillTile<HD, RB>;
   constexpr int NF = HD / 32;     // k-steps of the score product
   constexpr int ND = HD / 16;     // 16-wide blocks of the head dimension
   constexpr int KROW = Tile::KROW, VROW = Tile::VROW;
@@ -830,8 +839,8 @@ __global__ __launch_bounds__(PrefillTile<HD>::NT, (HD <= 128 ? 2 : 1)) void attn
   int* tbl = reinterpret_cast<int*>(smem_raw + Tile::BYTES);
 
   const int lane = threadIdx.x & 63;
-  const int wave = (threadIdx.x >> 6) & 3;  // the wave's row block
-  const int half = threadIdx.x >> 8;        // its share of a stage's keys
+  const int wave = (threadIdx.x >> 6) % RB;  // the wave's row block
+  const int half = threadIdx.x / (64 * RB);  // its share of a stage's keys
   const int c = lane & 15, s = lane >> 4;
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / p.n_chunks, chunk = blockIdx.y % p.n_chunks;
@@ -1046,35 +1055,41 @@ __global__ __launch_bounds__(PrefillTile<HD>::NT, (HD <= 128 ? 2 : 1)) void attn
     __syncthreads();
   }
 
-  // ---- the waves of the second half hand their rows' state to the first half through LDS
-  // (the tiles are dead after the loop's last barrier): o, then m and l, lanes side by side
-  if constexpr (NH == 2) {
+  // ---- the other sets of waves hand their rows' state to the first set through LDS (the tiles
+  // are dead after the loop's last barrier): o, then m and l, lanes side by side; the first set
+  // merges them in a fixed order
+  if constexpr (NH > 1) {
+    constexpr int SET = RB * 2 * ND * 64;  // accumulator vectors of one set
     f32x4_t* xo = reinterpret_cast<f32x4_t*>(smem_raw);
-    float* xml = reinterpret_cast<float*>(smem_raw + (size_t)4 * 2 * ND * 64 * sizeof(f32x4_t));
-    if (half == 1) {
+    float* xml = reinterpret_cast<float*>(smem_raw + Tile::XO_BYTES);
+    if (half > 0) {
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
 #pragma unroll
-        for (int db = 0; db < ND; ++db) xo[((wave * 2 + b) * ND + db) * 64 + lane] = o[b][db];
-        xml[((wave * 2 + b) * 2 + 0) * 64 + lane] = m_run[b];
-        xml[((wave * 2 + b) * 2 + 1) * 64 + lane] = l_run[b];
+        for (int db = 0; db < ND; ++db) xo[(half - 1) * SET + ((wave * 2 + b) * ND + db) * 64 + lane] = o[b][db];
+        xml[(((half - 1) * RB + wave) * 2 + b) * 128 + lane] = m_run[b];
+        xml[(((half - 1) * RB + wave) * 2 + b) * 128 + 64 + lane] = l_run[b];
       }
     }
     __syncthreads();
-    if (half == 1) return;
+    if (half > 0) return;
+#pragma unroll 1
+    for (int h = 0; h < NH - 1; ++h) {
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      const float m1 = xml[((wave * 2 + b) * 2 + 0) * 64 + lane];
-      const float l1 = xml[((wave * 2 + b) * 2 + 1) * 64 + lane];
-      const float m = fmaxf(m_run[b], m1);
-      const float msc = m == -INFINITY ? 0.0f : m * sl2;
-      const float a0 = __builtin_amdgcn_exp2f(m_run[b] * sl2 - msc);
-      const float a1 = __builtin_amdgcn_exp2f(m1 * sl2 - msc);
-      l_run[b] = l_run[b] * a0 + l1 * a1;
+      for (int b = 0; b < 2; ++b) {
+        const float m1 = xml[((h * RB + wave) * 2 + b) * 128 + lane];
+        const float l1 = xml[((h * RB + wave) * 2 + b) * 128 + 64 + lane];
+        const float m = fmaxf(m_run[b], m1);
+        const float msc = m == -INFINITY ? 0.0f : m * sl2;
+        const float a0 = __builtin_amdgcn_exp2f(m_run[b] * sl2 - msc);
+        const float a1 = __builtin_amdgcn_exp2f(m1 * sl2 - msc);
+        l_run[b] = l_run[b] * a0 + l1 * a1;
+        m_run[b] = m;
 #pragma unroll
-      for (int db = 0; db < ND; ++db) {
-        const f32x4_t o1 = xo[((wave * 2 + b) * ND + db) * 64 + lane];
-        o[b][db] = o[b][db] * a0 + o1 * a1;
+        for (int db = 0; db < ND; ++db) {
+          const f32x4_t o1 = xo[h * SET + ((wave * 2 + b) * ND + db) * 64 + lane];
+          o[b][db] = o[b][db] * a0 + o1 * a1;
+        }
       }
     }
   }
@@ -1107,17 +1122,48 @@ __global__ __launch_bounds__(PrefillTile<HD>::NT, (HD <= 128 ? 2 : 1)) void attn
 // 1 when this head size has the bfloat16 matrix-core kernel for portions (multiples of 32).
 CW_EXPORT int cw_attention_prefill_supported() { return CW_HAS_PREFILL; }
 
+#if CW_HAS_PREFILL
+template <bool POW2, int RB>
+static int launch_prefill(const AttnParams& p, int n_items, int table_stride, hipStream_t stream) {
+  using Tile = PrefillTile<CW_HD, RB>;
+  dim3 grid(n_items, p.nkv * p.n_chunks), block(Tile::NT);
+  // two stages of K and V tiles, then the window of the block table
+  const size_t entries = (size_t)table_stride < (size_t)Tile::TABLE ? table_stride : Tile::TABLE;
+  if ((Tile::KT + p.block_size - 1) / p.block_size + 1 > Tile::TABLE) return CW_ERR_SIZE;
+  const size_t smem = Tile::BYTES + sizeof(int) * entries;
+  if (smem > 160 * 1024) return CW_ERR_SIZE;
+  static size_t raised = 0;
+  if (smem > raised && smem > 48 * 1024) {
+    if (hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<CW_HD, POW2, RB>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return CW_ERR_LAUNCH;
+    raised = smem;
+  }
+  hipLaunchKernelGGL((attn_prefill_bf16_kernel<CW_HD, POW2, RB>), grid, block, smem, stream, p);
+  return cw_launch_status();
+}
+#endif
+
+// 1 if the kernel for portions can run with this many row blocks a workgroup (4, and 2 for head
+// sizes up to 128).
+CW_EXPORT int cw_attention_prefill_row_blocks_ok(int row_blocks) {
+  return CW_HAS_PREFILL && (row_blocks == 4 || (row_blocks == 2 && CW_HD <= 128)) ? 1 : 0;
+}
+
 // Portions of prompts, bfloat16. items: (request, first token, tokens, 0) with
-// tokens <= 4 * (32 / gh), gh = min(group, 32) heads of a group per workgroup.
+// tokens <= row_blocks * (32 / gh), gh = min(group, 32) heads of a group per workgroup; tokens of
+// an item beyond that are not computed. row_blocks: 4, or 2 (see PrefillTile).
 CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride,
                                         const void* k_cache, const void* v_cache, const int* block_tables,
                                         int table_stride, const int* ctx_lens, const int* cu_q,
                                         const int* items, int n_items, int nh, int nkv, int block_size,
-                                        int window, float scale, const void* zeros, hipStream_t stream) {
+                                        int window, float scale, const void* zeros, int row_blocks,
+                                        hipStream_t stream) {
 #if CW_HAS_PREFILL
   if (zeros == nullptr || ((uintptr_t)zeros & 15)) return CW_ERR_ARG;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || block_size <= 0 || table_stride <= 0 || window < 0)
     return CW_ERR_ARG;
+  if (!cw_attention_prefill_row_blocks_ok(row_blocks)) return CW_ERR_ARG;
   if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || ((uintptr_t)out & 7) ||
       (q_stride & 7) || (out_stride & 3))
     return CW_ERR_ARG;
@@ -1131,32 +1177,13 @@ CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* o
   p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = 1; p.window = window; p.scale = scale;
   p.part_o = nullptr; p.part_ml = nullptr; p.zeros = zeros;
   if ((int64_t)nkv * p.n_chunks > 65535) return CW_ERR_SIZE;
-  dim3 grid(n_items, nkv * p.n_chunks), block(PrefillTile<CW_HD>::NT);
-  // two stages of K and V tiles, then the window of the block table
-  const size_t entries = (size_t)table_stride < (size_t)PrefillTile<CW_HD>::TABLE ? table_stride : PrefillTile<CW_HD>::TABLE;
-  if ((PrefillTile<CW_HD>::KT + block_size - 1) / block_size + 1 > PrefillTile<CW_HD>::TABLE) return CW_ERR_SIZE;
-  const size_t smem = PrefillTile<CW_HD>::BYTES + sizeof(int) * entries;
-  if (smem > 160 * 1024) return CW_ERR_SIZE;
-  if (p.bs_shift >= 0) {
-    static size_t raised = 0;
-    if (smem > raised && smem > 48 * 1024) {
-      if (hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<CW_HD, true>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
-        return CW_ERR_LAUNCH;
-      raised = smem;
-    }
-    hipLaunchKernelGGL((attn_prefill_bf16_kernel<CW_HD, true>), grid, block, smem, stream, p);
-  } else {
-    static size_t raised = 0;
-    if (smem > raised && smem > 48 * 1024) {
-      if (hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<CW_HD, false>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
-        return CW_ERR_LAUNCH;
-      raised = smem;
-    }
-    hipLaunchKernelGGL((attn_prefill_bf16_kernel<CW_HD, false>), grid, block, smem, stream, p);
-  }
-  return cw_launch_status();
+#if CW_HD <= 128
+  if (row_blocks == 2)
+    return p.bs_shift >= 0 ? launch_prefill<true, 2>(p, n_items, table_stride, stream)
+                           : launch_prefill<false, 2>(p, n_items, table_stride, stream);
+#endif
+  return p.bs_shift >= 0 ? launch_prefill<true, 4>(p, n_items, table_stride, stream)
+                         : launch_prefill<false, 4>(p, n_items, table_stride, stream);
 #else
   return CW_ERR_ARG;
 #endif

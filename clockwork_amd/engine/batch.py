@@ -37,6 +37,7 @@ class AttentionPlan:
     gh_wide: int = 1
     mfma_items: Optional[torch.Tensor] = None   # the same portions cut for the bfloat16 matrix-core kernel
     n_mfma: int = 0
+    mfma_row_blocks: int = 4   # row blocks of that kernel's workgroups: 2 when 4 would leave compute units idle
     single_items: Optional[torch.Tensor] = None
     n_single: int = 0
     gh_single: int = 1
@@ -102,21 +103,31 @@ class StepContext:
         self._plans: dict = {}
         self.num_compute_units = 256
 
-    def attention_plan(self, nh: int, nkv: int) -> AttentionPlan:
-        key = (nh, nkv)
+    def attention_plan(self, nh: int, nkv: int, narrow_ok: bool = False) -> AttentionPlan:
+        """``narrow_ok``: the matrix-core kernel for portions also comes with two row blocks a
+        workgroup (see ``ops.prefill_row_blocks_ok``)."""
+        # a batch of single tokens has no portions: one plan, whatever the kernel for portions offers
+        narrow_ok = bool(narrow_ok) and any(q > 1 for q in self.h_q_lens)
+        key = (nh, nkv, narrow_ok)
         plan = self._plans.get(key)
         if plan is None:
-            plan = self._plans[key] = self._make_plan(nh, nkv)
+            plan = self._plans[key] = self._make_plan(nh, nkv, narrow_ok)
         return plan
 
-    def _make_plan(self, nh: int, nkv: int) -> AttentionPlan:
+    def _make_plan(self, nh: int, nkv: int, narrow_ok: bool = False) -> AttentionPlan:
         group = nh // nkv
         gh_wide = min(group, 64)
         tokens_per_tile = 64 // gh_wide
         gh_single = min(group, 16)
         wide: list[int] = []
         mfma: list[int] = []
-        tokens_per_mfma_item = 4 * (32 // min(group, 32))
+        # Workgroups of four row blocks share each key among the most rows, but a launch has to
+        # fill the compute units, and the workgroup with the longest key range decides its time:
+        # with fewer than 1.5 workgroups a compute unit, halve them.
+        tokens_of_four = 4 * (32 // min(group, 32))
+        workgroups = sum(-(-q // tokens_of_four) for q in self.h_q_lens if q > 1) * nkv * -(-group // 32)
+        row_blocks = 2 if narrow_ok and 2 * workgroups < 3 * self.num_compute_units else 4
+        tokens_per_mfma_item = row_blocks * (32 // min(group, 32))
         single: list[int] = []
         longest_single = 0
         for r, q_len in enumerate(self.h_q_lens):
@@ -129,7 +140,7 @@ class StepContext:
                 # longest key ranges first: the last tokens of a portion have the most work
                 for tok0 in reversed(range(0, q_len, tokens_per_mfma_item)):
                     mfma += [r, tok0, min(tokens_per_mfma_item, q_len - tok0), 0]
-        plan = AttentionPlan(gh_wide=gh_wide, gh_single=gh_single)
+        plan = AttentionPlan(gh_wide=gh_wide, gh_single=gh_single, mfma_row_blocks=row_blocks)
         plan.n_wide, plan.n_single, plan.n_mfma = len(wide) // 4, len(single) // 4, len(mfma) // 4
         plan.chunks_single = -(-group // gh_single)
         if plan.n_single:

@@ -108,7 +108,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_attention_workspace_floats": [I, I, I, I, I],
             "cw_attention": [I, I, P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P, L, P],
             "cw_attention_prefill_supported": [],
-            "cw_attention_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, P, P],
+            "cw_attention_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, P, I, P],
+            "cw_attention_prefill_row_blocks_ok": [I],
             "cw_attention_decode_supported": [],
             "cw_attention_decode_gh": [I],
             "cw_attention_decode_workspace_floats": [I, I, I, I],
@@ -524,9 +525,11 @@ def prefill_attention_supported(hd: int, dtype: torch.dtype) -> bool:
 
 def attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
                       nh: int, nkv: int, hd: int, block_size: int, window: int, scale: float,
-                      n_tokens: int, n_requests: int) -> None:
+                      n_tokens: int, n_requests: int, row_blocks: int = 4) -> None:
     """Portions of prompts through the bfloat16 matrix-core kernel; an item holds at most
-    4 * (32 // min(group, 32)) tokens. Other arguments as for ``attention``."""
+    ``prefill_tokens_per_item(nh // nkv, row_blocks)`` tokens. ``row_blocks`` 2 instead of 4: smaller
+    workgroups for launches with few items (head sizes up to 128). Other arguments as for ``attention``."""
+    _need(prefill_row_blocks_ok(hd, row_blocks), f"the kernel for head size {hd} does not take {row_blocks} row blocks")
     _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items)
     _need(q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16, "the kernel is bfloat16")
     _need(out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd, "attention output must be [T, nh * hd]")
@@ -540,9 +543,19 @@ def attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx
         _load("attention", hd).cw_attention_prefill_bf16(
             q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
             block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, nh, nkv, block_size,
-            window, float(scale), _zero_row(out.device), _stream()),
+            window, float(scale), _zero_row(out.device), int(row_blocks), _stream()),
         "attention_prefill_bf16",
     )
+
+
+def prefill_row_blocks_ok(hd: int, row_blocks: int) -> bool:
+    return bool(_load("attention", hd).cw_attention_prefill_row_blocks_ok(int(row_blocks)))
+
+
+def prefill_tokens_per_item(group: int, row_blocks: int = 4) -> int:
+    """Tokens one work item of ``attention_prefill`` may hold: a row block is 32 rows, a row a
+    (token, head of the group) pair."""
+    return row_blocks * (32 // min(group, 32))
 
 
 def decode_attention_supported(hd: int, dtype: torch.dtype) -> bool:

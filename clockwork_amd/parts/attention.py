@@ -74,15 +74,16 @@ class PagedAttention(Part):
             bias = self.qkv_bias[: self.q_width] if self.qkv_bias is not None else None
             self.position.rotate_and_store(qkv, bias, ctx.positions, None, nh, 0, hd, None, None)
         out = torch.empty((T, self.q_width), dtype=x.dtype, device=x.device)
-        plan = ctx.attention_plan(nh, nkv)
+        mfma = ops.prefill_attention_supported(hd, x.dtype)
+        plan = ctx.attention_plan(nh, nkv, narrow_ok=mfma and ops.prefill_row_blocks_ok(hd, 2))
         common = dict(
             q=qkv, q_stride=qkv.shape[1], out=out, k_cache=cache.k, v_cache=cache.v,
             block_tables=ctx.block_tables[cache.group], ctx_lens=ctx.ctx_lens, cu_q=ctx.cu_q,
             nh=nh, nkv=nkv, hd=hd, block_size=cache.block_size, window=s.window or 0,
             scale=s.scale, n_tokens=T, n_requests=ctx.num_requests,
         )
-        if plan.n_wide and ops.prefill_attention_supported(hd, x.dtype):
-            ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, **common)
+        if plan.n_wide and mfma:
+            ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, row_blocks=plan.mfma_row_blocks, **common)
         elif plan.n_wide:
             ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide,
                           n_splits=1, **common)

@@ -490,7 +490,11 @@ def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs,
     ctx = StepContext()
     ctx.device = torch.device(DEV)
     ctx.h_q_lens, ctx.h_ctx_lens = list(q_lens), list(ctx_lens)
-    plan = ctx.attention_plan(nh, nkv)
+    # prefill_kernel: True or 4 for workgroups of four row blocks, 2 for two (few work items here,
+    # so the plan takes the small workgroups whenever it may)
+    narrow = prefill_kernel == 2 and not isinstance(prefill_kernel, bool)
+    plan = ctx.attention_plan(nh, nkv, narrow_ok=narrow)
+    assert plan.mfma_row_blocks == (2 if narrow else 4)
     if splits is not None:
         plan.single_splits = splits
     R = len(q_lens)
@@ -511,7 +515,7 @@ def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs,
                   cu_q=cu, nh=nh, nkv=nkv, hd=hd, block_size=bs, window=window, scale=scale, n_tokens=T, n_requests=R)
     if plan.n_wide and prefill_kernel:
         assert ops.prefill_attention_supported(hd, dtype)
-        ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, **common)
+        ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, row_blocks=plan.mfma_row_blocks, **common)
     elif plan.n_wide:
         ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide, n_splits=1, **common)
     if plan.n_single and decode_kernel:
@@ -656,10 +660,13 @@ def test_decode_attention_kernel(nh, nkv, hd, bs, ctx_lens, splits, fixed_ranges
 @pytest.mark.parametrize("nh,nkv,hd,bs", [(4, 2, 32, 4), (6, 1, 32, 8), (3, 3, 64, 16), (12, 2, 128, 16), (2, 1, 256, 16),
                                           (40, 1, 64, 8), (7, 7, 96, 16), (4, 2, 160, 16), (2, 2, 224, 8)])
 @pytest.mark.parametrize("window", [0, 9, 40])
-def test_prefill_attention_kernel(nh, nkv, hd, bs, window):
+@pytest.mark.parametrize("row_blocks", [4, 2])
+def test_prefill_attention_kernel(nh, nkv, hd, bs, window, row_blocks):
     """The matrix-core kernel for portions: cached prefix + new tokens, ragged sizes, groups that
     do not divide 32, a group larger than 32, single tokens in the same batch, poisoned pages."""
     dtype = torch.bfloat16
+    if row_blocks == 2 and hd > 128:
+        pytest.skip("head sizes beyond 128 have the kernel with four row blocks only")
     ctx_lens = [21, 150, 2, 77, 1, 64, 333]
     q_lens = [6, 150, 2, 1, 1, 33, 40]
     num_blocks = sum(-(-c // bs) for c in ctx_lens) + 3
@@ -677,7 +684,7 @@ def test_prefill_attention_kernel(nh, nkv, hd, bs, window):
                 tables_dev[r][b] = -1
     qs = [torch.randn(q, nh, hd, device=DEV).to(dtype) for q in q_lens]
     out = _run_attention(dtype, nh, nkv, hd, bs, tables_dev, ctx_lens, q_lens, kc, vc, qs, window=window,
-                         prefill_kernel=True, decode_kernel=ops_decode_ok(hd))
+                         prefill_kernel=row_blocks, decode_kernel=ops_decode_ok(hd))
     assert not torch.isnan(out.float()).any()
     at = 0
     for r, q_len in enumerate(q_lens):
@@ -688,7 +695,8 @@ def test_prefill_attention_kernel(nh, nkv, hd, bs, window):
 
 
 @pytest.mark.parametrize("window", [0, 700])
-def test_prefill_attention_kernel_long_block_table(window):
+@pytest.mark.parametrize("row_blocks", [4, 2])
+def test_prefill_attention_kernel_long_block_table(window, row_blocks):
     """More pages than the kernel holds of a block table at a time (pages of one key): the table
     window moves on while the keys are walked."""
     dtype = torch.bfloat16
@@ -707,7 +715,8 @@ def test_prefill_attention_kernel_long_block_table(window):
     if window:
         for b in range(max(0, (ctx - q_len) - window + 1)):
             tables_dev[0][b] = -1
-    out = _run_attention(dtype, nh, nkv, hd, bs, tables_dev, [ctx], [q_len], kc, vc, [q], window=window, prefill_kernel=True)
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables_dev, [ctx], [q_len], kc, vc, [q], window=window,
+                         prefill_kernel=row_blocks)
     want = plain.attention_dense(q.float().cpu(), ks[0].float().cpu(), vs[0].float().cpu(), hd ** -0.5, window=window or None)
     torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
 
@@ -718,7 +727,8 @@ def ops_decode_ok(hd):
     return ops.decode_attention_supported(hd, torch.bfloat16)
 
 
-def test_prefill_attention_kernel_sharp_scores():
+@pytest.mark.parametrize("row_blocks", [4, 2])
+def test_prefill_attention_kernel_sharp_scores(row_blocks):
     """Scores of very different size, so that the running maximum moves from tile to tile and one
     far key dominates a row: rescaling and masking errors cannot hide behind near-uniform weights."""
     dtype = torch.bfloat16
@@ -726,7 +736,7 @@ def test_prefill_attention_kernel_sharp_scores():
     tables = [torch.randperm(20).tolist()[:19]]
     kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, 20, tables, [T])
     q = (3.0 * torch.randn(T, nh, hd, device=DEV)).to(dtype)
-    out = _run_attention(dtype, nh, nkv, hd, bs, tables, [T], [T], kc, vc, [q], prefill_kernel=True, scale=0.5)
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables, [T], [T], kc, vc, [q], prefill_kernel=row_blocks, scale=0.5)
     want = plain.attention_dense(q.float().cpu(), ks[0].float().cpu(), vs[0].float().cpu(), 0.5)
     torch.testing.assert_close(out.float().cpu(), want, rtol=3e-2, atol=3e-2)
 
