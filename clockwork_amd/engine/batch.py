@@ -101,6 +101,7 @@ class StepContext:
         self.h_state_slots: list[int] = []
         self.seq_ids: list[str] = []
         self._plans: dict = {}
+        self._pinned: list = []   # host buffers of the plans' uploads, alive as long as the step
         self.num_compute_units = 256
 
     def attention_plan(self, nh: int, nkv: int, narrow_ok: bool = False) -> AttentionPlan:
@@ -163,7 +164,7 @@ class StepContext:
         packer.add(single)
         packer.add(mfma)
         plan.wide_items, plan.single_items, plan.mfma_items = packer.upload(self.device)
-        self._keep = getattr(self, "_keep", []) + [packer]
+        self._pinned.append(packer)
         return plan
 
 
