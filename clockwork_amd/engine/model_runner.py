@@ -53,7 +53,7 @@ class ModelRunner:
         self.model_config = self.arch.parse_config(self.config_dict)
         self.spec = self.arch.build_spec(self.model_config)
         self.model = DecoderModel(self.spec)
-        ops.preload(self.model.head_dims())
+        ops.preload(self.model.head_dims(), tiled_products=cfg.model.hip_products)
         plan = self.arch.weight_plan(self.model_config, self.spec)
         params = load_parameters(
             cfg.model.model, plan, self.model.param_specs(), self.dtype, self.device, source=weight_source

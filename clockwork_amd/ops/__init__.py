@@ -62,9 +62,15 @@ def _load(name: str, head_dim: int | None = None) -> ctypes.CDLL:
     return lib
 
 
-def preload(head_dims) -> None:
-    """Build (side by side, if several are missing) and load what a model with these head sizes runs."""
-    jobs = [("core", None), ("gemm", None), ("gemm_tile", None), ("sampling", None)]
+def preload(head_dims=(), tiled_products: bool = False, sampling: bool = False) -> None:
+    """Build (side by side, if several are missing) and load what a model with these head sizes
+    runs: the common kernels, the products and one attention library per head size; the tiled
+    product and the sampling kernels only for a caller that uses them."""
+    jobs = [("core", None), ("gemm", None)]
+    if tiled_products:
+        jobs.append(("gemm_tile", None))
+    if sampling:
+        jobs.append(("sampling", None))
     jobs += [("attention", int(hd)) for hd in sorted(set(head_dims))]
     build.ensure_many(jobs)
     for name, hd in jobs:

@@ -22,6 +22,7 @@ class Sampler:
     def __init__(self, device, default_seed: int = 0) -> None:
         self.device = device
         self.default_seed = int(default_seed)
+        ops.preload(sampling=True)  # compiled now if it has to be, not at the first token
 
     def sample(self, logits: torch.Tensor, seqs: Seq[Sequence]) -> list[int]:
         """One token per row of ``logits`` (float32 [n, vocab]); row i belongs to ``seqs[i]``."""
