@@ -58,6 +58,7 @@ class LLMEngine:
         self._arrivals = itertools.count()
         self._generate_ids = itertools.count()
         self._ahead = None          # (SchedulerOutput, runner handle) made one step ahead
+        self._started = None        # (SchedulerOutput, sampled tokens on the device) of a step already on the GPU
         self.lookahead_steps = 0    # steps that ran from such a schedule
 
     def _look_ahead(self, out):
@@ -129,7 +130,60 @@ class LLMEngine:
     def step(self) -> list[RequestOutput]:
         """Schedule, run one batch, sample, finish; an output per request that got a token
         (llm_engine.py:99-125)."""
-        ahead, self._ahead = self._ahead, None
+        started, self._started = self._started, None
+        if started is not None:
+            out, drawn_on_device = started  # launched at the end of the previous call
+        else:
+            out, drawn_on_device = self._start_step()
+            if out is None:
+                return []
+        # the GPU is busy with this step: decide the next one now if it is plain decoding
+        if self.cfg.scheduler.lookahead:
+            self._ahead = self._look_ahead(out)
+        tokens = drawn_on_device.tolist() if drawn_on_device is not None else []
+        drawn = iter(tokens)
+        sampled: list[Sequence] = []
+        may_stop = False
+        for p in out.portions:
+            seq = p.seq
+            if seq.is_finished():  # aborted while its step was running: its token is dropped
+                if p.samples:
+                    next(drawn)
+                continue
+            seq.num_computed_tokens = p.start + p.num_tokens
+            prompt_done = p.start < len(seq.prompt_token_ids) <= seq.num_computed_tokens
+            if prompt_done and self.prefix_cache.enabled:
+                # the trie takes a hold only on blocks it adopts, so inserting while the
+                # request still holds its pages is safe (llm_engine.py:115-119)
+                n_full = len(seq.prompt_token_ids) // self.cfg.cache.block_size
+                self.prefix_cache.insert(seq.prompt_token_ids, self.manager.handles(seq.seq_id, n_full))
+            if p.samples:
+                token = next(drawn)
+                seq.append_token(token)
+                sampled.append(seq)
+                params = seq.sampling_params
+                may_stop = may_stop or bool(params.stop) or token in params.stop_token_ids or (
+                    not params.ignore_eos and token in self._eos_ids)
+        # The step decided ahead of time stays right unless a request stops with the token it just
+        # got (by length none does: such a step is not decided ahead). Then it can start before
+        # this step's outputs are made, and the GPU does not wait for them.
+        ahead = self._ahead
+        if ahead is not None and not may_stop and ahead[0].version == self.scheduler.version:
+            self._ahead = None
+            self._started = self._start_step(ahead)
+        outputs = [self._process(seq) for seq in sampled]
+        self.scheduler.free_finished()
+        for output in outputs:
+            if output.finished:
+                self._forget(output.request_id)
+        return outputs
+
+    def _start_step(self, ahead=None):
+        """Choose a step (the one decided ahead of time if it still holds, else the scheduler's),
+        put its kernels and the sampling kernels on the GPU's queue and return (schedule, sampled
+        tokens as a device tensor or None); (None, None) if nothing can run."""
+        if ahead is None:
+            ahead, self._ahead = self._ahead, None
         if ahead is not None and ahead[0].version == self.scheduler.version:
             # decided (and mostly laid out) while the last step ran; nothing has changed since
             out, handle = ahead
@@ -140,7 +194,7 @@ class LLMEngine:
             out = self.scheduler.schedule()
             if not out.portions:
                 if out.preempted or not self.scheduler.has_unfinished():
-                    return []
+                    return None, None
                 # nothing runs and the head does not fit: give it everything the prefix cache
                 # holds idle, once, before calling the request unschedulable (llm_engine.py:102-113)
                 if self.prefix_cache.evict(self.manager.num_blocks) > 0:
@@ -162,30 +216,7 @@ class LLMEngine:
             ]
             logits = self.runner.step(entries)
         sampling = [p.seq for p in out.portions if p.samples]
-        drawn_on_device = self.sampler.launch(logits, sampling) if sampling else None
-        # the GPU is busy with this step: decide the next one now if it is plain decoding
-        if self.cfg.scheduler.lookahead:
-            self._ahead = self._look_ahead(out)
-        tokens = drawn_on_device.tolist() if drawn_on_device is not None else []
-        outputs: list[RequestOutput] = []
-        drawn = iter(tokens)
-        for p in out.portions:
-            seq = p.seq
-            seq.num_computed_tokens = p.start + p.num_tokens
-            prompt_done = p.start < len(seq.prompt_token_ids) <= seq.num_computed_tokens
-            if prompt_done and self.prefix_cache.enabled:
-                # the trie takes a hold only on blocks it adopts, so inserting while the
-                # request still holds its pages is safe (llm_engine.py:115-119)
-                n_full = len(seq.prompt_token_ids) // self.cfg.cache.block_size
-                self.prefix_cache.insert(seq.prompt_token_ids, self.manager.handles(seq.seq_id, n_full))
-            if p.samples:
-                seq.append_token(next(drawn))
-                outputs.append(self._process(seq))
-        self.scheduler.free_finished()
-        for output in outputs:
-            if output.finished:
-                self._forget(output.request_id)
-        return outputs
+        return out, (self.sampler.launch(logits, sampling) if sampling else None)
 
     def generate(self, prompts, sampling_params: Optional[SamplingParams] = None) -> list[RequestOutput]:
         """Run prompts (strings or lists of token ids) to completion; final outputs in prompt order

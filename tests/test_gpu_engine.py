@@ -293,3 +293,29 @@ def test_cache_size_left_open_is_what_the_scheduler_can_use(model_dirs):
     plain = PlainQwen2(model_dirs["A"])
     for prompt, out in zip(prompts, eng.generate(prompts, greedy(6))):
         assert out.token_ids == plain.greedy(prompt, 6)
+
+
+def test_abort_while_the_next_step_already_runs(model_dirs):
+    """In a stretch of plain decoding the next step is put on the GPU before the current outputs
+    are made. A request aborted at that moment loses the token that step makes for it; the others
+    are untouched and every page comes back."""
+    name = "B"
+    prompts = prompts_for(name, [7, 12, 5], seed=9)
+    eng = engine(model_dirs[name], enable_prefix_cache=False)
+    for i, prompt in enumerate(prompts):
+        eng.add_request(f"r{i}", prompt_token_ids=prompt, sampling_params=greedy(16))
+    finals, aborted_after = {}, None
+    while eng.has_unfinished_requests():
+        for out in eng.step():
+            assert out.request_id != "r1" or aborted_after is None, "an aborted request produced an output"
+            if out.finished:
+                finals[out.request_id] = out.token_ids
+        if aborted_after is None and eng._started is not None:
+            aborted_after = len(eng._seqs["r1"].output_token_ids)
+            eng.abort_request("r1")
+    assert aborted_after is not None and 0 < aborted_after < 16
+    assert sorted(finals) == ["r0", "r2"]
+    plain = PlainQwen2(model_dirs[name])
+    assert finals["r0"] == plain.greedy(prompts[0], 16) and finals["r2"] == plain.greedy(prompts[2], 16)
+    assert eng.manager.min_free_blocks() == eng.manager.num_blocks
+    assert eng.stats()["lookahead_steps"] > 0
