@@ -13,6 +13,8 @@ import itertools
 from dataclasses import dataclass
 from typing import Optional
 
+import torch
+
 from clockwork_amd.cache.prefix import PrefixCache
 from clockwork_amd.config.engine import EngineConfig
 from clockwork_amd.engine.batch import StepEntry
@@ -58,7 +60,12 @@ class LLMEngine:
         self._arrivals = itertools.count()
         self._generate_ids = itertools.count()
         self._ahead = None          # (SchedulerOutput, runner handle) made one step ahead
-        self._started = None        # (SchedulerOutput, sampled tokens on the device) of a step already on the GPU
+        self._started = None        # (SchedulerOutput, sampled tokens on the device, their copy) of a step on the GPU
+        # sampled tokens come to the host through two pinned buffers, in turn: the copy of one
+        # step's tokens can be under way while the step before it is still being read
+        width = max(cfg.scheduler.max_num_seqs, GRAPH_BATCH_SIZES[-1], 1)
+        self._token_bufs = [torch.empty(width, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._token_buf_at = 0
         self.lookahead_steps = 0    # steps that ran from such a schedule
 
     def _look_ahead(self, out):
@@ -131,22 +138,30 @@ class LLMEngine:
         """Schedule, run one batch, sample, finish; an output per request that got a token
         (llm_engine.py:99-125)."""
         started, self._started = self._started, None
-        if started is not None:
-            out, drawn_on_device = started  # launched at the end of the previous call
-        else:
-            out, drawn_on_device = self._start_step()
-            if out is None:
+        if started is not None and all(p.seq.is_finished() for p in started[0].portions):
+            started = None  # queued for requests that have all stopped since: nothing of it is wanted
+        if started is None:
+            started = self._start_step()
+            if started is None:
                 return []
-        # the GPU is busy with this step: decide the next one now if it is plain decoding
+        out, drawn_on_device, fetch = started
+        # The GPU is busy with this step: decide the next one now if it is plain decoding, and
+        # put it on the GPU's queue at once, fed by this step's sampling kernels on the device,
+        # so that the GPU goes from one step to the next without waiting for the host. A request
+        # that stops with the token of this step is then run once too often: that costs nothing
+        # but the work, its extra token is dropped and its pages are reused only by later steps.
         if self.cfg.scheduler.lookahead:
             self._ahead = self._look_ahead(out)
-        tokens = drawn_on_device.tolist() if drawn_on_device is not None else []
+            if self._ahead is not None and self._ahead[1] is not None and drawn_on_device is not None:
+                ahead, self._ahead = self._ahead, None
+                self._started = self._start_step(ahead, device_tokens=drawn_on_device)
+        tokens = self._fetched(fetch)
         drawn = iter(tokens)
         sampled: list[Sequence] = []
         may_stop = False
         for p in out.portions:
             seq = p.seq
-            if seq.is_finished():  # aborted while its step was running: its token is dropped
+            if seq.is_finished():  # stopped or aborted while this step was queued: its token is dropped
                 if p.samples:
                     next(drawn)
                 continue
@@ -164,11 +179,11 @@ class LLMEngine:
                 params = seq.sampling_params
                 may_stop = may_stop or bool(params.stop) or token in params.stop_token_ids or (
                     not params.ignore_eos and token in self._eos_ids)
-        # The step decided ahead of time stays right unless a request stops with the token it just
-        # got (by length none does: such a step is not decided ahead). Then it can start before
-        # this step's outputs are made, and the GPU does not wait for them.
+        # A step decided ahead that could not be queued above (no captured graph for it yet) can
+        # still start before this step's outputs are made, unless a request may stop right now.
         ahead = self._ahead
-        if ahead is not None and not may_stop and ahead[0].version == self.scheduler.version:
+        if (self._started is None and ahead is not None and not may_stop
+                and ahead[0].version == self.scheduler.version):
             self._ahead = None
             self._started = self._start_step(ahead)
         outputs = [self._process(seq) for seq in sampled]
@@ -178,10 +193,33 @@ class LLMEngine:
                 self._forget(output.request_id)
         return outputs
 
-    def _start_step(self, ahead=None):
+    def _fetching(self, drawn_on_device):
+        """Begin to copy sampled tokens to the host; ``_fetched`` waits for them. The copy is
+        queued before whatever the GPU is given next, so waiting for it waits for nothing else."""
+        if drawn_on_device is None:
+            return None
+        buf = self._token_bufs[self._token_buf_at]
+        self._token_buf_at ^= 1
+        view = buf[: drawn_on_device.numel()]
+        view.copy_(drawn_on_device, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return view, event
+
+    @staticmethod
+    def _fetched(fetch) -> list[int]:
+        if fetch is None:
+            return []
+        view, event = fetch
+        event.synchronize()
+        return view.tolist()
+
+    def _start_step(self, ahead=None, device_tokens=None):
         """Choose a step (the one decided ahead of time if it still holds, else the scheduler's),
         put its kernels and the sampling kernels on the GPU's queue and return (schedule, sampled
-        tokens as a device tensor or None); (None, None) if nothing can run."""
+        tokens as a device tensor or None, the copy of those tokens to the host under way); None
+        if nothing can run. ``device_tokens``: the tokens the step before it sampled, still on
+        the device and not yet appended to their requests (a step decided ahead only)."""
         if ahead is None:
             ahead, self._ahead = self._ahead, None
         if ahead is not None and ahead[0].version == self.scheduler.version:
@@ -190,11 +228,13 @@ class LLMEngine:
             self.scheduler.commit_ahead(out)
             self.lookahead_steps += 1
         else:
+            if device_tokens is not None:
+                raise RuntimeError("tokens that are still on the device can only feed a step decided ahead")
             handle = None
             out = self.scheduler.schedule()
             if not out.portions:
                 if out.preempted or not self.scheduler.has_unfinished():
-                    return None, None
+                    return None
                 # nothing runs and the head does not fit: give it everything the prefix cache
                 # holds idle, once, before calling the request unschedulable (llm_engine.py:102-113)
                 if self.prefix_cache.evict(self.manager.num_blocks) > 0:
@@ -203,7 +243,8 @@ class LLMEngine:
                     raise RuntimeError("waiting request cannot be admitted even with an empty prefix cache")
             self.runner.apply_copies(out.copies)
         if handle is not None:
-            logits = self.runner.step_prepared(handle, [p.seq.output_token_ids[-1] for p in out.portions])
+            tokens = device_tokens if device_tokens is not None else [p.seq.output_token_ids[-1] for p in out.portions]
+            logits = self.runner.step_prepared(handle, tokens)
         else:
             entries = [
                 StepEntry(
@@ -216,7 +257,9 @@ class LLMEngine:
             ]
             logits = self.runner.step(entries)
         sampling = [p.seq for p in out.portions if p.samples]
-        return out, (self.sampler.launch(logits, sampling) if sampling else None)
+        pending = 1 if device_tokens is not None else 0
+        drawn = self.sampler.launch(logits, sampling, pending=pending) if sampling else None
+        return out, drawn, self._fetching(drawn)
 
     def generate(self, prompts, sampling_params: Optional[SamplingParams] = None) -> list[RequestOutput]:
         """Run prompts (strings or lists of token ids) to completion; final outputs in prompt order

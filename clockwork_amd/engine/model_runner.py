@@ -203,18 +203,26 @@ class ModelRunner:
         return key, entries
 
     @torch.no_grad()
-    def step_prepared(self, handle, tokens: Sequence[int]) -> torch.Tensor:
+    def step_prepared(self, handle, tokens) -> torch.Tensor:
         """Run the step that ``prepare_decode`` got ready, now that its tokens are known; every
-        entry's logits are returned, float32 [entries, vocab]."""
+        entry's logits are returned, float32 [entries, vocab]. ``tokens``: a sequence of ids, or
+        an int32 device tensor (what the sampling kernels of the step before wrote, possibly
+        still being computed: the tokens then never visit the host)."""
         key, entries = handle
         if len(tokens) != len(entries):
             raise ValueError(f"{len(tokens)} tokens for {len(entries)} prepared entries")
-        for e, tok in zip(entries, tokens):
-            if not 0 <= int(tok) < self.spec.vocab_size:
-                raise ValueError(f"request {e.seq_id}: token id {tok} outside the vocabulary")
         batch, graph, out = self._graphs[key]
-        batch.set_tokens(tokens)
-        batch.upload()
+        if isinstance(tokens, torch.Tensor):
+            if tokens.dtype != torch.int32 or tokens.device != self.device or tokens.dim() != 1:
+                raise ValueError("tokens on the device must be a 1-d int32 tensor on the engine's GPU")
+            batch.upload()
+            batch.ctx.token_ids[: len(entries)].copy_(tokens)  # after the upload, in stream order
+        else:
+            for e, tok in zip(entries, tokens):
+                if not 0 <= int(tok) < self.spec.vocab_size:
+                    raise ValueError(f"request {e.seq_id}: token id {tok} outside the vocabulary")
+            batch.set_tokens(tokens)
+            batch.upload()
         graph.replay()
         for e in entries:
             self.manager.release_behind_window(e.seq_id, e.start + 1)

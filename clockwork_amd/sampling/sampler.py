@@ -29,9 +29,10 @@ class Sampler:
         drawn = self.launch(logits, seqs)
         return [] if drawn is None else drawn.tolist()
 
-    def launch(self, logits: torch.Tensor, seqs: Seq[Sequence]):
+    def launch(self, logits: torch.Tensor, seqs: Seq[Sequence], pending: int = 0):
         """Start the kernels of ``sample`` and return the tokens as a device tensor (int32 [n]),
-        without waiting for them; None for no sequences."""
+        without waiting for them; None for no sequences. ``pending``: tokens of each sequence
+        that are sampled already but not yet appended to it (they count as draws made)."""
         n = len(seqs)
         if n == 0:
             return None
@@ -47,7 +48,7 @@ class Sampler:
         seeds = torch.tensor(
             [p.seed if p.seed is not None else self.default_seed for p in params], dtype=torch.int64
         )
-        draws = torch.tensor([len(s.output_token_ids) for s in seqs], dtype=torch.int64)
+        draws = torch.tensor([len(s.output_token_ids) + pending for s in seqs], dtype=torch.int64)
         dev = self.device
         return ops.sample(
             logits, temperature.to(dev), top_k.to(dev), top_p.to(dev), seeds.to(dev), draws.to(dev)

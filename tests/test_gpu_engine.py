@@ -319,3 +319,32 @@ def test_abort_while_the_next_step_already_runs(model_dirs):
     assert finals["r0"] == plain.greedy(prompts[0], 16) and finals["r2"] == plain.greedy(prompts[2], 16)
     assert eng.manager.min_free_blocks() == eng.manager.num_blocks
     assert eng.stats()["lookahead_steps"] > 0
+
+
+def test_sampled_tokens_do_not_depend_on_steps_queued_ahead(model_dirs):
+    """Temperature sampling: a step queued before the tokens of the step before it have reached
+    the host must make the same draws as one started afterwards (the n-th draw of a request is a
+    function of its seed and n alone)."""
+    from clockwork_amd.engine.llm_engine import LLMEngine
+
+    name = "B"
+    prompts = prompts_for(name, [9, 4, 30], seed=2)
+    params = [SamplingParams(max_tokens=14, temperature=0.8, top_k=50, top_p=0.9, seed=100 + i, ignore_eos=True)
+              for i in range(3)]
+
+    def session(lookahead: bool):
+        eng = LLMEngine(EngineConfig.defaults(str(model_dirs[name]), dtype="float32", block_size=4, num_blocks=128,
+                                              watermark=0.0, lookahead=lookahead))
+        for i, prompt in enumerate(prompts):
+            eng.add_request(f"r{i}", prompt_token_ids=prompt, sampling_params=params[i])
+        finals = {}
+        while eng.has_unfinished_requests():
+            for out in eng.step():
+                if out.finished:
+                    finals[out.request_id] = out.token_ids
+        return finals, eng.stats()["lookahead_steps"]
+
+    ahead, used = session(True)
+    plain_order, unused = session(False)
+    assert ahead == plain_order and used > 5 and unused == 0
+    assert len({tuple(v) for v in ahead.values()}) == 3
