@@ -348,3 +348,63 @@ def test_sampled_tokens_do_not_depend_on_steps_queued_ahead(model_dirs):
     plain_order, unused = session(False)
     assert ahead == plain_order and used > 5 and unused == 0
     assert len({tuple(v) for v in ahead.values()}) == 3
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_long_random_session_equals_every_request_alone(model_dirs, seed):
+    """Arrivals at random times, stop tokens, aborts, so few pages that requests are preempted,
+    shared prefixes, steps queued ahead: every request that finishes gives the tokens and the
+    reason it gives alone, and every page comes back."""
+    import random
+
+    name = "B"
+    vocab = TINY_CONFIGS[name][0]["vocab_size"]
+    rng = random.Random(seed)
+
+    def make(num_blocks, max_seqs, prefix):
+        return engine(model_dirs[name], block_size=8, num_blocks=num_blocks, watermark=0.01, max_num_seqs=max_seqs,
+                      max_num_batched_tokens=96, max_model_len=400, enable_prefix_cache=prefix)
+
+    shared = [rng.randrange(vocab) for _ in range(40)]
+    requests = []
+    for i in range(70):
+        prompt = shared[: rng.choice([0, 16, 40])] + [rng.randrange(vocab) for _ in range(rng.choice([1, 3, 9, 30, 70, 150]))]
+        stops = [rng.randrange(vocab) for _ in range(rng.choice([0, 0, 30, 120]))]
+        requests.append((f"q{i}", prompt, rng.choice([2, 10, 40, 90]), stops))
+
+    def params(n, stops):
+        return SamplingParams(max_tokens=n, temperature=0.0, stop_token_ids=stops, ignore_eos=True)
+
+    eng = make(num_blocks=140, max_seqs=12, prefix=True)
+    finals, aborted, live = {}, set(), []
+    arrivals = iter(requests)
+    while True:
+        for _ in range(rng.choice([0, 0, 1, 2])):
+            r = next(arrivals, None)
+            if r is not None:
+                eng.add_request(r[0], prompt_token_ids=r[1], sampling_params=params(r[2], r[3]))
+                live.append(r[0])
+        if live and rng.random() < 0.03:
+            victim = rng.choice(live)
+            eng.abort_request(victim)
+            aborted.add(victim)
+            live.remove(victim)
+        if not eng.has_unfinished_requests():
+            if len(finals) + len(aborted) == len(requests):
+                break
+            continue
+        for out in eng.step():
+            assert out.request_id not in aborted
+            if out.finished:
+                finals[out.request_id] = (out.token_ids, out.finish_reason)
+                live.remove(out.request_id)
+    stats = eng.stats()
+    assert stats["num_preempted_total"] > 0 and stats["lookahead_steps"] > 0 and stats["total_cached_tokens"] > 0
+    assert any(reason == "stop" for _, reason in finals.values())
+    eng.prefix_cache.reset()
+    assert eng.manager.min_free_blocks() == eng.manager.num_blocks
+    alone = make(num_blocks=200, max_seqs=2, prefix=False)
+    for rid, prompt, n, stops in requests:
+        if rid not in aborted:
+            out = alone.generate([prompt], params(n, stops))[0]
+            assert (out.token_ids, out.finish_reason) == finals[rid], rid
