@@ -9,45 +9,11 @@
 // result depends on that row, its seed and its draw index only.
 #include "common.h"
 
-#define SAMPLE_THREADS 1024
-#define SAMPLE_WAVES (SAMPLE_THREADS / 64)
 
 __device__ __forceinline__ uint32_t order_key(float x) {
   if (x != x) x = -INFINITY;
   const uint32_t u = __float_as_uint(x);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-
-__device__ __forceinline__ float block_sum(float v, float* red) {
-  v = cw_wave_sum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float t = 0.0f;
-#pragma unroll
-  for (int i = 0; i < SAMPLE_WAVES; ++i) t += red[i];
-  return t;
-}
-__device__ __forceinline__ float block_max(float v, float* red) {
-  v = cw_wave_max(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float t = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < SAMPLE_WAVES; ++i) t = fmaxf(t, red[i]);
-  return t;
-}
-__device__ __forceinline__ int block_sum_int(int v, int* red) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  int t = 0;
-#pragma unroll
-  for (int i = 0; i < SAMPLE_WAVES; ++i) t += red[i];
-  return t;
 }
 
 // ---------------------------------------------------------------- arg-max, two stages
@@ -144,158 +110,521 @@ __device__ __forceinline__ uint32_t philox_first_word(uint64_t seed, uint64_t co
   return c0;
 }
 
-// ---------------------------------------------------------------- sampling, one workgroup per row
-__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
-    const float* __restrict__ logits, int64_t row_stride, int V, const float* __restrict__ temperature,
-    const int* __restrict__ top_k, const float* __restrict__ top_p, const int64_t* __restrict__ seeds,
-    const int64_t* __restrict__ draws, int* __restrict__ out) {
-  __shared__ float red[SAMPLE_WAVES];
-  __shared__ int redi[SAMPLE_WAVES];
-  __shared__ float sums[SAMPLE_THREADS];
-  __shared__ int pick_thread;
-  __shared__ float pick_base;
-  const int row = blockIdx.x;
-  const int tid = threadIdx.x;
-  const float* x = logits + (int64_t)row * row_stride;
-  const float temp = temperature[row];
+// ---------------------------------------------------------------- sampling
+// A row is cut into chunks and every step of the selection is one small kernel over
+// (chunk, row), so a row's work is spread over many compute units and a step costs little more
+// than its launch; what a step needs of the step before it goes through the workspace: the
+// chunks add their histograms into the row's with integer atomics (a sum that no order changes),
+// and every workgroup of the next step reads that one histogram.
+//
+//   MAX      per chunk: the largest logit and its first index (greedy rows end here);
+//   TOPK 0-3 the k-th largest logit by radix selection, 8 bits of the order-preserving key a
+//            step: per chunk a histogram of the next byte among the keys that share the bytes
+//            found so far. Dividing by the temperature keeps the order, so the selection runs on
+//            the raw logits and the floor of what is kept is (k-th largest) / temperature:
+//            ties at the k-th value survive, also ties that the division makes;
+//   ZSUM     per chunk: the sum of the weights exp(logit / T - max) of what top-k left;
+//   TOPP 0-3 the same radix selection with weights instead of counts: the largest key K with
+//            weight(keys >= K) > top_p * total; everything from K up stays, i.e. a token stays
+//            while the tokens strictly more likely than it weigh <= top_p * total;
+//   SUMS     the chunk sums again with the final floor (rows with top-p only);
+//   LOCATE   u * total falls into a chunk, and in it on the first index whose running sum
+//            exceeds it.
+// Weights are integers, exp(.) * 2^40 rounded down: their sums do not depend on the order of
+// addition, so every comparison above gives the same answer however the row is cut and however
+// the additions are scheduled (LDS atomics included), run after run.
+#define SAMPLE_THREADS 256
+#define SAMPLE_MAX_CHUNKS 64
+#define SAMPLE_WEIGHT_SCALE 1099511627776.0f  // 2^40
 
-  if (!(temp > 0.0f)) {  // greedy row inside a sampled batch
-    float bv = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int i = tid; i < V; i += SAMPLE_THREADS) {
-      float v = x[i];
-      if (v != v) v = -INFINITY;
-      argmax_merge(bv, bi, v, i);
+typedef unsigned long long u64_t;
+
+struct SampleArgs {
+  const float* logits;
+  int64_t row_stride;
+  int n, V, chunks, per;
+  const float* temperature;
+  const int* top_k;
+  const float* top_p;
+  const int64_t* seeds;
+  const int64_t* draws;
+  int* out;
+  // workspace
+  float* pmax;       // [n][chunks]
+  int* pmax_i;       // [n][chunks]
+  uint32_t* hist_k;  // [4 steps][n][256], zeroed by the MAX step
+  u64_t* hist_p;     // [4 steps][n][256], zeroed by the MAX step
+  uint32_t* state_k; // [2][n][2]: key bits found so far, rank still to go
+  u64_t* state_p;    // [2][n][2]: key bits found so far, weight above them
+  uint32_t* floor_k; // [n] scaled-key floor after top-k
+  u64_t* psum;       // [n][chunks] chunk sums of weights
+};
+
+CW_EXPORT int cw_sample_chunks(int V) {
+  int c = (V + 2047) / 2048;
+  return c < 1 ? 1 : (c > SAMPLE_MAX_CHUNKS ? SAMPLE_MAX_CHUNKS : c);
+}
+
+CW_EXPORT int64_t cw_sample_workspace_bytes(int n, int V) {
+  const int64_t rc = (int64_t)n * cw_sample_chunks(V);
+  // hist_p, state_p, psum, the second psum with a floor per row; hist_k, state_k, floor_k, pmax, pmax_i
+  return 8 * (4 * (int64_t)n * 256 + 4 * (int64_t)n + rc + rc + n) + 4 * (4 * (int64_t)n * 256 + 4 * (int64_t)n + n + 2 * rc) + 64;
+}
+
+__device__ __forceinline__ float key_to_float(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+__device__ __forceinline__ bool row_has_top_k(const SampleArgs& a, int row) {
+  const int k = a.top_k[row];
+  return k > 0 && k < a.V;
+}
+__device__ __forceinline__ bool row_has_top_p(const SampleArgs& a, int row) { return a.top_p[row] < 1.0f; }
+__device__ __forceinline__ u64_t weight_of(float v, float mx) {
+  return (u64_t)(expf(v - mx) * SAMPLE_WEIGHT_SCALE);
+}
+
+// The row's largest logit (NaN counts as -inf) and its first index, from the chunk maxima: the
+// first wave takes a chunk a lane (there are at most 64), every thread gets the result.
+__device__ __forceinline__ void row_max(const SampleArgs& a, int row, float& bv, int& bi) {
+  __shared__ float best_v;
+  __shared__ int best_i;
+  if (threadIdx.x < 64) {
+    float v = -INFINITY;
+    int i = 0x7fffffff;
+    if ((int)threadIdx.x < a.chunks) {
+      v = a.pmax[row * a.chunks + threadIdx.x];
+      i = a.pmax_i[row * a.chunks + threadIdx.x];
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
-      const float ov = __shfl_xor(bv, off, 64);
-      const int oi = __shfl_xor(bi, off, 64);
-      argmax_merge(bv, bi, ov, oi);
+      const float ov = __shfl_xor(v, off, 64);
+      const int oi = __shfl_xor(i, off, 64);
+      argmax_merge(v, i, ov, oi);
     }
-    if ((tid & 63) == 0) { red[tid >> 6] = bv; redi[tid >> 6] = bi; }
+    if (threadIdx.x == 0) { best_v = v; best_i = i; }
+  }
+  __syncthreads();
+  bv = best_v;
+  bi = best_i;
+  __syncthreads();
+}
+
+// For every thread b < 256: suf = sum of the bins b..255 of a row's histogram (a scan through
+// LDS) and next = the bins above b.
+template <typename T>
+__device__ __forceinline__ T suffix_of_bins(const T* hist_row, T* sh, T& next) {
+  const int b = threadIdx.x;
+  const T t = hist_row[b];
+  __syncthreads();
+  sh[b] = t;
+  __syncthreads();
+  for (int off = 1; off < 256; off <<= 1) {
+    const T add = b + off < 256 ? sh[b + off] : (T)0;
     __syncthreads();
-    if (tid == 0) {
-      for (int w = 1; w < SAMPLE_WAVES; ++w) argmax_merge(bv, bi, red[w], redi[w]);
-      out[row] = bi < V ? bi : 0;
-    }
-    return;
+    sh[b] += add;
+    __syncthreads();
   }
+  const T suf = sh[b];
+  next = suf - t;
+  return suf;
+}
 
-  // ---- top-k: the k-th largest scaled logit, by bisection on the order-preserving key
-  uint32_t key_floor = 0u;  // tokens with key < key_floor are masked
-  const int k = top_k[row];
-  if (k > 0 && k < V) {
-    uint32_t K = 0u;
-    for (int b = 31; b >= 0; --b) {
-      const uint32_t cand = K | (1u << b);
-      int cnt = 0;
-      for (int i = tid; i < V; i += SAMPLE_THREADS) cnt += order_key(x[i] / temp) >= cand;
-      if (block_sum_int(cnt, redi) >= k) K = cand;
+// MAX
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_max_kernel(SampleArgs a) {
+  __shared__ float sv[SAMPLE_THREADS / 64];
+  __shared__ int si[SAMPLE_THREADS / 64];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  if (chunk == 0) {  // the row's histograms start at zero
+#pragma unroll
+    for (int step = 0; step < 4; ++step) {
+      a.hist_k[((int64_t)step * a.n + row) * 256 + threadIdx.x] = 0u;
+      a.hist_p[((int64_t)step * a.n + row) * 256 + threadIdx.x] = 0;
     }
-    key_floor = K;  // largest key with at least k tokens at or above it: the k-th largest
   }
-
-  // ---- maximum of what is left
-  float mx = -INFINITY;
-  for (int i = tid; i < V; i += SAMPLE_THREADS) {
-    const float v = x[i] / temp;
-    if (order_key(v) >= key_floor && v == v) mx = fmaxf(mx, v);
+  const int lo = chunk * a.per, hi = min(a.V, lo + a.per);
+  const float* x = a.logits + (int64_t)row * a.row_stride;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = lo + threadIdx.x; i < hi; i += SAMPLE_THREADS) {
+    float v = x[i];
+    if (v != v) v = -INFINITY;
+    argmax_merge(bv, bi, v, i);
   }
-  mx = block_max(mx, red);
-
-  // ---- top-p
-  const float p = top_p[row];
-  if (p < 1.0f) {
-    float z = 0.0f;
-    for (int i = tid; i < V; i += SAMPLE_THREADS) {
-      const float v = x[i] / temp;
-      if (order_key(v) >= key_floor) z += expf(v - mx);
-    }
-    z = block_sum(z, red);
-    const float limit = p * z;  // compare unnormalised masses with top_p * total
-    // largest key K with mass(keys > K) > limit; everything above it stays
-    uint32_t K = 0u;
-    bool any = false;
-    for (int b = 31; b >= 0; --b) {
-      const uint32_t cand = K | (1u << b);
-      float mass = 0.0f;
-      for (int i = tid; i < V; i += SAMPLE_THREADS) {
-        const float v = x[i] / temp;
-        const uint32_t key = order_key(v);
-        if (key > cand && key >= key_floor) mass += expf(v - mx);
-      }
-      if (block_sum(mass, red) > limit) { K = cand; any = true; }
-    }
-    if (!any) {
-      // is mass(keys > 0) > limit at all? if not, nothing is cut
-      float mass = 0.0f;
-      for (int i = tid; i < V; i += SAMPLE_THREADS) {
-        const float v = x[i] / temp;
-        const uint32_t key = order_key(v);
-        if (key > 0u && key >= key_floor) mass += expf(v - mx);
-      }
-      any = block_sum(mass, red) > limit;
-    }
-    if (any && K + 1u > key_floor) key_floor = K + 1u;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, 64);
+    const int oi = __shfl_xor(bi, off, 64);
+    argmax_merge(bv, bi, ov, oi);
   }
-
-  // ---- draw: weights in index order, thread t owns [t * per, (t + 1) * per)
-  const int per = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-  const int lo = min(V, tid * per), hi = min(V, lo + per);
-  float w = 0.0f;
-  for (int i = lo; i < hi; ++i) {
-    const float v = x[i] / temp;
-    if (order_key(v) >= key_floor) w += expf(v - mx);
-  }
-  sums[tid] = w;
+  if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
   __syncthreads();
-  if (tid == 0) {
-    float total = 0.0f;
-    for (int t = 0; t < SAMPLE_THREADS; ++t) total += sums[t];
-    const uint32_t r = philox_first_word((uint64_t)seeds[row], (uint64_t)draws[row]);
-    const float u = (float)(r >> 8) * (1.0f / 16777216.0f);
-    const float target = u * total;
-    float run = 0.0f;
-    int chosen = -1;
-    float base = 0.0f;
-    int last_nonzero = 0;
-    for (int t = 0; t < SAMPLE_THREADS; ++t) {
-      if (sums[t] > 0.0f) last_nonzero = t;
-      if (chosen < 0 && run + sums[t] > target && sums[t] > 0.0f) { chosen = t; base = run; }
-      run += sums[t];
-    }
-    if (chosen < 0) {  // target fell on the total through rounding: take the last weighted chunk
-      chosen = last_nonzero;
-      base = -INFINITY;
-    }
-    pick_thread = chosen;
-    pick_base = base;
-    sums[0] = target;
-  }
-  __syncthreads();
-  if (tid == pick_thread) {
-    const float target = sums[0];
-    float run = pick_base == -INFINITY ? 0.0f : pick_base;
-    int chosen = -1, last = lo;
-    for (int i = lo; i < hi; ++i) {
-      const float v = x[i] / temp;
-      if (order_key(v) < key_floor) continue;
-      const float e = expf(v - mx);
-      if (e > 0.0f) last = i;
-      run += e;
-      if (pick_base != -INFINITY && run > target && e > 0.0f) { chosen = i; break; }
-    }
-    out[row] = chosen >= 0 ? chosen : last;
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < SAMPLE_THREADS / 64; ++w) argmax_merge(bv, bi, sv[w], si[w]);
+    a.pmax[row * a.chunks + chunk] = bv;
+    a.pmax_i[row * a.chunks + chunk] = bi;
   }
 }
 
+// State of the top-k descent after `done` steps, from the state after done - 1 steps (in the
+// workspace, written by the step before) and that step's histograms: (key bits, rank to go).
+__device__ __forceinline__ void topk_state(const SampleArgs& a, int row, int done, uint32_t* sh, uint32_t& prefix,
+                                           uint32_t& rank) {
+  __shared__ uint32_t picked[2];
+  if (done == 0) {
+    prefix = 0u;
+    rank = (uint32_t)a.top_k[row];
+    return;
+  }
+  uint32_t p0 = 0u, r0 = (uint32_t)a.top_k[row];
+  if (done > 1) {
+    const uint32_t* st = a.state_k + ((int64_t)((done - 2) & 1) * a.n + row) * 2;
+    p0 = st[0];
+    r0 = st[1];
+  }
+  const uint32_t* hist = a.hist_k + ((int64_t)(done - 1) * a.n + row) * 256;
+  uint32_t above;
+  const uint32_t suf = suffix_of_bins<uint32_t>(hist, sh, above);
+  // the bin that holds the rank-th largest: at least `rank` keys from it up, fewer above it
+  if (suf >= r0 && above < r0) {
+    picked[0] = threadIdx.x;
+    picked[1] = r0 - above;
+  }
+  __syncthreads();
+  prefix = p0 | (picked[0] << (24 - 8 * (done - 1)));
+  rank = picked[1];
+  __syncthreads();
+}
+
+// TOPK step `step` (0..3): histogram of byte `step` of the raw keys that share the bytes found.
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_topk_kernel(SampleArgs a, int step) {
+  __shared__ uint32_t sh[256];
+  __shared__ uint32_t bins[SAMPLE_THREADS / 64][256];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  if (!(a.temperature[row] > 0.0f) || !row_has_top_k(a, row)) return;
+  uint32_t prefix, rank;
+  topk_state(a, row, step, sh, prefix, rank);
+  if (chunk == 0 && threadIdx.x == 0 && step > 0) {
+    uint32_t* st = a.state_k + ((int64_t)((step - 1) & 1) * a.n + row) * 2;
+    st[0] = prefix;
+    st[1] = rank;
+  }
+  for (int i = threadIdx.x; i < (SAMPLE_THREADS / 64) * 256; i += SAMPLE_THREADS) (&bins[0][0])[i] = 0u;
+  __syncthreads();
+  const int lo = chunk * a.per, hi = min(a.V, lo + a.per);
+  const float* x = a.logits + (int64_t)row * a.row_stride;
+  const int shift = 24 - 8 * step;
+  const uint32_t mask = step == 0 ? 0u : (0xffffffffu << (shift + 8));
+  uint32_t* mine = bins[threadIdx.x >> 6];
+  for (int i0 = lo + threadIdx.x; i0 < hi; i0 += 4 * SAMPLE_THREADS) {  // four loads in flight
+    float raw[4];
+    bool in[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      in[u] = i0 + u * SAMPLE_THREADS < hi;
+      raw[u] = in[u] ? x[i0 + u * SAMPLE_THREADS] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t key = order_key(raw[u]);
+      if (in[u] && (key & mask) == prefix) atomicAdd(&mine[(key >> shift) & 255u], 1u);
+    }
+  }
+  __syncthreads();
+  uint32_t t = 0u;
+#pragma unroll
+  for (int w = 0; w < SAMPLE_THREADS / 64; ++w) t += bins[w][threadIdx.x];
+  if (t) atomicAdd(&a.hist_k[((int64_t)step * a.n + row) * 256 + threadIdx.x], t);
+}
+
+// The floor top-k leaves, as a key of the scaled logits (0: nothing is cut). Every thread of the
+// workgroup gets it; after ZSUM it is in the workspace.
+__device__ __forceinline__ uint32_t topk_floor(const SampleArgs& a, int row, float temp, uint32_t* sh) {
+  if (!row_has_top_k(a, row)) return 0u;
+  uint32_t key, rank;
+  topk_state(a, row, 4, sh, key, rank);
+  return order_key(key_to_float(key) / temp);
+}
+
+// Sum of the weights of the chunk's kept tokens, every thread gets it.
+__device__ __forceinline__ u64_t chunk_weight(const SampleArgs& a, int row, int chunk, float temp, float mx,
+                                              uint32_t floor_key, u64_t* red) {
+  const int lo = chunk * a.per, hi = min(a.V, lo + a.per);
+  const float* x = a.logits + (int64_t)row * a.row_stride;
+  u64_t w = 0;
+  for (int i0 = lo + threadIdx.x; i0 < hi; i0 += 4 * SAMPLE_THREADS) {  // four loads in flight
+    float raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) raw[u] = i0 + u * SAMPLE_THREADS < hi ? x[i0 + u * SAMPLE_THREADS] : NAN;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float v = raw[u] / temp;
+      if (v == v && order_key(v) >= floor_key) w += weight_of(v, mx);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) w += __shfl_xor(w, off, 64);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = w;
+  __syncthreads();
+  u64_t t = 0;
+#pragma unroll
+  for (int i = 0; i < SAMPLE_THREADS / 64; ++i) t += red[i];
+  return t;
+}
+
+// ZSUM
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_zsum_kernel(SampleArgs a) {
+  __shared__ uint32_t sh[256];
+  __shared__ u64_t red[SAMPLE_THREADS / 64];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const float temp = a.temperature[row];
+  if (!(temp > 0.0f)) return;
+  const uint32_t floor_key = topk_floor(a, row, temp, sh);
+  if (chunk == 0 && threadIdx.x == 0) a.floor_k[row] = floor_key;
+  float mraw;
+  int mi;
+  row_max(a, row, mraw, mi);
+  const u64_t w = chunk_weight(a, row, chunk, temp, mraw / temp, floor_key, red);
+  if (threadIdx.x == 0) a.psum[row * a.chunks + chunk] = w;
+}
+
+// State of the top-p descent after `done` steps: (key bits, weight of the keys above them).
+__device__ __forceinline__ void topp_state(const SampleArgs& a, int row, int done, u64_t limit, u64_t* sh,
+                                           uint32_t& prefix, u64_t& above_all) {
+  __shared__ u64_t picked[2];
+  if (done == 0) {
+    prefix = 0u;
+    above_all = 0;
+    return;
+  }
+  uint32_t p0 = 0u;
+  u64_t a0 = 0;
+  if (done > 1) {
+    const u64_t* st = a.state_p + ((int64_t)((done - 2) & 1) * a.n + row) * 2;
+    p0 = (uint32_t)st[0];
+    a0 = st[1];
+  }
+  const u64_t* hist = a.hist_p + ((int64_t)(done - 1) * a.n + row) * 256;
+  u64_t above;
+  const u64_t suf = suffix_of_bins<u64_t>(hist, sh, above);
+  // the largest byte b with weight(keys >= (bytes so far, b, 0...)) > limit
+  if (a0 + suf > limit && !(a0 + above > limit)) {
+    picked[0] = threadIdx.x;
+    picked[1] = a0 + above;
+  }
+  __syncthreads();
+  prefix = p0 | ((uint32_t)picked[0] << (24 - 8 * (done - 1)));
+  above_all = picked[1];
+  __syncthreads();
+}
+
+// Sum of a row's chunk sums (order does not matter: integers); every thread gets it.
+__device__ __forceinline__ u64_t row_total(const u64_t* sums, int chunks) {
+  __shared__ u64_t total;
+  if (threadIdx.x < 64) {
+    u64_t t = (int)threadIdx.x < chunks ? sums[threadIdx.x] : 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
+    if (threadIdx.x == 0) total = t;
+  }
+  __syncthreads();
+  const u64_t t = total;
+  __syncthreads();
+  return t;
+}
+__device__ __forceinline__ u64_t topp_limit(float p, u64_t total) { return (u64_t)((double)p * (double)total); }
+
+// TOPP step `step` (0..3): weight per value of byte `step` among the kept raw keys that share
+// the bytes found so far.
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_topp_kernel(SampleArgs a, int step) {
+  __shared__ u64_t sh[256];
+  __shared__ u64_t bins[SAMPLE_THREADS / 64][256];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const float temp = a.temperature[row];
+  if (!(temp > 0.0f) || !row_has_top_p(a, row)) return;
+  const u64_t limit = topp_limit(a.top_p[row], row_total(a.psum + row * a.chunks, a.chunks));
+  uint32_t prefix;
+  u64_t above;
+  topp_state(a, row, step, limit, sh, prefix, above);
+  if (chunk == 0 && threadIdx.x == 0 && step > 0) {
+    u64_t* st = a.state_p + ((int64_t)((step - 1) & 1) * a.n + row) * 2;
+    st[0] = prefix;
+    st[1] = above;
+  }
+  for (int i = threadIdx.x; i < (SAMPLE_THREADS / 64) * 256; i += SAMPLE_THREADS) (&bins[0][0])[i] = 0;
+  __syncthreads();
+  float mraw;
+  int mi;
+  row_max(a, row, mraw, mi);
+  const float mx = mraw / temp;
+  const uint32_t floor_key = a.floor_k[row];
+  const int lo = chunk * a.per, hi = min(a.V, lo + a.per);
+  const float* x = a.logits + (int64_t)row * a.row_stride;
+  const int shift = 24 - 8 * step;
+  const uint32_t mask = step == 0 ? 0u : (0xffffffffu << (shift + 8));
+  u64_t* mine = bins[threadIdx.x >> 6];
+  for (int i0 = lo + threadIdx.x; i0 < hi; i0 += 4 * SAMPLE_THREADS) {  // four loads in flight
+    float raws[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) raws[u] = i0 + u * SAMPLE_THREADS < hi ? x[i0 + u * SAMPLE_THREADS] : NAN;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float raw = raws[u];
+      const uint32_t key = order_key(raw);
+      if (raw != raw || (key & mask) != prefix) continue;
+      const float v = raw / temp;
+      if (v == v && order_key(v) >= floor_key) atomicAdd(&mine[(key >> shift) & 255u], weight_of(v, mx));
+    }
+  }
+  __syncthreads();
+  u64_t t = 0;
+#pragma unroll
+  for (int w = 0; w < SAMPLE_THREADS / 64; ++w) t += bins[w][threadIdx.x];
+  if (t) atomicAdd(&a.hist_p[((int64_t)step * a.n + row) * 256 + threadIdx.x], t);
+}
+
+// SUMS: the chunk sums with the floor that top-p adds (rows with top-p).
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_sums_kernel(SampleArgs a, u64_t* psum_out) {
+  __shared__ u64_t sh[256];
+  __shared__ u64_t red[SAMPLE_THREADS / 64];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const float temp = a.temperature[row];
+  if (!(temp > 0.0f) || !row_has_top_p(a, row)) return;
+  const u64_t limit = topp_limit(a.top_p[row], row_total(a.psum + row * a.chunks, a.chunks));
+  uint32_t key;
+  u64_t above;
+  topp_state(a, row, 4, limit, sh, key, above);
+  uint32_t floor_key = order_key(key_to_float(key) / temp);
+  if (floor_key < a.floor_k[row]) floor_key = a.floor_k[row];
+  float mraw;
+  int mi;
+  row_max(a, row, mraw, mi);
+  const u64_t w = chunk_weight(a, row, chunk, temp, mraw / temp, floor_key, red);
+  if (threadIdx.x == 0) {
+    psum_out[row * a.chunks + chunk] = w;
+    if (chunk == 0) psum_out[(int64_t)a.n * a.chunks + row] = floor_key;  // for LOCATE
+  }
+}
+
+// LOCATE: one workgroup per row.
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_locate_kernel(SampleArgs a, const u64_t* psum2) {
+  __shared__ u64_t scan[SAMPLE_THREADS];
+  __shared__ int found;
+  const int row = blockIdx.x;
+  const float temp = a.temperature[row];
+  float mraw;
+  int mi;
+  row_max(a, row, mraw, mi);
+  if (!(temp > 0.0f)) {  // greedy row inside a sampled batch
+    if (threadIdx.x == 0) a.out[row] = mi < a.V ? mi : 0;
+    return;
+  }
+  const bool with_p = row_has_top_p(a, row);
+  const u64_t* sums = (with_p ? psum2 : a.psum) + row * a.chunks;
+  const uint32_t floor_key = with_p ? (uint32_t)psum2[(int64_t)a.n * a.chunks + row] : a.floor_k[row];
+  const u64_t total = row_total(sums, a.chunks);
+  const uint32_t r = philox_first_word((uint64_t)a.seeds[row], (uint64_t)a.draws[row]);
+  // u = (r >> 8) / 2^24; the drawn token is the first whose running weight exceeds u * total
+  u64_t target = (u64_t)((double)(r >> 8) * (1.0 / 16777216.0) * (double)total);
+  if (target >= total) target = total - 1;  // (total >= 2^40: the largest logit weighs that much)
+  // the chunk the target falls into: a running sum over the chunks in the first wave
+  __shared__ int sel_chunk;
+  __shared__ u64_t sel_base;
+  if (threadIdx.x < 64) {
+    const u64_t v = (int)threadIdx.x < a.chunks ? sums[threadIdx.x] : 0;
+    u64_t incl = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const u64_t up = __shfl_up(incl, off, 64);
+      if ((int)threadIdx.x >= off) incl += up;
+    }
+    if (v > 0 && incl - v <= target && target < incl) {
+      sel_chunk = threadIdx.x;
+      sel_base = incl - v;
+    }
+  }
+  __syncthreads();
+  const int chunk = sel_chunk;
+  const u64_t base = sel_base;
+  // in the chunk: thread t owns a run of consecutive tokens
+  const float mx = mraw / temp;
+  const int lo = chunk * a.per, hi = min(a.V, lo + a.per);
+  const int run = (hi - lo + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int my_lo = min(hi, lo + (int)threadIdx.x * run), my_hi = min(hi, my_lo + run);
+  const float* x = a.logits + (int64_t)row * a.row_stride;
+  u64_t w = 0;
+  for (int i = my_lo; i < my_hi; ++i) {
+    const float v = x[i] / temp;
+    if (v == v && order_key(v) >= floor_key) w += weight_of(v, mx);
+  }
+  scan[threadIdx.x] = w;
+  if (threadIdx.x == 0) found = -1;
+  __syncthreads();
+  for (int off = 1; off < SAMPLE_THREADS; off <<= 1) {  // inclusive scan
+    const u64_t add = threadIdx.x >= off ? scan[threadIdx.x - off] : 0;
+    __syncthreads();
+    scan[threadIdx.x] += add;
+    __syncthreads();
+  }
+  const u64_t incl = base + scan[threadIdx.x], excl = incl - w;
+  if (w > 0 && excl <= target && target < incl) {
+    u64_t at = excl;
+    int chosen = my_lo;
+    for (int i = my_lo; i < my_hi; ++i) {
+      const float v = x[i] / temp;
+      if (!(v == v && order_key(v) >= floor_key)) continue;
+      const u64_t q = weight_of(v, mx);
+      if (q == 0) continue;
+      chosen = i;
+      at += q;
+      if (at > target) break;
+    }
+    found = chosen;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) a.out[row] = found >= 0 ? found : (mi < a.V ? mi : 0);
+}
+
+// flags: bit 0 some row may have top-k, bit 1 some row may have top-p (3 when unknown): the
+// steps no row needs are not launched. workspace: cw_sample_workspace_bytes(n, V) bytes, 16-byte
+// aligned.
 CW_EXPORT int cw_sample(const float* logits, int64_t row_stride, int n, int V,
                         const float* temperature, const int* top_k, const float* top_p,
-                        const int64_t* seeds, const int64_t* draws, int* out, hipStream_t stream) {
+                        const int64_t* seeds, const int64_t* draws, int* out, void* workspace,
+                        int64_t workspace_bytes, int flags, hipStream_t stream) {
   if (n < 0 || V <= 0 || row_stride < V) return CW_ERR_ARG;
   if (n == 0) return CW_OK;
-  hipLaunchKernelGGL(sample_kernel, dim3(n), dim3(SAMPLE_THREADS), 0, stream, logits, row_stride, V,
-                     temperature, top_k, top_p, seeds, draws, out);
+  if (n > 65535) return CW_ERR_SIZE;
+  if (workspace == nullptr || ((uintptr_t)workspace & 15) || workspace_bytes < cw_sample_workspace_bytes(n, V))
+    return CW_ERR_ARG;
+  SampleArgs a;
+  a.logits = logits; a.row_stride = row_stride; a.n = n; a.V = V;
+  a.chunks = cw_sample_chunks(V);
+  a.per = (V + a.chunks - 1) / a.chunks;
+  a.temperature = temperature; a.top_k = top_k; a.top_p = top_p; a.seeds = seeds; a.draws = draws; a.out = out;
+  const int64_t rc = (int64_t)n * a.chunks;
+  // 8-byte items first
+  u64_t* p8 = (u64_t*)workspace;
+  a.hist_p = p8; p8 += 4 * (int64_t)n * 256;
+  a.state_p = p8; p8 += (int64_t)n * 4;
+  a.psum = p8; p8 += rc;
+  u64_t* psum2 = p8; p8 += rc + n;
+  uint32_t* p4 = (uint32_t*)p8;
+  a.hist_k = p4; p4 += 4 * (int64_t)n * 256;
+  a.state_k = p4; p4 += (int64_t)n * 4;
+  a.floor_k = p4; p4 += n;
+  a.pmax = (float*)p4; p4 += rc;
+  a.pmax_i = (int*)p4; p4 += rc;
+  if ((char*)p4 > (char*)workspace + workspace_bytes) return CW_ERR_ARG;
+  const dim3 grid(a.chunks, n), block(SAMPLE_THREADS);
+  hipLaunchKernelGGL(sample_max_kernel, grid, block, 0, stream, a);
+  if (flags & 1)
+    for (int step = 0; step < 4; ++step) hipLaunchKernelGGL(sample_topk_kernel, grid, block, 0, stream, a, step);
+  hipLaunchKernelGGL(sample_zsum_kernel, grid, block, 0, stream, a);
+  if (flags & 2) {
+    for (int step = 0; step < 4; ++step) hipLaunchKernelGGL(sample_topp_kernel, grid, block, 0, stream, a, step);
+    hipLaunchKernelGGL(sample_sums_kernel, grid, block, 0, stream, a, psum2);
+  }
+  hipLaunchKernelGGL(sample_locate_kernel, dim3(n), block, 0, stream, a, psum2);
   return cw_launch_status();
 }

@@ -107,7 +107,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
         "sampling": {
             "cw_argmax_chunks": [I],
             "cw_argmax": [P, L, I, I, P, P, L, P],
-            "cw_sample": [P, L, I, I, P, P, P, P, P, P, P],
+            "cw_sample": [P, L, I, I, P, P, P, P, P, P, P, L, I, P],
+            "cw_sample_workspace_bytes": [I, I],
         },
         "attention": {
             "cw_attention_head_dim": [],
@@ -125,7 +126,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
     for fn, argtypes in sigs.items():
         f = getattr(lib, fn)
         f.argtypes = argtypes
-        f.restype = c_int64 if fn.endswith("workspace_floats") else c_int
+        f.restype = c_int64 if fn.endswith(("workspace_floats", "workspace_bytes")) else c_int
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -664,8 +665,11 @@ def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tenso
     return out
 
 
-def sample(logits, temperature, top_k, top_p, seeds, draws, out=None) -> torch.Tensor:
-    """One token per row: rows with temperature 0 take the arg-max, the others are drawn."""
+def sample(logits, temperature, top_k, top_p, seeds, draws, out=None, any_top_k: bool = True,
+           any_top_p: bool = True) -> torch.Tensor:
+    """One token per row: rows with temperature 0 take the arg-max, the others are drawn.
+    ``any_top_k`` / ``any_top_p`` off: the caller knows that no row has that option, and its
+    kernels are not launched."""
     _gpu(logits, temperature, top_k, top_p, seeds, draws, out)
     _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be float32 [n, V]")
     n, V = logits.shape
@@ -677,9 +681,11 @@ def sample(logits, temperature, top_k, top_p, seeds, draws, out=None) -> torch.T
     if out is None:
         out = torch.empty(n, dtype=torch.int32, device=logits.device)
     _i32(out, n, "out")
+    lib = _load("sampling")
+    ws = torch.empty(int(lib.cw_sample_workspace_bytes(n, V)), dtype=torch.uint8, device=logits.device)
     _check(
-        _load("sampling").cw_sample(_ptr(logits), V, n, V, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds),
-                                    _ptr(draws), _ptr(out), _stream()),
+        lib.cw_sample(_ptr(logits), V, n, V, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds), _ptr(draws),
+                      _ptr(out), _ptr(ws), ws.numel(), int(bool(any_top_k)) | (int(bool(any_top_p)) << 1), _stream()),
         "sample",
     )
     return out

@@ -51,5 +51,6 @@ class Sampler:
         draws = torch.tensor([len(s.output_token_ids) + pending for s in seqs], dtype=torch.int64)
         dev = self.device
         return ops.sample(
-            logits, temperature.to(dev), top_k.to(dev), top_p.to(dev), seeds.to(dev), draws.to(dev)
+            logits, temperature.to(dev), top_k.to(dev), top_p.to(dev), seeds.to(dev), draws.to(dev),
+            any_top_k=bool((top_k > 0).any()), any_top_p=bool((top_p < 1.0).any()),
         )

@@ -831,11 +831,16 @@ def test_argmax_first_index_wins(n, V):
     assert got[0] == V // 2
 
 
-def test_sampling_matches_plain_definition():
+@pytest.mark.parametrize("V,scale", [(1000, 3.0), (4099, 1.0), (151936, 3.0), (151936, 0.3)])
+def test_sampling_matches_plain_definition(V, scale):
+    """Every combination of temperature, top-k and top-p against the plain definition with the same
+    uniform number; a vocabulary of the model's size (a row is cut into chunks), one that no chunk
+    size divides, peaked and nearly flat rows."""
     from clockwork_amd import ops
 
-    V, n = 1000, 24
-    logits = 3 * torch.randn(n, V, device=DEV)
+    n = 24
+    logits = scale * torch.randn(n, V, device=DEV)
+    logits[3, 7] = logits[3, V - 5] = logits[3].max() + 1.0  # equal maxima
     temps = torch.tensor([0.0, 0.8, 1.5, 1.0] * 6, device=DEV)
     top_k = torch.tensor(([-1] * 4 + [5] * 4 + [1] * 4 + [-1] * 4 + [50] * 4 + [V] * 4), dtype=torch.int32, device=DEV)
     top_p = torch.tensor(([1.0] * 12 + [0.9] * 4 + [0.5] * 4 + [0.05] * 4), device=DEV)
@@ -853,6 +858,36 @@ def test_sampling_matches_plain_definition():
         assert got[i] == want or margin < 1e-4, f"row {i}: got {got[i]}, plain draws {want} (margin {margin})"
         if int(top_k[i]) == 1:
             assert got[i] == int(logits[i].argmax())  # tests/test_server.py:323
+    # the caller may say that no row has an option: the same tokens without those kernels
+    plain_rows = [i for i in range(n) if int(top_k[i]) in (-1, V) and float(top_p[i]) == 1.0]
+    sel = torch.tensor(plain_rows, device=DEV)
+    again = ops.sample(logits[sel].contiguous(), temps[sel], top_k[sel], top_p[sel], seeds[sel], draws[sel],
+                       any_top_k=False, any_top_p=False).tolist()
+    assert again == [got[i] for i in plain_rows]
+
+
+def test_sampling_keeps_exactly_the_top_k_and_the_nucleus():
+    """Many draws from one row: every token of the kept set comes up and no other does (a selection
+    that is off by one place shows here, not in single draws)."""
+    from clockwork_amd import ops
+
+    V, n = 3000, 6000
+    row = torch.randn(V, device=DEV)
+    row[torch.randperm(V, device=DEV)[:12]] += 6.0  # a dozen likely tokens
+    logits = row.repeat(n, 1)
+    seeds = torch.full((n,), 5, dtype=torch.int64, device=DEV)
+    draws = torch.arange(n, dtype=torch.int64, device=DEV)
+    ones = torch.ones(n, device=DEV)
+    for k, p in ((8, 1.0), (-1, 0.6), (10, 0.8)):
+        got = ops.sample(logits, ones, torch.full((n,), k, dtype=torch.int32, device=DEV), p * ones, seeds, draws)
+        probs = plain.sampling_probs(row.cpu(), 1.0, k, p)
+        kept = set(torch.nonzero(probs > 0).flatten().tolist())
+        seen = set(got.tolist())
+        assert seen <= kept
+        likely = {i for i in kept if float(probs[i]) > 5.0 / n}
+        assert likely <= seen
+        freq = torch.bincount(got.long(), minlength=V).float().cpu() / n
+        assert float((freq - probs.float()).abs().max()) < 0.03
 
 
 def test_sampling_is_reproducible_and_follows_the_distribution():
