@@ -73,8 +73,9 @@ def build_runner(args, prefix_cache: bool = False, max_batch: int = 0):
     return cfg, runner
 
 
-def time_decode(cfg, runner, batch: int, steps: int, warmup: int):
-    """Prefill ``batch`` prompts of PROMPT_LEN tokens, then time ``steps`` decode steps."""
+def time_decode(cfg, runner, batch: int, steps: int, warmup: int, sampling=None):
+    """Prefill ``batch`` prompts of PROMPT_LEN tokens, then time ``steps`` decode steps.
+    ``sampling``: (temperature, top_k, top_p) instead of greedy."""
     import torch
 
     from clockwork_amd.engine.llm_engine import LLMEngine
@@ -83,8 +84,10 @@ def time_decode(cfg, runner, batch: int, steps: int, warmup: int):
     engine = LLMEngine(cfg, runner=runner)
     gen = torch.Generator().manual_seed(batch)
     vocab = runner.spec.vocab_size
-    params = SamplingParams(max_tokens=warmup + steps + batch + 2, temperature=0.0, ignore_eos=True)
+    temperature, top_k, top_p = sampling or (0.0, -1, 1.0)
     for i in range(batch):
+        params = SamplingParams(max_tokens=warmup + steps + batch + 2, temperature=temperature, top_k=top_k, top_p=top_p,
+                                seed=i, ignore_eos=True)
         engine.add_request(f"b{batch}-{i}", prompt_token_ids=torch.randint(0, vocab, (PROMPT_LEN,), generator=gen).tolist(),
                            sampling_params=params)
     while any(s.is_prefilling() or s.num_computed_tokens == 0 for s in engine.scheduler.running + engine.scheduler.waiting):
@@ -277,6 +280,9 @@ def main() -> int:
                     help="decode: the recorded benchmark; mixed: a continuous batch of --requests prompts of mixed lengths")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--peaks", action="store_true", help="measure a device copy and a large library product instead")
+    ap.add_argument("--temperature", type=float, default=0.0, help="sample instead of the greedy decoding of the recorded benchmark")
+    ap.add_argument("--top-k", type=int, default=-1)
+    ap.add_argument("--top-p", type=float, default=1.0)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
@@ -295,7 +301,8 @@ def main() -> int:
         t = time_prefill(cfg, runner)
         print(json.dumps({"prefill_ms": round(1e3 * t, 3), "tokens_per_s": round(PROMPT_LEN / t, 1)}))
         return 0
-    elapsed, mean_ctx = time_decode(cfg, runner, args.batch, args.steps, args.warmup)
+    sampling = (args.temperature, args.top_k, args.top_p) if args.temperature > 0 else None
+    elapsed, mean_ctx = time_decode(cfg, runner, args.batch, args.steps, args.warmup, sampling)
     value = args.batch * args.steps / elapsed
     ms = 1e3 * elapsed / args.steps
     step_bytes = runner.model.weight_bytes_per_step() + args.batch * mean_ctx * runner.pools.kv_bytes_per_token()
@@ -329,7 +336,7 @@ def main() -> int:
             "prompt_len": PROMPT_LEN,
             "seq_len": CONTEXT,
             "block_size": BLOCK,
-            "sampling": "greedy",
+            "sampling": "greedy" if sampling is None else f"temperature {args.temperature} top_k {args.top_k} top_p {args.top_p}",
             "parallelism": "single GPU",
         },
         "roofline": {
@@ -351,7 +358,7 @@ def main() -> int:
         }
         points = {}
         for b in (1, 64):
-            e, _ = time_decode(cfg, runner, b, args.steps, args.warmup)
+            e, _ = time_decode(cfg, runner, b, args.steps, args.warmup, sampling)
             points[f"decode_b{b}"] = round(b * args.steps / e, 1)
         record["points"] = points
     print(json.dumps(record))
