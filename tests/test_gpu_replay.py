@@ -245,6 +245,46 @@ def test_graph_replays_equal_eager_steps(model_dirs, dtype):
     replay.compare(got_g, ref, **TOL[dtype])
 
 
+@pytest.mark.parametrize("tuned", [False, True])
+def test_wide_decode_batches_of_a_large_layer_replay_as_eager(tmp_path, tuned):
+    """40 requests decoding together through one layer of the 7B shape: at this width some products
+    are library products inside the captured graph (also a kernel the library's tuning picked,
+    which may clear a workspace before it runs). Every replay, with eager steps of another batch
+    size and synchronisations in between, must equal the same step of a runner without graphs."""
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests import configs
+
+    config = configs.LAYER_7B
+    model_dir = write_random_model(tmp_path / "layer7b", config, 3)
+    gen = torch.Generator().manual_seed(5)
+    n_req, prompt, decode = 40, 6, 7
+    toks = {f"r{i}": torch.randint(0, config["vocab_size"], (prompt + decode,), generator=gen).tolist() for i in range(n_req)}
+    # 40 rows a step (a graph of 48), now and then only the first 19 (one of 24): a request left
+    # out of a step simply goes on later
+    fixed = [{"entries": [{"id": rid, "tokens": t[:prompt], "want": []} for rid, t in toks.items()], "end": []}]
+    at = {rid: prompt for rid in toks}
+    for d in range(decode):
+        ids = list(toks) if d % 3 != 2 else list(toks)[:19]
+        fixed.append({"entries": [{"id": rid, "tokens": toks[rid][at[rid] : at[rid] + 1], "want": [0]} for rid in ids], "end": []})
+        for rid in ids:
+            at[rid] += 1
+    pages = n_req * 2 + 4
+    with_graphs = replay.make_runner(model_dir, "bfloat16", 16, pages, use_graphs=True)
+    eager = replay.make_runner(model_dir, "bfloat16", 16, pages, use_graphs=False)
+    if tuned:
+        assert with_graphs.tune_products([48, 24]) == [48, 24]
+    got_g = replay.run_trace(with_graphs, [dict(s) for s in fixed])
+    got_e = replay.run_trace(eager, [dict(s) for s in fixed])
+    captured = [k for k, v in with_graphs._graphs.items() if isinstance(v, tuple)]
+    assert {size for size, _ in captured} == {48, 24}
+    assert got_g.keys() == got_e.keys() and len(got_g) > 200
+    scale = torch.stack(list(got_e.values())).square().mean().sqrt().item()
+    for key in got_e:
+        assert not torch.isnan(got_g[key]).any()
+        # the same kernels in the same order; only the attention splits are planned for the padded batch
+        assert (got_g[key] - got_e[key]).abs().max().item() < 2e-2 * scale, f"graph replay differs from the eager step at {key}"
+
+
 def test_negative_control_a_small_weight_change_breaks_the_match(model_dirs, tmp_path):
     """tests/test_hf_equivalence.py:141-153: the 1e-5 bar must bite. One q_proj row of layer 1
     moved by 2^-7 is far more than the bar allows."""
