@@ -160,3 +160,17 @@ def test_attention_spec_refuses_sizes_the_kernels_do_not_take():
     with pytest.raises(ValueError, match="not a multiple"):
         AttentionSpec(64, 5, 2, 16, True, False, 1.0)
     assert KVPagesSpec(2, 16).group_key() != KVPagesSpec(2, 16, window=8).group_key()
+
+
+def test_bench_refuses_more_than_one_gpu_with_one_line():
+    """The benchmark is a one-GPU program: asked for more it says so in one line and exits with 2,
+    before anything touches a GPU."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parent.parent
+    run = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2", "--steps", "3", "--warmup", "1"],
+                         capture_output=True, text=True, timeout=120)
+    assert run.returncode == 2
+    assert len(run.stdout.strip().splitlines()) == 1 and "one GPU" in run.stdout
