@@ -871,6 +871,7 @@ def test_sampling_keeps_exactly_the_top_k_and_the_nucleus():
     that is off by one place shows here, not in single draws)."""
     from clockwork_amd import ops
 
+    torch.manual_seed(77)  # the same row every run: what must be seen below depends on it
     V, n = 3000, 6000
     row = torch.randn(V, device=DEV)
     row[torch.randperm(V, device=DEV)[:12]] += 6.0  # a dozen likely tokens
@@ -884,7 +885,7 @@ def test_sampling_keeps_exactly_the_top_k_and_the_nucleus():
         kept = set(torch.nonzero(probs > 0).flatten().tolist())
         seen = set(got.tolist())
         assert seen <= kept
-        likely = {i for i in kept if float(probs[i]) > 5.0 / n}
+        likely = {i for i in kept if float(probs[i]) > 20.0 / n}  # missed with probability e^-20
         assert likely <= seen
         freq = torch.bincount(got.long(), minlength=V).float().cpu() / n
         assert float((freq - probs.float()).abs().max()) < 0.03
