@@ -810,13 +810,15 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 template <int HD, int RB>
 struct PrefillTile {
   static_assert(RB == 4 || (RB == 2 && HD <= 128), "two row blocks only with the eight-wave workgroup");
-  static constexpr int KROW = HD + 8;   // K rows: 16 bytes of padding spread the 16-byte reads over the banks
-  static constexpr int VROW = HD + 16;  // V rows: 32 bytes, for the 8-byte transposing reads
+  // The K tile lies in LDS as HD / 32 blocks of [key][32 elements]: the 64 lanes of a fragment
+  // read (16 keys x 4 slots of 8 elements) and of a stash store (16 keys x 4 chunks) then touch
+  // 1 KB without a gap, so no bank is hit twice and the rows need no padding.
+  static constexpr int VROW = HD + 16;  // V rows: 32 bytes of padding, for the 8-byte transposing reads
   static constexpr int NH = HD <= 128 ? 8 / RB : 1;  // waves that share a row block and split its keys
   static constexpr int KW = HD <= 128 ? 128 / NH : 32;  // keys a wave takes from a stage
   static constexpr int KT = KW * NH;            // keys of one stage
   static constexpr int NT = 64 * RB * NH;       // threads of a workgroup
-  static constexpr int STAGE = KT * (KROW + VROW);  // elements of one stage: a K tile, then a V tile
+  static constexpr int STAGE = KT * (HD + VROW);  // elements of one stage: a K tile, then a V tile
   static constexpr size_t BYTES = 2 * STAGE * sizeof(bf16_t);
   static constexpr int TABLE = 2048;  // block-table entries held in LDS at a time
   // what the sets of waves exchange at the end: accumulators, then maxima and sums
@@ -830,7 +832,7 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
   using Tile = PrefillTile<HD, RB>;
   constexpr int NF = HD / 32;     // k-steps of the score product
   constexpr int ND = HD / 16;     // 16-wide blocks of the head dimension
-  constexpr int KROW = Tile::KROW, VROW = Tile::VROW;
+  constexpr int VROW = Tile::VROW;
   constexpr int CPR = HD / 8;     // 16-byte chunks of a row
   constexpr int NH = Tile::NH, KW = Tile::KW, KT = Tile::KT, NT = Tile::NT;
   constexpr int NKB = KW / 16;  // 16-key blocks of a wave's keys
@@ -930,12 +932,13 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
     }
   };
   auto stash = [&](int stage) __attribute__((always_inline)) {  // registers -> LDS
-    bf16_t* ks = tiles + stage * Tile::STAGE + f_key * KROW + f_ch * 8;
-    bf16_t* vs = tiles + stage * Tile::STAGE + KT * KROW + f_key * VROW + f_ch * 8;
+    bf16_t* ks = tiles + stage * Tile::STAGE + f_key * 32;
+    bf16_t* vs = tiles + stage * Tile::STAGE + KT * HD + f_key * VROW + f_ch * 8;
 #pragma unroll
     for (int i = 0; i < NCK; ++i) {
       if (CPR % TPK == 0 || f_ch + i * TPK < CPR) {
-        *reinterpret_cast<u32x4_t*>(ks + i * TPK * 8) = gk[i];
+        const int ch = f_ch + i * TPK;  // 16-byte chunk of the row: block ch / 4, place ch % 4
+        *reinterpret_cast<u32x4_t*>(ks + (ch >> 2) * (KT * 32) + (ch & 3) * 8) = gk[i];
         *reinterpret_cast<u32x4_t*>(vs + i * TPK * 8) = gv[i];
       }
     }
@@ -959,8 +962,8 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
     }
     const bool active = wave_on && kv0 <= p_last && kv0 + KW - 1 >= lo;
     if (active) {
-      const bf16_t* ks = tiles + stage * Tile::STAGE + half * KW * KROW;
-      const bf16_t* vs = tiles + stage * Tile::STAGE + KT * KROW + half * KW * VROW;
+      const bf16_t* ks = tiles + stage * Tile::STAGE + half * KW * 32;
+      const bf16_t* vs = tiles + stage * Tile::STAGE + KT * HD + half * KW * VROW;
       // ---- S^T = K Q^T
       f32x4_t sc[NKB][2];
 #pragma unroll
@@ -968,7 +971,7 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
         bf16x8_t kf[NF];
 #pragma unroll
         for (int j = 0; j < NF; ++j)
-          kf[j] = *reinterpret_cast<const bf16x8_t*>(ks + (kb * 16 + c) * KROW + (j * 4 + s) * 8);
+          kf[j] = *reinterpret_cast<const bf16x8_t*>(ks + j * (KT * 32) + (kb * 16 + c) * 32 + s * 8);
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
           sc[kb][b] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};

@@ -281,8 +281,14 @@ def test_wide_decode_batches_of_a_large_layer_replay_as_eager(tmp_path, tuned):
     scale = torch.stack(list(got_e.values())).square().mean().sqrt().item()
     for key in got_e:
         assert not torch.isnan(got_g[key]).any()
-        # the same kernels in the same order; only the attention splits are planned for the padded batch
-        assert (got_g[key] - got_e[key]).abs().max().item() < 2e-2 * scale, f"graph replay differs from the eager step at {key}"
+        # The graph runs the padded batch (48 or 24 rows), the eager step the live rows (40 or 19):
+        # the library may take another kernel for another row count and add in another order, and
+        # at this many rows the logits come out of a bfloat16 product, so a logit may differ by a
+        # unit in the last place of bfloat16 (2^-8 of its value; two allowed). A replay that read
+        # a stale or cleared buffer is off by the logits' own scale.
+        diff = (got_g[key] - got_e[key]).abs()
+        bound = 2e-2 * scale + 2.0 ** -7 * got_e[key].abs()
+        assert bool((diff <= bound).all()), f"graph replay differs from the eager step at {key}: {diff.max().item()}"
 
 
 def test_negative_control_a_small_weight_change_breaks_the_match(model_dirs, tmp_path):
