@@ -180,7 +180,8 @@ __device__ __forceinline__ bool row_has_top_k(const SampleArgs& a, int row) {
 }
 __device__ __forceinline__ bool row_has_top_p(const SampleArgs& a, int row) { return a.top_p[row] < 1.0f; }
 __device__ __forceinline__ u64_t weight_of(float v, float mx) {
-  return (u64_t)(expf(v - mx) * SAMPLE_WEIGHT_SCALE);
+  const float e = expf(v - mx);  // NaN for inf - inf: no weight
+  return e == e ? (u64_t)(e * SAMPLE_WEIGHT_SCALE) : 0;
 }
 
 // The row's largest logit (NaN counts as -inf) and its first index, from the chunk maxima: the
@@ -282,6 +283,10 @@ __device__ __forceinline__ void topk_state(const SampleArgs& a, int row, int don
     r0 = st[1];
   }
   const uint32_t* hist = a.hist_k + ((int64_t)(done - 1) * a.n + row) * 256;
+  if (threadIdx.x == 0) {  // what stands if no bin qualifies (it always does for counts that add up)
+    picked[0] = 0u;
+    picked[1] = r0;
+  }
   uint32_t above;
   const uint32_t suf = suffix_of_bins<uint32_t>(hist, sh, above);
   // the bin that holds the rank-th largest: at least `rank` keys from it up, fewer above it
@@ -405,6 +410,10 @@ __device__ __forceinline__ void topp_state(const SampleArgs& a, int row, int don
     a0 = st[1];
   }
   const u64_t* hist = a.hist_p + ((int64_t)(done - 1) * a.n + row) * 256;
+  if (threadIdx.x == 0) {  // what stands if no bin qualifies (a row without any weight)
+    picked[0] = 0;
+    picked[1] = a0;
+  }
   u64_t above;
   const u64_t suf = suffix_of_bins<u64_t>(hist, sh, above);
   // the largest byte b with weight(keys >= (bytes so far, b, 0...)) > limit
@@ -523,6 +532,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_locate_kernel(SampleArg
   const u64_t* sums = (with_p ? psum2 : a.psum) + row * a.chunks;
   const uint32_t floor_key = with_p ? (uint32_t)psum2[(int64_t)a.n * a.chunks + row] : a.floor_k[row];
   const u64_t total = row_total(sums, a.chunks);
+  if (total == 0) {  // no token has any weight (every logit -inf or NaN): the first maximum, as greedy
+    if (threadIdx.x == 0) a.out[row] = mi < a.V ? mi : 0;
+    return;
+  }
   const uint32_t r = philox_first_word((uint64_t)a.seeds[row], (uint64_t)a.draws[row]);
   // u = (r >> 8) / 2^24; the drawn token is the first whose running weight exceeds u * total
   u64_t target = (u64_t)((double)(r >> 8) * (1.0 / 16777216.0) * (double)total);
@@ -530,6 +543,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_locate_kernel(SampleArg
   // the chunk the target falls into: a running sum over the chunks in the first wave
   __shared__ int sel_chunk;
   __shared__ u64_t sel_base;
+  if (threadIdx.x == 0) {
+    sel_chunk = 0;
+    sel_base = 0;
+  }
+  __syncthreads();
   if (threadIdx.x < 64) {
     const u64_t v = (int)threadIdx.x < a.chunks ? sums[threadIdx.x] : 0;
     u64_t incl = v;

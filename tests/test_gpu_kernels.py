@@ -866,6 +866,30 @@ def test_sampling_matches_plain_definition(V, scale):
     assert again == [got[i] for i in plain_rows]
 
 
+def test_sampling_of_rows_without_finite_logits_is_the_first_maximum():
+    """Rows of -inf, a +inf among finite logits, NaNs among them: no weight can be formed for some
+    of these rows; the kernels must neither fault nor leave the vocabulary."""
+    from clockwork_amd import ops
+
+    V = 5000
+    rows = torch.randn(6, V, device=DEV)
+    rows[0] = float("-inf")
+    rows[1] = float("-inf"); rows[1, 123] = 0.5          # one finite logit
+    rows[2, 777] = float("inf")                           # an infinite one wins
+    rows[3, ::2] = float("nan")                           # NaN counts as -inf
+    rows[4] = float("nan")
+    n = rows.shape[0]
+    for k, p in ((-1, 1.0), (20, 1.0), (-1, 0.7), (20, 0.7)):
+        got = ops.sample(rows, torch.full((n,), 0.9, device=DEV), torch.full((n,), k, dtype=torch.int32, device=DEV),
+                         torch.full((n,), p, device=DEV), torch.arange(n, dtype=torch.int64, device=DEV),
+                         torch.zeros(n, dtype=torch.int64, device=DEV)).tolist()
+        assert all(0 <= t < V for t in got)
+        assert got[0] == 0 and got[1] == 123 and got[2] == 777 and got[4] == 0
+        assert got[3] % 2 == 1
+        probs = plain.sampling_probs(rows[5].cpu(), 0.9, k, p)
+        assert probs[got[5]] > 0
+
+
 def test_sampling_keeps_exactly_the_top_k_and_the_nucleus():
     """Many draws from one row: every token of the kept set comes up and no other does (a selection
     that is off by one place shows here, not in single draws)."""
