@@ -86,7 +86,7 @@ def time_decode(cfg, runner, batch: int, steps: int, warmup: int, sampling=None)
     vocab = runner.spec.vocab_size
     temperature, top_k, top_p = sampling or (0.0, -1, 1.0)
     for i in range(batch):
-        params = SamplingParams(max_tokens=warmup + steps + batch + 2, temperature=temperature, top_k=top_k, top_p=top_p,
+        params = SamplingParams(max_tokens=warmup + steps + 2 * batch + 8,  # the first requests decode while the others' prompts run temperature=temperature, top_k=top_k, top_p=top_p,
                                 seed=i, ignore_eos=True)
         engine.add_request(f"b{batch}-{i}", prompt_token_ids=torch.randint(0, vocab, (PROMPT_LEN,), generator=gen).tolist(),
                            sampling_params=params)

@@ -26,7 +26,7 @@ from clockwork_amd.weights.loader import load_parameters, read_config_json
 
 
 # padded batch sizes a decode graph is captured for, and the step in which the planned context grows
-GRAPH_BATCH_SIZES = (1, 2, 4, 8, 16, 24, 32, 48, 64)
+GRAPH_BATCH_SIZES = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)
 GRAPH_KEY_BUCKET = 512
 
 
