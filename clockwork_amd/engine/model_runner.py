@@ -28,6 +28,9 @@ from clockwork_amd.weights.loader import load_parameters, read_config_json
 # padded batch sizes a decode graph is captured for, and the step in which the planned context grows
 GRAPH_BATCH_SIZES = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)
 GRAPH_KEY_BUCKET = 512
+# captured graphs kept at a time (each holds index buffers of its own): the least recently
+# replayed one goes when another shape is captured beyond this many
+GRAPH_LIMIT = 48
 
 
 def require_gpu() -> torch.device:
@@ -170,6 +173,8 @@ class ModelRunner:
             if self._graph_pool is None:
                 self._graph_pool = graph.pool()
             state = self._graphs[key] = (batch, graph, out)
+            self._drop_old_graphs()
+        self._graphs[key] = self._graphs.pop(key)  # most recently used last
         batch, graph, out = state
         batch.fill(entries, self.manager)
         graph.replay()
@@ -181,6 +186,14 @@ class ModelRunner:
         if len(rows) == n:
             return out[:n]
         return out[torch.tensor(rows, device=self.device)]
+
+    def _drop_old_graphs(self) -> None:
+        captured = [k for k, v in self._graphs.items() if isinstance(v, tuple)]
+        if len(captured) <= GRAPH_LIMIT:
+            return
+        torch.cuda.synchronize()  # none of them may still be running
+        for k in captured[: len(captured) - GRAPH_LIMIT]:
+            del self._graphs[k]
 
     def prepare_decode(self, positions: Sequence[tuple[str, int]]):
         """Get a decode-only step ready before its tokens are known: ``positions`` names each
@@ -211,6 +224,7 @@ class ModelRunner:
         key, entries = handle
         if len(tokens) != len(entries):
             raise ValueError(f"{len(tokens)} tokens for {len(entries)} prepared entries")
+        self._graphs[key] = self._graphs.pop(key)  # most recently used last
         batch, graph, out = self._graphs[key]
         if isinstance(tokens, torch.Tensor):
             if tokens.dtype != torch.int32 or tokens.device != self.device or tokens.dim() != 1:
