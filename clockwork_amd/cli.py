@@ -39,6 +39,7 @@ def _generate(argv) -> int:
     p.add_argument("--seed", type=int, default=None)
     p.add_argument("--ignore-eos", action="store_true")
     p.add_argument("--stop-token-ids", default="", metavar="I,J")
+    p.add_argument("--stop", action="append", default=[], metavar="TEXT", help="a stop string (needs --tokenizer)")
     args = p.parse_args(argv)
 
     if (args.config is None) == (args.model is None):
@@ -69,7 +70,7 @@ def _generate(argv) -> int:
     params = SamplingParams(
         max_tokens=args.max_tokens, temperature=args.temperature, top_p=args.top_p, top_k=args.top_k,
         seed=args.seed, ignore_eos=args.ignore_eos,
-        stop_token_ids=[int(t) for t in args.stop_token_ids.split(",") if t.strip()],
+        stop_token_ids=[int(t) for t in args.stop_token_ids.split(",") if t.strip()], stop=list(args.stop),
     )
     for out in engine.generate(prompts, params):
         print(json.dumps({
