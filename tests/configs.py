@@ -37,6 +37,13 @@ WIDE = dict(
 # One layer each of the larger models the engine is meant for (Qwen2.5-7B and -32B layer sizes, a
 # small vocabulary): products whose K does not fit the streaming kernel's registers, groups of 7
 # and 5 query heads per key head, 18944 / 27648-wide feed-forwards.
+# One layer of exactly the benchmark's model (Qwen2.5-1.5B): its widths, its full vocabulary, its
+# tied output head.
+LAYER_1P5B = dict(
+    model_type="qwen2", vocab_size=151936, hidden_size=1536, num_hidden_layers=1, num_attention_heads=12,
+    num_key_value_heads=2, intermediate_size=8960, rms_norm_eps=1e-6, rope_theta=1000000.0,
+    tie_word_embeddings=True,
+)
 LAYER_7B = dict(
     model_type="qwen2", vocab_size=1501, hidden_size=3584, num_hidden_layers=1, num_attention_heads=28,
     num_key_value_heads=4, intermediate_size=18944, rms_norm_eps=1e-6, rope_theta=1000000.0,

@@ -113,6 +113,36 @@ def test_wide_layers_take_the_streaming_and_fused_paths(tmp_path, mode):
     assert not runner.manager.live_requests()
 
 
+def test_a_layer_of_the_benchmark_model_in_both_precisions(tmp_path):
+    """One layer with exactly the sizes of the benchmark's model, the full vocabulary of 151,936
+    and the tied head, mixed batches: float32 at the 1e-5 bar (25 million logits), bfloat16 within
+    the rounding of its 8-bit mantissas."""
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests.configs import LAYER_1P5B
+
+    model_dir = write_random_model(tmp_path / "layer1p5b", LAYER_1P5B, 2)
+    gen = torch.Generator().manual_seed(11)
+    requests = {f"w{i}": torch.randint(0, LAYER_1P5B["vocab_size"], (n,), generator=gen).tolist()
+                for i, n in enumerate([40, 70, 55])}
+    # Sums of 1,536 and 8,960 float32 products carry rounding of about 1e-5 themselves, in the
+    # engine and in a float32 plain implementation alike (they differ by up to 1.3e-5 here), so
+    # the plain side runs in float64: what is measured is the engine's own rounding.
+    plain = PlainQwen2(model_dir, dtype=torch.float64)
+    want = {rid: plain.logits(toks).float() for rid, toks in requests.items()}
+    scale = torch.cat([w.flatten() for w in want.values()]).square().mean().sqrt().item()
+    pages = replay.pages_needed(requests, 3, 16)
+    got = replay.run_trace(replay.make_runner(model_dir, "float32", 16, pages), replay.mixed(requests))
+    worst = replay.compare(got, want, **TOL["float32"])
+    print(f"benchmark layer float32 mixed: largest error {worst:.3e}")
+    got = replay.run_trace(replay.make_runner(model_dir, "bfloat16", 16, pages), replay.mixed(requests))
+    errors = torch.stack([row - want[rid][pos] for (rid, pos), row in sorted(got.items())])
+    assert not torch.isnan(errors).any()
+    rms, worst = errors.square().mean().sqrt().item(), errors.abs().max().item()
+    print(f"benchmark layer bfloat16 mixed: logits' scale {scale:.3f}, rms error {rms:.3e}, largest {worst:.3e}")
+    # as for the layers of the larger models below: relative to the logits' own scale
+    assert rms < 2e-2 * scale and worst < 1e-1 * scale
+
+
 @pytest.mark.parametrize("which", ["LAYER_7B", "LAYER_32B"])
 def test_layers_of_the_larger_models(tmp_path, which):
     """One layer of the 7B and of the 32B shape, bfloat16: a prompt in two portions, then tokens
