@@ -25,6 +25,24 @@ TINY_C = dict(
 # name -> (config, weight seed, cache block size)
 TINY_CONFIGS = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8), "C": (TINY_C, 5, 16)}
 
+# Sizes that none of the above pins: groups of 5, 7, 14 and 17 query heads (17: more than one
+# workgroup of the decode kernel takes), widths that are multiples of 2 only, a feed-forward of 7,
+# pages of 4, 24 and 48 tokens, head sizes 32 to 256. name -> (config, weight seed, block size)
+ODD_CONFIGS = {
+    "group14": (dict(model_type="qwen2", vocab_size=1001, hidden_size=66, head_dim=96, num_hidden_layers=2,
+                     num_attention_heads=42, num_key_value_heads=3, intermediate_size=255, rms_norm_eps=1e-5,
+                     rope_theta=50000.0, tie_word_embeddings=False), 11, 16),
+    "pages_of_4": (dict(model_type="qwen2", vocab_size=127, hidden_size=130, head_dim=256, num_hidden_layers=3,
+                        num_attention_heads=15, num_key_value_heads=3, intermediate_size=33, rms_norm_eps=3e-4,
+                        rope_theta=10000.0, tie_word_embeddings=False), 12, 4),
+    "narrow": (dict(model_type="qwen2", vocab_size=51, hidden_size=66, head_dim=32, num_hidden_layers=2,
+                    num_attention_heads=14, num_key_value_heads=2, intermediate_size=7, rms_norm_eps=1e-6,
+                    rope_theta=1000000.0, tie_word_embeddings=True), 13, 24),
+    "group17": (dict(model_type="qwen2", vocab_size=2049, hidden_size=1032, head_dim=160, num_hidden_layers=1,
+                     num_attention_heads=34, num_key_value_heads=2, intermediate_size=1000, rms_norm_eps=1e-6,
+                     rope_theta=1000000.0, tie_word_embeddings=True), 14, 48),
+}
+
 # Layers wide enough for the decode kernels that only take large shapes (the persistent
 # weight-streaming product, the norm fused into the gate/up product): hidden >= 1024 and at least
 # 512 row tiles of 8 in the feed-forward. Two layers and a small vocabulary keep it quick.

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from tests import replay
-from tests.configs import TINY_CONFIGS
+from tests.configs import ODD_CONFIGS, TINY_CONFIGS
 from tests.plain.qwen2_plain import PlainQwen2
 
 pytestmark = pytest.mark.gpu
@@ -58,6 +58,34 @@ def test_replay_matches_plain(model_dirs, name, dtype, mode):
     print(f"{name} {dtype} {mode}: largest error {worst:.3e}")
     assert not runner.manager.live_requests()
     assert runner.manager.min_free_blocks() == runner.manager.num_blocks
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(ODD_CONFIGS))
+def test_odd_sizes_replay_like_the_plain_implementation(tmp_path, name, dtype):
+    """Head counts, groups, widths and page sizes that the three tiny models do not have."""
+    from clockwork_amd.weights.random_init import write_random_model
+
+    cfg, seed, block_size = ODD_CONFIGS[name]
+    model_dir = write_random_model(tmp_path / name, cfg, seed)
+    gen = torch.Generator().manual_seed(seed)
+    requests = {f"r{i}": torch.randint(0, cfg["vocab_size"], (n,), generator=gen).tolist()
+                for i, n in enumerate([65, 3, 130, 1, 200, 33])}
+    plain = PlainQwen2(model_dir)
+    ref = {rid: plain.logits(toks) for rid, toks in requests.items()}
+    tol = dict(TOL[dtype])
+    if dtype == "bfloat16":
+        # 8 bits: the error follows the logits' size where that is above 1 (the 1032-wide model)
+        tol["atol"] *= max(1.0, max(float(v.abs().max()) for v in ref.values()))
+    for mode in ("prefill_then_decode", "mixed"):
+        live = 4 if mode == "mixed" else 1
+        runner = replay.make_runner(model_dir, dtype, block_size, replay.pages_needed(requests, live, block_size))
+        got = replay.run_trace(runner, getattr(replay, mode)(requests))
+        assert len(got) == sum(len(t) for t in requests.values())
+        worst = replay.compare(got, ref, **tol)
+        print(f"{name} {dtype} {mode}: largest error {worst:.3e}")
+        assert not runner.manager.live_requests()
+        assert runner.manager.min_free_blocks() == runner.manager.num_blocks
 
 
 def test_wide_layers_in_float32(tmp_path):
