@@ -634,12 +634,16 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnParams p) {
   }
 }
 
-// Merge of the decode kernel's splits: one workgroup per (item, head), one thread per element.
-// The statistics of all splits go through LDS first, and partial outputs are fetched four at
-// a time, so the kernel is a few memory round trips long whatever the number of splits.
+// Merge of the decode kernel's splits: one workgroup per (item, head) of blockDim.x = G * HD
+// threads. Thread (g, d) sums element d over splits g, g + G, ...; the G sums meet in LDS. The
+// statistics of all splits go through LDS first, and partial outputs are fetched eight at a
+// time, so the kernel is a few memory round trips long whatever the number of splits.
+#define DEC_MAX_SPLITS 256
+
 template <int HD>
-__global__ void attn_decode_merge_kernel(AttnParams p) {
-  __shared__ float ms[64], ls[64];
+__global__ __launch_bounds__(1024) void attn_decode_merge_kernel(AttnParams p) {
+  __shared__ float ms[DEC_MAX_SPLITS], ls[DEC_MAX_SPLITS];
+  __shared__ float o_s[1024], l_s[1024 / HD];
   const int gh = p.gh;
   const int item = blockIdx.x;
   const int y = blockIdx.y / gh, g = blockIdx.y % gh;
@@ -659,25 +663,37 @@ __global__ void attn_decode_merge_kernel(AttnParams p) {
   __syncthreads();
   float M = -INFINITY;
   for (int sp = 0; sp < p.n_splits; ++sp) M = fmaxf(M, ms[sp]);
-  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
-    float L = 0.0f, O = 0.0f;
-    for (int sp0 = 0; sp0 < p.n_splits; sp0 += 4) {
-      float ov[4];
+  const int G = blockDim.x / HD;
+  const int tg = threadIdx.x / HD, d = threadIdx.x - tg * HD;
+  float L = 0.0f, O = 0.0f;
+  for (int sp0 = tg; sp0 < p.n_splits; sp0 += 8 * G) {
+    float ov[8];
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
-        ov[u] = sp0 + u < p.n_splits ? p.part_o[((base + sp0 + u) * gh + g) * HD + d] : 0.0f;
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        if (sp0 + u >= p.n_splits) continue;
-        const float mv = ms[sp0 + u];
-        const float wgt = mv == -INFINITY ? 0.0f : __expf(mv - M);
-        L = fmaf(ls[sp0 + u], wgt, L);
-        O = fmaf(ov[u], wgt, O);
-      }
+    for (int u = 0; u < 8; ++u) {
+      const int sp = sp0 + u * G;
+      ov[u] = sp < p.n_splits ? p.part_o[((base + sp) * gh + g) * HD + d] : 0.0f;
     }
-    ((bf16_t*)p.out)[(int64_t)(q_begin + tok0) * p.out_stride + (kvh * group + hg) * HD + d] =
-        __float2bfloat16(O / L);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int sp = sp0 + u * G;
+      if (sp >= p.n_splits) continue;
+      const float mv = ms[sp];
+      const float wgt = mv == -INFINITY ? 0.0f : __expf(mv - M);
+      L = fmaf(ls[sp], wgt, L);
+      O = fmaf(ov[u], wgt, O);
+    }
   }
+  if (G > 1) {
+    o_s[threadIdx.x] = O;
+    if (d == 0) l_s[tg] = L;
+    __syncthreads();
+    if (tg > 0) return;
+    for (int w = 1; w < G; ++w) {
+      O += o_s[w * HD + d];
+      L += l_s[w];
+    }
+  }
+  ((bf16_t*)p.out)[(int64_t)(q_begin + tok0) * p.out_stride + (kvh * group + hg) * HD + d] = __float2bfloat16(O / L);
 }
 
 #if CW_HD % 32 == 0
@@ -688,6 +704,9 @@ __global__ void attn_decode_merge_kernel(AttnParams p) {
 
 // 1 when this head size has the bfloat16 decode kernel (multiples of 32).
 CW_EXPORT int cw_attention_decode_supported() { return CW_HAS_DECODE; }
+
+// The most splits cw_attention_decode_bf16 takes.
+CW_EXPORT int cw_attention_decode_max_splits() { return DEC_MAX_SPLITS; }
 
 // Heads of a group one workgroup of the decode kernel takes, for a group of this size.
 CW_EXPORT int cw_attention_decode_gh(int group) { return group < 16 ? group : 16; }
@@ -721,7 +740,11 @@ static int launch_decode(AttnParams& p, int n_items, hipStream_t stream) {
   hipLaunchKernelGGL((attn_decode_bf16_kernel<HD, POW2>), grid, block, smem, stream, p);
   if (p.n_splits > 1) {
     dim3 mgrid(n_items, p.nkv * p.n_chunks * p.gh);
-    hipLaunchKernelGGL((attn_decode_merge_kernel<HD>), mgrid, dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0, stream, p);
+    // thread groups that share the splits: about eight splits for each, as many as 1024 threads hold
+    int groups = p.n_splits / 8;
+    if (groups > 1024 / HD) groups = 1024 / HD;
+    if (groups < 1) groups = 1;
+    hipLaunchKernelGGL((attn_decode_merge_kernel<HD>), mgrid, dim3(groups * HD), 0, stream, p);
   }
   return cw_launch_status();
 }
@@ -743,7 +766,7 @@ CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* ou
 #if CW_HAS_DECODE
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || block_size <= 0 || table_stride <= 0)
     return CW_ERR_ARG;
-  if (n_splits < 1 || n_splits > 64 || window < 0) return CW_ERR_ARG;
+  if (n_splits < 1 || n_splits > DEC_MAX_SPLITS || window < 0) return CW_ERR_ARG;
   if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || (q_stride & 7))
     return CW_ERR_ARG;
   if (zeros == nullptr || ((uintptr_t)zeros & 15)) return CW_ERR_ARG;

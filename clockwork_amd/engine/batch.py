@@ -151,7 +151,8 @@ class StepContext:
             plan.single_splits = max(1, min(by_occupancy, by_length, 64))
             # decode kernel: a workgroup per (request, kv head, split); a split is at least 128 keys
             # (one 32-key tile for each of its four waves), and about two workgroups per compute
-            # unit are enough to keep memory busy
+            # unit are enough to keep memory busy. More than 64 splits never paid: one request
+            # with 30000 keys takes 16 us with 64 to 128 splits and 19 us with 235.
             base = plan.n_single * nkv * -(-group // min(group, 16))
             plan.decode_splits = max(1, min(-(-2 * self.num_compute_units // base), longest_single // 128, 64))
             # fixed places for the splits: a workgroup then knows its pages before it knows the

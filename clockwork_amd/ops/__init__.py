@@ -119,6 +119,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_attention_prefill_row_blocks_ok": [I],
             "cw_attention_decode_supported": [],
             "cw_attention_decode_gh": [I],
+            "cw_attention_decode_max_splits": [],
             "cw_attention_decode_workspace_floats": [I, I, I, I],
             "cw_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, P, I, I, I, P],
         },
@@ -567,6 +568,10 @@ def prefill_tokens_per_item(group: int, row_blocks: int = 4) -> int:
 
 def decode_attention_supported(hd: int, dtype: torch.dtype) -> bool:
     return dtype == torch.bfloat16 and bool(_load("attention", hd).cw_attention_decode_supported())
+
+
+# the most splits the bfloat16 decode kernel takes (DEC_MAX_SPLITS in csrc/attention.hip)
+DECODE_MAX_SPLITS = 256
 
 
 def decode_attention_workspace_floats(hd: int, n_items: int, nh: int, nkv: int, n_splits: int) -> int:

@@ -636,10 +636,13 @@ DECODE_KERNEL_CASES = [
 
 
 @pytest.mark.parametrize("nh,nkv,hd,bs,ctx_lens", DECODE_KERNEL_CASES)
-@pytest.mark.parametrize("splits", [1, 2, 7])
+@pytest.mark.parametrize("splits", [1, 2, 7, 40, 256])
 @pytest.mark.parametrize("fixed_ranges", [False, True])
 def test_decode_attention_kernel(nh, nkv, hd, bs, ctx_lens, splits, fixed_ranges):
     dtype = torch.bfloat16
+    from clockwork_amd import ops
+
+    assert ops._load("attention", hd).cw_attention_decode_max_splits() == ops.DECODE_MAX_SPLITS == 256
     num_blocks = sum(-(-c // bs) for c in ctx_lens) + 5
     perm = torch.randperm(num_blocks).tolist()
     tables, at = [], 0
