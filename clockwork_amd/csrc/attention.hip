@@ -655,6 +655,16 @@ __global__ __launch_bounds__(1024) void attn_decode_merge_kernel(AttnParams p) {
   const int tok0 = ident ? 0 : p.items[4 * item + 1];
   const int q_begin = ident ? item : p.cu_q[p.items[4 * item]];
   const int64_t base = ((int64_t)item * (p.nkv * p.n_chunks) + y) * p.n_splits;
+  const int G = blockDim.x / HD;
+  const int tg = threadIdx.x / HD, d = threadIdx.x - tg * HD;
+  // the thread's first eight partial outputs are requested together with the statistics: they do
+  // not depend on them, and a trip to memory that waits for another is most of this kernel's time
+  float ov[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int sp = tg + u * G;
+    ov[u] = sp < p.n_splits ? p.part_o[((base + sp) * gh + g) * HD + d] : 0.0f;
+  }
   for (int sp = threadIdx.x; sp < p.n_splits; sp += blockDim.x) {
     const float2 ml = *reinterpret_cast<const float2*>(&p.part_ml[((base + sp) * gh + g) * 2]);
     ms[sp] = ml.x;
@@ -663,15 +673,14 @@ __global__ __launch_bounds__(1024) void attn_decode_merge_kernel(AttnParams p) {
   __syncthreads();
   float M = -INFINITY;
   for (int sp = 0; sp < p.n_splits; ++sp) M = fmaxf(M, ms[sp]);
-  const int G = blockDim.x / HD;
-  const int tg = threadIdx.x / HD, d = threadIdx.x - tg * HD;
   float L = 0.0f, O = 0.0f;
   for (int sp0 = tg; sp0 < p.n_splits; sp0 += 8 * G) {
-    float ov[8];
+    if (sp0 != tg) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int sp = sp0 + u * G;
-      ov[u] = sp < p.n_splits ? p.part_o[((base + sp) * gh + g) * HD + d] : 0.0f;
+      for (int u = 0; u < 8; ++u) {
+        const int sp = sp0 + u * G;
+        ov[u] = sp < p.n_splits ? p.part_o[((base + sp) * gh + g) * HD + d] : 0.0f;
+      }
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {

@@ -150,19 +150,28 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     }
   }
   if (dl) {
+    // the partial sums are added in order, but fetched PU at a time: every trip to memory that
+    // waits for the one before costs about a microsecond, more than the rest of this kernel
+    constexpr int PU = KC <= 4 ? 4 : 2;
     float acc[KC][4];
-    for (int q = 0; q < parts; ++q) {
-      float d[KC][4];
+    for (int q0 = 0; q0 < parts; q0 += PU) {
+      float d[PU][KC][4];
 #pragma unroll
-      for (int k = 0; k < KC; ++k) {
-        const int ch = threadIdx.x + k * 256;
-        if (ch < n_chunks) Chunk4<DT>::load(dl + q * part_stride + ch * 4, d[k]);
-        else d[k][0] = d[k][1] = d[k][2] = d[k][3] = 0.0f;
+      for (int u = 0; u < PU; ++u)
+#pragma unroll
+        for (int k = 0; k < KC; ++k) {
+          const int ch = threadIdx.x + k * 256;
+          if (q0 + u < parts && ch < n_chunks) Chunk4<DT>::load(dl + (q0 + u) * part_stride + ch * 4, d[u][k]);
+          else d[u][k][0] = d[u][k][1] = d[u][k][2] = d[u][k][3] = 0.0f;
+        }
+#pragma unroll
+      for (int u = 0; u < PU; ++u) {
+        if (q0 + u >= parts) break;
+#pragma unroll
+        for (int k = 0; k < KC; ++k)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[k][e] = q0 + u == 0 ? d[u][k][e] : acc[k][e] + d[u][k][e];
       }
-#pragma unroll
-      for (int k = 0; k < KC; ++k)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[k][e] = q == 0 ? d[k][e] : acc[k][e] + d[k][e];
     }
 #pragma unroll
     for (int k = 0; k < KC; ++k)

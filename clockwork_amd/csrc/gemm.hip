@@ -685,6 +685,36 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_qkv_rope_bf16_kernel(
     xrow[mt] = X + (int64_t)(xok[mt] ? mt * 16 + r : 0) * ldx;
   }
 
+  auto bias_at = [&](int col) -> float {
+    if (bias == nullptr) return 0.0f;
+    return bias_f32 ? ((const float*)bias)[col] : __bfloat162float(((const bf16_t*)bias)[col]);
+  };
+  // MT == 1: what this thread's part of the epilogue needs (position, slot, frequency, bias) is
+  // requested here, beside the weights, and not after the product, where it would be one more
+  // trip to memory with nothing else to do meanwhile
+  int e_pos = 0;
+  int64_t e_slot = -1;
+  float e_inv = 0.0f, e_ba = 0.0f, e_bb = 0.0f;
+  if constexpr (MT == 1) {
+    if (is_v) {
+      const int j = threadIdx.x & 15, m = threadIdx.x >> 4;
+      if (m < 16 && m < M) {
+        e_slot = slots[m];
+        e_ba = bias_at(head * hd + tile * 16 + j);
+      }
+    } else {
+      const int p = threadIdx.x & 7, m = threadIdx.x >> 3;
+      if (m < 16 && m < M) {
+        const int i = tile * 8 + p;
+        e_pos = positions[m];
+        e_slot = slots[m];
+        e_inv = inv_freq[i];
+        e_ba = bias_at(head * hd + i);
+        e_bb = bias_at(head * hd + half + i);
+      }
+    }
+  }
+
   f32x4_t acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
@@ -721,11 +751,37 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_qkv_rope_bf16_kernel(
     red[0][idx] = sum;
   }
   __syncthreads();
-  auto bias_at = [&](int col) -> float {
-    if (bias == nullptr) return 0.0f;
-    return bias_f32 ? ((const float*)bias)[col] : __bfloat162float(((const bf16_t*)bias)[col]);
-  };
   auto summed = [&](int row, int m) -> float { return red[0][m * 16 + row]; };
+  if constexpr (MT == 1) {
+    // every thread has at most one output (v: 256 of them, q and k: 128 pairs)
+    if (is_v) {
+      const int j = threadIdx.x & 15, m = threadIdx.x >> 4;
+      if (m < 16 && m < M && e_slot >= 0 && e_slot < cache_rows) {
+        const int d = tile * 16 + j;
+        v_cache[(e_slot * nkv + (head - nh - nkv)) * hd + d] = __float2bfloat16(summed(j, m) + e_ba);
+      }
+    } else {
+      const int p = threadIdx.x & 7, m = threadIdx.x >> 3;
+      if (m < 16 && m < M) {
+        const int i = tile * 8 + p;
+        const float a = summed(p, m) + e_ba;
+        const float b = summed(p + 8, m) + e_bb;
+        float sn, cs;
+        sincosf((float)e_pos * e_inv, &sn, &cs);
+        const bf16_t oa = __float2bfloat16(a * cs - b * sn), ob = __float2bfloat16(b * cs + a * sn);
+        if (head < nh) {
+          bf16_t* q = q_out + (int64_t)m * nh * hd + head * hd;
+          q[i] = oa;
+          q[i + half] = ob;
+        } else if (e_slot >= 0 && e_slot < cache_rows) {
+          bf16_t* kd = k_cache + (e_slot * nkv + (head - nh)) * hd;
+          kd[i] = oa;
+          kd[i + half] = ob;
+        }
+      }
+    }
+    return;
+  }
   if (is_v) {
     // idx -> (token m, row j), j fastest: 16 consecutive elements of a cache row
     for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {
