@@ -40,6 +40,8 @@ def main(argv=None) -> int:
         dtype=args.dtype,
         block_size=PAGE,
         num_blocks=max(1, -(-args.max_tokens // PAGE)),
+        # one request may hold every token of the pool
+        max_model_len=max(PAGE, PAGE * -(-args.max_tokens // PAGE)),
         enable_prefix_cache=False,
         watermark=0.0,
     )
