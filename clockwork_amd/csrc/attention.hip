@@ -946,8 +946,11 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
   const int t_first = wg_lo / KT, t_last = wg_last / KT;
   const int f_key = threadIdx.x / TPK, f_ch = threadIdx.x % TPK;
   const int64_t row_elems = (int64_t)p.nkv * HD;
-  u32x4_t gk[NCK], gv[NCK];
-  auto fetch = [&](int t) __attribute__((always_inline)) {  // global -> registers; a masked key reads a row of zeros
+  // Two row blocks: the workgroups are short of work per stage, so a stage's loads get two stages
+  // to arrive (a second register set); with four row blocks the registers are full and one is enough
+  constexpr bool DEEP = RB == 2;
+  u32x4_t gk[NCK], gv[NCK], gk1[DEEP ? NCK : 1], gv1[DEEP ? NCK : 1];
+  auto fetch = [&](int t, u32x4_t* gk, u32x4_t* gv) __attribute__((always_inline)) {  // global -> registers; a masked key reads a row of zeros
     const int kp = t * KT + f_key;
     bool ok = kp >= wg_lo && kp <= wg_last;
     const int page = tbl[ok ? cw_page_index<POW2>(kp, bs, sh) - page0 : 0];
@@ -963,7 +966,7 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
       gv[i] = *reinterpret_cast<const u32x4_t*>(vr + (in_row ? i * step : 0));
     }
   };
-  auto stash = [&](int stage) __attribute__((always_inline)) {  // registers -> LDS
+  auto stash = [&](int stage, const u32x4_t* gk, const u32x4_t* gv) __attribute__((always_inline)) {  // registers -> LDS
     bf16_t* ks = tiles + stage * Tile::STAGE + f_key * 32;
     bf16_t* vs = tiles + stage * Tile::STAGE + KT * HD + f_key * VROW + f_ch * 8;
 #pragma unroll
@@ -975,23 +978,18 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
       }
     }
   };
-  fetch(t_first);
-  stash(0);
-  __syncthreads();
-
-  for (int t = t_first; t <= t_last; ++t) {
-    const int kv0 = t * KT + half * KW;  // the wave's keys of this stage
-    const int stage = (t - t_first) & 1;
-    if (t < t_last) {
-      // the next stage's pages must lie in the table window; nobody reads the window right now
-      const int need = cw_page_index<POW2>(min((t + 1) * KT + KT - 1, wg_last), bs, sh);
-      if (need >= page0 + Tile::TABLE) {
-        page0 = cw_page_index<POW2>(max((t + 1) * KT, wg_lo), bs, sh);
-        load_table();
-        __syncthreads();
-      }
-      fetch(t + 1);  // in flight while this tile is computed
+  // the pages of stage tn must lie in the table window before it is fetched; every wave comes
+  // here between the same two barriers and nobody reads the window meanwhile
+  auto window_for = [&](int tn) __attribute__((always_inline)) {
+    const int need = cw_page_index<POW2>(min(tn * KT + KT - 1, wg_last), bs, sh);
+    if (need >= page0 + Tile::TABLE) {
+      page0 = cw_page_index<POW2>(max(tn * KT, wg_lo), bs, sh);
+      load_table();
+      __syncthreads();
     }
+  };
+  auto compute = [&](int t, int stage) __attribute__((always_inline)) {
+    const int kv0 = t * KT + half * KW;  // the wave's keys of this stage
     const bool active = wave_on && kv0 <= p_last && kv0 + KW - 1 >= lo;
     if (active) {
       const bf16_t* ks = tiles + stage * Tile::STAGE + half * KW * 32;
@@ -1086,8 +1084,45 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
           for (int b = 0; b < 2; ++b) o[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pf[b][k2], o[b][db], 0, 0, 0);
         }
     }
-    if (t < t_last) stash(stage ^ 1);  // tile t + 1, read in the next round; nobody reads that buffer now
+  };
+
+  fetch(t_first, gk, gv);
+  stash(0, gk, gv);
+  if constexpr (DEEP) {
+    // set 0 holds stage t + 1 while an even round computes stage t, set 1 stage t + 2; each set is
+    // stashed at the end of the round before its stage is computed and filled again at once
+    if (t_first + 1 <= t_last) fetch(t_first + 1, gk, gv);
+    if (t_first + 2 <= t_last) fetch(t_first + 2, gk1, gv1);
     __syncthreads();
+    for (int t = t_first; t <= t_last; t += 2) {
+      compute(t, 0);
+      if (t + 1 <= t_last) stash(1, gk, gv);
+      if (t + 3 <= t_last) {
+        window_for(t + 3);
+        fetch(t + 3, gk, gv);
+      }
+      __syncthreads();
+      if (t + 1 > t_last) break;
+      compute(t + 1, 1);
+      if (t + 2 <= t_last) stash(0, gk1, gv1);
+      if (t + 4 <= t_last) {
+        window_for(t + 4);
+        fetch(t + 4, gk1, gv1);
+      }
+      __syncthreads();
+    }
+  } else {
+    __syncthreads();
+    for (int t = t_first; t <= t_last; ++t) {
+      const int stage = (t - t_first) & 1;
+      if (t < t_last) {
+        window_for(t + 1);
+        fetch(t + 1, gk, gv);  // in flight while this tile is computed
+      }
+      compute(t, stage);
+      if (t < t_last) stash(stage ^ 1, gk, gv);  // tile t + 1, read in the next round; nobody reads that buffer now
+      __syncthreads();
+    }
   }
 
   // ---- the other sets of waves hand their rows' state to the first set through LDS (the tiles
