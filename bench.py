@@ -34,7 +34,7 @@ QWEN25_7B = dict(QWEN25_1P5B, vocab_size=152064, hidden_size=3584, num_attention
 QWEN25_32B = dict(QWEN25_1P5B, vocab_size=152064, hidden_size=5120, num_hidden_layers=64, num_attention_heads=40,
                   num_key_value_heads=8, intermediate_size=27648, tie_word_embeddings=False)
 SHAPES = {"1.5b": ("Qwen2.5-1.5B", QWEN25_1P5B), "7b": ("Qwen2.5-7B", QWEN25_7B), "32b": ("Qwen2.5-32B", QWEN25_32B)}
-PROMPT_LEN = 2048
+PROMPT_LEN = 2048   # the prefill measurement, and the decode requests' prompts unless --prompt-len says otherwise
 CONTEXT = 4096
 BLOCK = 16
 
@@ -43,6 +43,11 @@ def _sync():
     import torch
 
     torch.cuda.synchronize()
+
+
+def context_of(args) -> int:
+    """The context limit of the run: twice the decode requests' prompts, 4096 for the recorded 2048."""
+    return max(CONTEXT, 2 * getattr(args, "prompt_len", PROMPT_LEN))
 
 
 def build_runner(args, prefix_cache: bool = False, max_batch: int = 0):
@@ -61,9 +66,10 @@ def build_runner(args, prefix_cache: bool = False, max_batch: int = 0):
     spec = arch.build_spec(mcfg)
     source = RandomSource(arch.weight_plan(mcfg, spec), model_param_specs(spec), seed=2, device="cuda")
     max_batch = max(args.batch, 64, max_batch)
+    context = context_of(args)
     cfg = EngineConfig.defaults(
-        "random:qwen2.5-1.5b", dtype=args.dtype, max_model_len=CONTEXT, block_size=BLOCK,
-        num_blocks=max_batch * CONTEXT // BLOCK, enable_prefix_cache=prefix_cache, watermark=0.0,
+        "random:qwen2.5-1.5b", dtype=args.dtype, max_model_len=context, block_size=BLOCK,
+        num_blocks=max_batch * context // BLOCK, enable_prefix_cache=prefix_cache, watermark=0.0,
         max_num_seqs=max_batch, max_num_batched_tokens=max(PROMPT_LEN, max_batch),
     )
     runner = ModelRunner(cfg, weight_source=source, config_dict=config)
@@ -73,8 +79,8 @@ def build_runner(args, prefix_cache: bool = False, max_batch: int = 0):
     return cfg, runner
 
 
-def time_decode(cfg, runner, batch: int, steps: int, warmup: int, sampling=None):
-    """Prefill ``batch`` prompts of PROMPT_LEN tokens, then time ``steps`` decode steps.
+def time_decode(cfg, runner, batch: int, steps: int, warmup: int, sampling=None, prompt_len: int = PROMPT_LEN):
+    """Prefill ``batch`` prompts of ``prompt_len`` tokens, then time ``steps`` decode steps.
     ``sampling``: (temperature, top_k, top_p) instead of greedy."""
     import torch
 
@@ -86,9 +92,11 @@ def time_decode(cfg, runner, batch: int, steps: int, warmup: int, sampling=None)
     vocab = runner.spec.vocab_size
     temperature, top_k, top_p = sampling or (0.0, -1, 1.0)
     for i in range(batch):
-        params = SamplingParams(max_tokens=warmup + steps + 2 * batch + 8,  # the first requests decode while the others' prompts run temperature=temperature, top_k=top_k, top_p=top_p,
-                                seed=i, ignore_eos=True)
-        engine.add_request(f"b{batch}-{i}", prompt_token_ids=torch.randint(0, vocab, (PROMPT_LEN,), generator=gen).tolist(),
+        # the first requests decode while the others' prompts run, portion by portion: a margin of tokens for those steps
+        portions = -(-prompt_len // cfg.scheduler.max_num_batched_tokens)
+        params = SamplingParams(max_tokens=warmup + steps + 2 * batch * portions + 8, temperature=temperature, top_k=top_k,
+                                top_p=top_p, seed=i, ignore_eos=True)
+        engine.add_request(f"b{batch}-{i}", prompt_token_ids=torch.randint(0, vocab, (prompt_len,), generator=gen).tolist(),
                            sampling_params=params)
     while any(s.is_prefilling() or s.num_computed_tokens == 0 for s in engine.scheduler.running + engine.scheduler.waiting):
         engine.step()
@@ -270,6 +278,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
+                    help="tokens each decode request holds before it decodes (the recorded benchmark: 2048)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (both numbers are recorded)")
     ap.add_argument("--shape", default="1.5b", choices=sorted(SHAPES), help="layer sizes: the 1.5B shape is the recorded benchmark")
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
@@ -302,14 +312,14 @@ def main() -> int:
         print(json.dumps({"prefill_ms": round(1e3 * t, 3), "tokens_per_s": round(PROMPT_LEN / t, 1)}))
         return 0
     sampling = (args.temperature, args.top_k, args.top_p) if args.temperature > 0 else None
-    elapsed, mean_ctx = time_decode(cfg, runner, args.batch, args.steps, args.warmup, sampling)
+    elapsed, mean_ctx = time_decode(cfg, runner, args.batch, args.steps, args.warmup, sampling, args.prompt_len)
     value = args.batch * args.steps / elapsed
     ms = 1e3 * elapsed / args.steps
     step_bytes = runner.model.weight_bytes_per_step() + args.batch * mean_ctx * runner.pools.kv_bytes_per_token()
     achieved = step_bytes / (elapsed / args.steps) / 1e9
 
     record = {
-        "metric": f"decode tok/s, {SHAPES[args.shape][0]} shape, batch {args.batch}, 2048-token prompts",
+        "metric": f"decode tok/s, {SHAPES[args.shape][0]} shape, batch {args.batch}, {args.prompt_len}-token prompts",
         "value": round(value, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -333,8 +343,8 @@ def main() -> int:
             "vocab": runner.spec.info["vocab"],
             "tied_embeddings": runner.spec.info["tied"],
             "global_batch": args.batch,
-            "prompt_len": PROMPT_LEN,
-            "seq_len": CONTEXT,
+            "prompt_len": args.prompt_len,
+            "seq_len": context_of(args),
             "block_size": BLOCK,
             "sampling": "greedy" if sampling is None else f"temperature {args.temperature} top_k {args.top_k} top_p {args.top_p}",
             "parallelism": "single GPU",
@@ -358,7 +368,7 @@ def main() -> int:
         }
         points = {}
         for b in (1, 64):
-            e, _ = time_decode(cfg, runner, b, args.steps, args.warmup, sampling)
+            e, _ = time_decode(cfg, runner, b, args.steps, args.warmup, sampling, args.prompt_len)
             points[f"decode_b{b}"] = round(b * args.steps / e, 1)
         record["points"] = points
     print(json.dumps(record))
