@@ -118,19 +118,23 @@ def time_decode(cfg, runner, batch: int, steps: int, warmup: int, sampling=None,
     return elapsed, mean_ctx
 
 
-def time_prefill(cfg, runner, repeats: int = 3):
+def time_prefill(cfg, runner, repeats: int = 3, total: int = PROMPT_LEN):
+    """Seconds for one prompt of ``total`` tokens, in portions of PROMPT_LEN tokens (one step when
+    total is PROMPT_LEN, the recorded measurement): the best of ``repeats`` runs."""
     import torch
 
     from clockwork_amd.engine.batch import StepEntry
 
     vocab = runner.spec.vocab_size
-    tokens = torch.randint(0, vocab, (PROMPT_LEN,), generator=torch.Generator().manual_seed(99)).tolist()
+    tokens = torch.randint(0, vocab, (total,), generator=torch.Generator().manual_seed(99)).tolist()
     best = None
     for i in range(repeats + 1):
-        runner.reserve("prefill", 0, PROMPT_LEN)
         _sync()
         t0 = time.perf_counter()
-        logits = runner.step([StepEntry("prefill", 0, tokens, [PROMPT_LEN - 1])])
+        for at in range(0, total, PROMPT_LEN):
+            n = min(PROMPT_LEN, total - at)
+            runner.reserve("prefill", at, n)
+            logits = runner.step([StepEntry("prefill", at, tokens[at:at + n], [n - 1] if at + n == total else [])])
         _sync()
         dt = time.perf_counter() - t0
         runner.release("prefill")
@@ -285,7 +289,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--no-tune", action="store_true", help="leave the matrix library's kernel choice at its default")
-    ap.add_argument("--only-prefill", action="store_true", help="run the 2048-token prefill alone (for profiling)")
+    ap.add_argument("--only-prefill", action="store_true", help="run the prefill alone: 2048 tokens, or --prompt-len tokens in portions of 2048")
     ap.add_argument("--workload", default="decode", choices=("decode", "mixed"),
                     help="decode: the recorded benchmark; mixed: a continuous batch of --requests prompts of mixed lengths")
     ap.add_argument("--requests", type=int, default=64)
@@ -308,8 +312,9 @@ def main() -> int:
         return 0
     cfg, runner = build_runner(args)
     if args.only_prefill:
-        t = time_prefill(cfg, runner)
-        print(json.dumps({"prefill_ms": round(1e3 * t, 3), "tokens_per_s": round(PROMPT_LEN / t, 1)}))
+        t = time_prefill(cfg, runner, total=args.prompt_len)
+        print(json.dumps({"prefill_ms": round(1e3 * t, 3), "tokens": args.prompt_len, "portion": PROMPT_LEN,
+                          "tokens_per_s": round(args.prompt_len / t, 1)}))
         return 0
     sampling = (args.temperature, args.top_k, args.top_p) if args.temperature > 0 else None
     elapsed, mean_ctx = time_decode(cfg, runner, args.batch, args.steps, args.warmup, sampling, args.prompt_len)

@@ -124,10 +124,16 @@ class StepContext:
         mfma: list[int] = []
         # Workgroups of four row blocks share each key among the most rows, but a launch has to
         # fill the compute units, and the workgroup with the longest key range decides its time:
-        # with fewer than 1.5 workgroups a compute unit, halve them.
+        # with fewer than 1.5 workgroups a compute unit, halve them. Behind a long cached prefix
+        # every workgroup's key range is long and about the same, and sharing the keys among more
+        # rows wins again (2048 tokens of the 1.5B shape: 46 against 52 us with no prefix, 94
+        # against 96 us behind 2048 tokens, 197 against 182 us behind 6144).
         tokens_of_four = 4 * (32 // min(group, 32))
         workgroups = sum(-(-q // tokens_of_four) for q in self.h_q_lens if q > 1) * nkv * -(-group // 32)
-        row_blocks = 2 if narrow_ok and 2 * workgroups < 3 * self.num_compute_units else 4
+        portion_tokens = sum(q for q in self.h_q_lens if q > 1)
+        keys = sum(q * (c - q / 2.0) for q, c in zip(self.h_q_lens, self.h_ctx_lens) if q > 1)
+        short_ranges = portion_tokens > 0 and keys / portion_tokens < 3072
+        row_blocks = 2 if narrow_ok and short_ranges and 2 * workgroups < 3 * self.num_compute_units else 4
         tokens_per_mfma_item = row_blocks * (32 // min(group, 32))
         single: list[int] = []
         longest_single = 0
