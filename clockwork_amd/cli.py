@@ -1,4 +1,4 @@
-"""Command line: offline generation from a config file plus KEY=VALUE overrides.
+r"""Command line: offline generation from a config file plus KEY=VALUE overrides.
 
 The option style is the reference's launcher (scripts/serve.py:33-55: ``--config`` naming a
 YAML file with ``model:``, ``cache:``, ``scheduler:`` sections, repeatable ``--set KEY=VALUE``
