@@ -549,8 +549,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnParams p) {
         tmax = fmaxf(tmax, v);
       }
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    tmax = cw_quad_max(tmax);
     const float m_new = fmaxf(m_run, tmax);
     float alpha = 1.0f, psum = 0.0f;
     bf16x8_t pf;
@@ -565,8 +564,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnParams p) {
         pf[e] = (__bf16)pe;
       }
     }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
+    psum = cw_quad_sum(psum);
     l_run = l_run * alpha + psum;
     m_run = m_new;
     if (__any(alpha != 1.0f)) {
@@ -1036,9 +1034,7 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
           tmax[b] = fmaxf(tmax[b], fmaxf(fmaxf(sc[kb][b][0], sc[kb][b][1]), fmaxf(sc[kb][b][2], sc[kb][b][3])));
       }
 #pragma unroll
-      for (int b = 0; b < 2; ++b) tmax[b] = fmaxf(tmax[b], __shfl_xor(tmax[b], 16, 64));
-#pragma unroll
-      for (int b = 0; b < 2; ++b) tmax[b] = fmaxf(tmax[b], __shfl_xor(tmax[b], 32, 64));
+      for (int b = 0; b < 2; ++b) tmax[b] = cw_quad_max(tmax[b]);
       bf16x8_t pf[2][NKB / 2];
       float alpha[2];
 #pragma unroll
@@ -1168,8 +1164,7 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
     float l = l_run[b];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    l = cw_quad_sum(l);
     if (row_pos[b] < 0) continue;
     const float inv = 1.0f / l;
     bf16_t* orow = (bf16_t*)p.out + (int64_t)(q_begin + (row_pos[b] - (ctx - qlen))) * p.out_stride + row_off[b];

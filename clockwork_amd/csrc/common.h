@@ -39,6 +39,24 @@ __device__ __forceinline__ uint16_t cw_float_to_bf16_bits(float f) {
   return (uint16_t)(u >> 16);
 }
 
+// Maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 of a wave, on the vector unit: the
+// swaps of 16-lane rows and of the wave's halves (v_permlane16_swap, v_permlane32_swap) hand every
+// lane both values of its pair, so all four lanes end with the same result, summed as
+// (l + l^16) + (l^32 + l^48). (A shuffle goes through the LDS unit and waits behind its queue.)
+typedef __attribute__((ext_vector_type(2))) unsigned int cw_u32x2_t;
+__device__ __forceinline__ float cw_quad_max(float v) {
+  const cw_u32x2_t a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const cw_u32x2_t b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float cw_quad_sum(float v) {
+  const cw_u32x2_t a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const cw_u32x2_t b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 __device__ __forceinline__ float cw_wave_sum(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);

@@ -336,8 +336,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
         for (int e = 0; e < 8; ++e) ss += v[u][e] * v[u][e];
       }
     }
-    ss += __shfl_xor(ss, 16, 64);
-    ss += __shfl_xor(ss, 32, 64);
+    ss = cw_quad_sum(ss);
     if (s == 0) ssq[wave][r] = ss;
     __syncthreads();
     float total = 0.0f;
