@@ -1084,6 +1084,10 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
 
   fetch(t_first, gk, gv);
   stash(0, gk, gv);
+  // Every load so far (the query fragments among them) has to be home before the loop starts:
+  // the loop's first use of a fragment would otherwise carry a wait for "all loads but the last
+  // few", and in every later round that wait would sit on the stage just requested, in order.
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   if constexpr (DEEP) {
     // set 0 holds stage t + 1 while an even round computes stage t, set 1 stage t + 2; each set is
     // stashed at the end of the round before its stage is computed and filled again at once
