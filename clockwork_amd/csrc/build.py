@@ -33,6 +33,9 @@ FLAGS = [
     "-fvisibility=hidden",
     # hipcc -O3 forms packed float32 instructions by itself; they are kept out of these kernels
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first kernel arguments arrive in scalar registers with the wave instead of by a load
+    # from the argument buffer: a short kernel's first addresses are ready that much sooner
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
 PLAIN_SOURCES = {"core": "core.hip", "gemm": "gemm.hip", "gemm_tile": "gemm_tile.hip", "sampling": "sampling.hip"}
 ATTENTION_SOURCE = "attention.hip"
