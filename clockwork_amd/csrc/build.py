@@ -24,10 +24,29 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent
 ARCH = "gfx950"
+
+
+def target_arch() -> str:
+    """The offload target: gfx950 with XNACK (page-fault replay) ruled out, which is how these
+    cards run and lets the compiler schedule loads more freely; plain gfx950 (code that runs
+    either way) only where the card at hand says it has XNACK on. ``CLOCKWORK_AMD_ARCH`` overrides."""
+    override = os.environ.get("CLOCKWORK_AMD_ARCH")
+    if override:
+        return override
+    torch = sys.modules.get("torch")
+    try:
+        if torch is not None and torch.cuda.is_available():
+            name = torch.cuda.get_device_properties(torch.cuda.current_device()).gcnArchName
+            if "xnack+" in name:
+                return ARCH
+    except Exception:  # no usable card here: cross-compiling
+        pass
+    return f"{ARCH}:xnack-"
+
+
 FLAGS = [
     "-O3",
     "-std=c++17",
-    f"--offload-arch={ARCH}",
     "-shared",
     "-fPIC",
     "-fvisibility=hidden",
@@ -91,7 +110,7 @@ def _digest(src: Path, defines: list[str]) -> str:
     h = hashlib.sha256()
     h.update(src.read_bytes())
     h.update((CSRC / "common.h").read_bytes())
-    h.update(" ".join(FLAGS + defines).encode())
+    h.update(" ".join([f"--offload-arch={target_arch()}"] + FLAGS + defines).encode())
     return h.hexdigest()[:12]
 
 
@@ -116,9 +135,9 @@ def _find_built(name: str, head_dim: int | None) -> Path | None:
 def _compile(name: str, head_dim: int | None, out: Path) -> Path:
     stem, src, defines = _spec(name, head_dim)
     tmp = out.with_suffix(f".tmp{os.getpid()}.so")
-    cmd = [_hipcc(), *FLAGS, *defines, "-I", str(CSRC), "-o", str(tmp), str(src)]
+    cmd = [_hipcc(), f"--offload-arch={target_arch()}", *FLAGS, *defines, "-I", str(CSRC), "-o", str(tmp), str(src)]
     t0 = time.time()
-    _log(f"compiling {stem} for {ARCH} ...")
+    _log(f"compiling {stem} for {target_arch()} ...")
     env = dict(os.environ)
     env.setdefault("HOME", tempfile.gettempdir())
     proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)

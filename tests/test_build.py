@@ -38,3 +38,11 @@ def test_the_digest_follows_the_source_and_the_flags(monkeypatch):
     before = build.library_path("core").name
     monkeypatch.setattr(build, "FLAGS", build.FLAGS + ["-DSOMETHING_ELSE"])
     assert build.library_path("core").name != before
+
+
+def test_the_target_rules_xnack_out_unless_told_otherwise(monkeypatch):
+    monkeypatch.delenv("CLOCKWORK_AMD_ARCH", raising=False)
+    assert build.target_arch() in ("gfx950:xnack-", "gfx950")  # the latter only on a card with XNACK on
+    monkeypatch.setenv("CLOCKWORK_AMD_ARCH", "gfx950")
+    assert build.target_arch() == "gfx950"
+    assert "--offload-arch" not in " ".join(build.FLAGS)  # the target is added per compile
