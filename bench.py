@@ -118,7 +118,7 @@ def time_decode(cfg, runner, batch: int, steps: int, warmup: int, sampling=None,
     return elapsed, mean_ctx
 
 
-def time_prefill(cfg, runner, repeats: int = 3, total: int = PROMPT_LEN):
+def time_prefill(cfg, runner, repeats: int = 6, total: int = PROMPT_LEN):
     """Seconds for one prompt of ``total`` tokens, in portions of PROMPT_LEN tokens (one step when
     total is PROMPT_LEN, the recorded measurement): the best of ``repeats`` runs."""
     import torch
