@@ -20,7 +20,6 @@ _ROLES = ("mixer", "feed_forward", "mixer_norm", "ffn_norm")
 
 def _build_layers(spec: ModelSpec) -> list:
     layers = []
-    built: dict[int, object] = {}
     for layer_spec in spec.layers:
         # identical spec objects still get parts of their own: every layer has its own weights
         layers.append(
@@ -32,7 +31,6 @@ def _build_layers(spec: ModelSpec) -> list:
                 ffn_norm=build_part(layer_spec.ffn_norm),
             )
         )
-    del built
     return layers
 
 
