@@ -21,7 +21,7 @@ is in ``clockwork_amd.cache.pools``.
 
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Optional, Sequence
 
 from clockwork_amd.cache.allocator import OutOfPages, PagePool

@@ -8,7 +8,7 @@ in a single copy; the kernels read device views of that buffer.
 
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Optional, Sequence
 
 import numpy as np

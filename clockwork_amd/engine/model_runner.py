@@ -10,7 +10,6 @@ tokens (clockwork/engine/model_runner.py:48-132); here they are one batch.
 
 from __future__ import annotations
 
-from pathlib import Path
 from typing import Optional, Sequence
 
 import torch
@@ -19,7 +18,7 @@ from clockwork_amd import ops
 from clockwork_amd.cache.manager import CacheManager, cache_needs_of, plan_groups
 from clockwork_amd.cache.pools import CachePools, pages_that_fit
 from clockwork_amd.config.engine import EngineConfig
-from clockwork_amd.engine.batch import StaticDecodeBatch, StepContext, StepEntry, build_context
+from clockwork_amd.engine.batch import StaticDecodeBatch, StepEntry, build_context
 from clockwork_amd.parts.model import DecoderModel
 from clockwork_amd.registry import resolve_architecture
 from clockwork_amd.weights.loader import load_parameters, read_config_json
