@@ -24,6 +24,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Optional, Sequence
 
+import numpy as np
+
 from clockwork_amd.cache.allocator import OutOfPages, PagePool
 from clockwork_amd.config.spec import KVPagesSpec, ModelSpec, StateSpec
 
@@ -325,13 +327,19 @@ class CacheManager:
         covered = len(table) * size
         if not 0 <= start <= end <= covered:
             raise ValueError(f"token range [{start}, {end}) outside covered range [0, {covered})")
-        out = []
-        for pos in range(start, end):
-            page = table[pos // size]
-            if page == NO_PAGE:
-                raise ValueError(f"position {pos} lies in a page that was given back")
-            out.append(page * size + pos % size)
-        return out
+        if end - start <= 8:  # a decoded token or two: not worth an array
+            out = []
+            for pos in range(start, end):
+                page = table[pos // size]
+                if page == NO_PAGE:
+                    raise ValueError(f"position {pos} lies in a page that was given back")
+                out.append(page * size + pos % size)
+            return out
+        pos = np.arange(start, end, dtype=np.int64)
+        pages = np.asarray(table[start // size : (end - 1) // size + 1], dtype=np.int64)[pos // size - start // size]
+        if (pages == NO_PAGE).any():
+            raise ValueError(f"position {int(pos[pages == NO_PAGE][0])} lies in a page that was given back")
+        return (pages * size + pos % size).tolist()
 
     def audit(self) -> None:
         """No page lost or held twice: per pool, holders' counts equal reference counts."""

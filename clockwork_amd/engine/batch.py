@@ -120,8 +120,8 @@ class StepContext:
         gh_wide = min(group, 64)
         tokens_per_tile = 64 // gh_wide
         gh_single = min(group, 16)
-        wide: list[int] = []
-        mfma: list[int] = []
+        wide: list = []   # one array of items per portion
+        mfma: list = []
         # Workgroups of four row blocks share each key among the most rows, but a launch has to
         # fill the compute units, and the workgroup with the longest key range decides its time:
         # with fewer than 1.5 workgroups a compute unit, halve them. Behind a long cached prefix
@@ -137,16 +137,28 @@ class StepContext:
         tokens_per_mfma_item = row_blocks * (32 // min(group, 32))
         single: list[int] = []
         longest_single = 0
+
+        def items_of(r: int, q_len: int, step: int, longest_first: bool) -> np.ndarray:
+            """(request, first token, tokens, 0) for runs of ``step`` tokens of one portion."""
+            tok0 = np.arange(0, q_len, step, dtype=np.int32)
+            if longest_first:
+                tok0 = tok0[::-1]
+            out = np.zeros((tok0.size, 4), dtype=np.int32)
+            out[:, 0] = r
+            out[:, 1] = tok0
+            out[:, 2] = np.minimum(step, q_len - tok0)
+            return out.reshape(-1)
+
         for r, q_len in enumerate(self.h_q_lens):
             if q_len == 1:
                 single += [r, 0, 1, 0]
                 longest_single = max(longest_single, self.h_ctx_lens[r])
             else:
-                for tok0 in range(0, q_len, tokens_per_tile):
-                    wide += [r, tok0, min(tokens_per_tile, q_len - tok0), 0]
+                wide.append(items_of(r, q_len, tokens_per_tile, False))
                 # longest key ranges first: the last tokens of a portion have the most work
-                for tok0 in reversed(range(0, q_len, tokens_per_mfma_item)):
-                    mfma += [r, tok0, min(tokens_per_mfma_item, q_len - tok0), 0]
+                mfma.append(items_of(r, q_len, tokens_per_mfma_item, True))
+        wide = np.concatenate(wide) if wide else np.zeros(0, dtype=np.int32)
+        mfma = np.concatenate(mfma) if mfma else np.zeros(0, dtype=np.int32)
         plan = AttentionPlan(gh_wide=gh_wide, gh_single=gh_single, mfma_row_blocks=row_blocks)
         plan.n_wide, plan.n_single, plan.n_mfma = len(wide) // 4, len(single) // 4, len(mfma) // 4
         plan.chunks_single = -(-group // gh_single)
@@ -180,8 +192,8 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int
     ctx = StepContext()
     ctx.device = device
     ctx.block_size = manager.block_size
-    tokens: list[int] = []
-    positions: list[int] = []
+    tokens: list = []     # one array per entry
+    positions: list = []
     cu = [0]
     logit_rows: list[int] = []
     state_slots: list[int] = []
@@ -189,15 +201,16 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int
         n = len(e.tokens)
         if n < 1:
             raise ValueError(f"request {e.seq_id}: a step entry needs at least one token")
-        for t in e.tokens:
-            if not 0 <= int(t) < vocab_size:
-                raise ValueError(f"request {e.seq_id}: token id {t} outside the vocabulary [0, {vocab_size})")
+        ids = np.asarray(e.tokens, dtype=np.int64)  # a long portion is checked as an array, not token by token
+        if ids.shape != (n,) or ids.min() < 0 or ids.max() >= vocab_size:
+            bad = next((t for t in e.tokens if not 0 <= int(t) < vocab_size), None)
+            raise ValueError(f"request {e.seq_id}: token id {bad} outside the vocabulary [0, {vocab_size})")
         for w in e.want:
             if not 0 <= int(w) < n:
                 raise ValueError(f"request {e.seq_id}: wanted index {w} outside its {n} tokens")
             logit_rows.append(cu[-1] + int(w))
-        tokens += [int(t) for t in e.tokens]
-        positions += range(e.start, e.start + n)
+        tokens.append(ids)
+        positions.append(np.arange(e.start, e.start + n, dtype=np.int64))
         cu.append(cu[-1] + n)
         ctx.h_q_lens.append(n)
         ctx.h_starts.append(e.start)
@@ -209,8 +222,8 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int
     ctx.num_logit_rows = len(logit_rows)
 
     packer = _Packer()
-    i_tok = packer.add(tokens)
-    i_pos = packer.add(positions)
+    i_tok = packer.add(np.concatenate(tokens))
+    i_pos = packer.add(np.concatenate(positions))
     i_cu = packer.add(cu)
     i_ctx = packer.add(ctx.h_ctx_lens)
     i_start = packer.add(ctx.h_starts)
