@@ -132,7 +132,7 @@ class StepContext:
         workgroups = sum(-(-q // tokens_of_four) for q in self.h_q_lens if q > 1) * nkv * -(-group // 32)
         portion_tokens = sum(q for q in self.h_q_lens if q > 1)
         keys = sum(q * (c - q / 2.0) for q, c in zip(self.h_q_lens, self.h_ctx_lens) if q > 1)
-        short_ranges = portion_tokens > 0 and keys / portion_tokens < 3072
+        short_ranges = portion_tokens > 0 and keys / portion_tokens < 3072  # portion_has_long_ranges says the same of one portion
         row_blocks = 2 if narrow_ok and short_ranges and 2 * workgroups < 3 * self.num_compute_units else 4
         tokens_per_mfma_item = row_blocks * (32 // min(group, 32))
         single: list[int] = []
@@ -386,3 +386,111 @@ class StaticDecodeBatch:
         self.device_buf.copy_(self.host, non_blocking=True)
         self._sent = torch.cuda.Event()
         self._sent.record()
+
+
+class StaticPortionBatch:
+    """One request's portion of a fixed number of tokens with fixed shapes, for a captured HIP graph.
+
+    A full-budget portion of a long prompt comes again and again with the same shape: its index
+    arrays live at fixed device addresses, refreshed by one host-to-device copy per step, and its
+    attention work items are made once. ``long_ranges`` only chooses the attention kernel's
+    workgroup shape, as the step's plan would (behind a long cached prefix or not); ``wanted``:
+    the logits of the portion's last token are made (else none).
+    """
+
+    def __init__(self, num_tokens: int, long_ranges: bool, wanted: bool, table_width: int, manager, device,
+                 geometries, num_compute_units: int, vocab_size: int) -> None:
+        self.num_tokens = n = num_tokens
+        self.vocab_size = vocab_size
+        self.table_width = table_width
+        self.block_size = manager.block_size
+        n_groups = len(manager.kv_groups)
+        offsets = {}
+        at = 0
+
+        def take(name, count):
+            nonlocal at
+            offsets[name] = (at, count)
+            at += -(-count // 4) * 4
+
+        take("token_ids", n)
+        take("positions", n)
+        for name in ("ctx_lens", "starts", "state_slots"):
+            take(name, 1)
+        for g in range(n_groups):
+            take(f"slots{g}", n)
+            take(f"table{g}", table_width)
+        self._offsets = offsets
+        self.host = torch.zeros(at, dtype=torch.int32, pin_memory=True)
+        self.device_buf = torch.zeros(at, dtype=torch.int32, device=device)
+        self._np = self.host.numpy()
+
+        def view(name):
+            o, count = offsets[name]
+            return self.device_buf[o : o + count]
+
+        ctx = StepContext()
+        ctx.device = device
+        ctx.block_size = manager.block_size
+        ctx.num_tokens, ctx.num_requests, ctx.num_logit_rows = n, 1, int(wanted)
+        ctx.token_ids, ctx.positions = view("token_ids"), view("positions")
+        ctx.ctx_lens, ctx.starts, ctx.state_slots = view("ctx_lens"), view("starts"), view("state_slots")
+        ctx.cu_q = torch.tensor([0, n], dtype=torch.int32, device=device)
+        ctx.logit_rows = torch.tensor([n - 1] if wanted else [], dtype=torch.int32, device=device)
+        for g in range(n_groups):
+            ctx.slots.append(view(f"slots{g}"))
+            ctx.block_tables.append(view(f"table{g}").view(1, table_width))
+        # what the attention plan looks at: the portion's length and whether its key ranges are long
+        behind = PORTION_LONG_RANGE if long_ranges else 0
+        ctx.h_q_lens = [n]
+        ctx.h_ctx_lens = [behind + n]
+        ctx.h_starts = [behind]
+        ctx.h_state_slots = [-1]
+        ctx.seq_ids = [""]
+        ctx.num_compute_units = num_compute_units
+        for nh, nkv in geometries:  # work items are the same every step: made once, outside the graph
+            for narrow_ok in (False, True):
+                ctx.attention_plan(nh, nkv, narrow_ok=narrow_ok)
+        self.ctx = ctx
+
+    def fill(self, entry: StepEntry, manager) -> None:
+        """This step's indices into the pinned buffer, then to the device."""
+        n, bs, width = self.num_tokens, self.block_size, self.table_width
+        a = self._np
+        sent = getattr(self, "_sent", None)
+        if sent is not None:
+            sent.synchronize()  # the copy of the step before must have read the buffer
+
+        def region(name):
+            o, count = self._offsets[name]
+            return a[o : o + count]
+
+        ids = np.asarray(entry.tokens, dtype=np.int64)
+        if ids.shape != (n,) or ids.min() < 0 or ids.max() >= self.vocab_size:
+            raise ValueError(f"request {entry.seq_id}: a token id outside the vocabulary [0, {self.vocab_size})")
+        region("token_ids")[:] = ids
+        region("positions")[:] = np.arange(entry.start, entry.start + n, dtype=np.int32)
+        region("ctx_lens")[0] = entry.start + n
+        region("starts")[0] = entry.start
+        region("state_slots")[0] = manager.state_slot(entry.seq_id)
+        for g in range(len(manager.kv_groups)):
+            region(f"slots{g}")[:] = manager.slot_mapping(entry.seq_id, entry.start, entry.start + n, g)
+            row = manager.block_table(entry.seq_id, g)
+            if len(row) > width:
+                raise ValueError(f"request {entry.seq_id} holds {len(row)} pages, the graph was sized for {width}")
+            table = region(f"table{g}")
+            table[: len(row)] = row
+            table[len(row) :] = -1
+        self.ctx.seq_ids = [entry.seq_id]
+        self.device_buf.copy_(self.host, non_blocking=True)
+        self._sent = torch.cuda.Event()
+        self._sent.record()
+
+
+# keys a portion has before it when its key ranges count as long (see StepContext._make_plan)
+PORTION_LONG_RANGE = 1 << 16
+
+
+def portion_has_long_ranges(start: int, num_tokens: int) -> bool:
+    """The plan's rule for one portion: its tokens see 3072 keys or more on average."""
+    return start + num_tokens / 2.0 >= 3072

@@ -18,7 +18,13 @@ from clockwork_amd import ops
 from clockwork_amd.cache.manager import CacheManager, cache_needs_of, plan_groups
 from clockwork_amd.cache.pools import CachePools, pages_that_fit
 from clockwork_amd.config.engine import EngineConfig
-from clockwork_amd.engine.batch import StaticDecodeBatch, StepEntry, build_context
+from clockwork_amd.engine.batch import (
+    StaticDecodeBatch,
+    StaticPortionBatch,
+    StepEntry,
+    build_context,
+    portion_has_long_ranges,
+)
 from clockwork_amd.parts.model import DecoderModel
 from clockwork_amd.registry import resolve_architecture
 from clockwork_amd.weights.loader import load_parameters, read_config_json
@@ -186,6 +192,40 @@ class ModelRunner:
             return out[:n]
         return out[torch.tensor(rows, device=self.device)]
 
+    def _portion_graph_step(self, entry: StepEntry):
+        """A step that is one full-budget portion of one request (what a long prompt's prefill is
+        made of) replays a captured graph as the decode steps do: the first step of a shape runs
+        eagerly, the second is captured. Returns NotImplemented when the step has to take the
+        ordinary path."""
+        n = len(entry.tokens)
+        want = [int(w) for w in entry.want]
+        if want not in ([], [n - 1]) or entry.start + n > self._table_width * self.manager.block_size:
+            return NotImplemented
+        key = ("portion", n, portion_has_long_ranges(entry.start, n), bool(want))
+        state = self._graphs.get(key)
+        if state is None:
+            self._graphs[key] = "seen"
+            return NotImplemented
+        if state == "seen":
+            batch = StaticPortionBatch(n, key[2], key[3], self._table_width, self.manager, self.device,
+                                       self.model.attention_geometries(), self.num_compute_units,
+                                       self.spec.vocab_size)
+            batch.fill(entry, self.manager)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                out = self.model.forward(batch.ctx, self.caches)
+            if self._graph_pool is None:
+                self._graph_pool = graph.pool()
+            state = self._graphs[key] = (batch, graph, out)
+            self._drop_old_graphs()
+        self._graphs[key] = self._graphs.pop(key)  # most recently used last
+        batch, graph, out = state
+        batch.fill(entry, self.manager)
+        graph.replay()
+        self.manager.release_behind_window(entry.seq_id, entry.start + n)
+        return out if want else None
+
     def _drop_old_graphs(self) -> None:
         captured = [k for k, v in self._graphs.items() if isinstance(v, tuple)]
         if len(captured) <= GRAPH_LIMIT:
@@ -251,6 +291,12 @@ class ModelRunner:
         if (self.use_graphs and not self.manager.state_groups and len(entries) <= GRAPH_BATCH_SIZES[-1]
                 and all(len(e.tokens) == 1 for e in entries)):
             logits = self._graph_step(entries)
+            if logits is not NotImplemented:
+                return logits
+        if (self.use_graphs and not self.manager.state_groups and len(entries) == 1
+                and len(entries[0].tokens) == self.cfg.scheduler.max_num_batched_tokens
+                and len(entries[0].tokens) > ops.STREAM_MAX_ROWS):
+            logits = self._portion_graph_step(entries[0])
             if logits is not NotImplemented:
                 return logits
         if self.manager.state_groups:

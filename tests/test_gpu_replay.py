@@ -351,6 +351,62 @@ def test_graph_replays_equal_eager_steps(model_dirs, dtype, graph_limit, monkeyp
     replay.compare(got_g, ref, **TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_full_budget_portions_replay_as_graphs(model_dirs, dtype):
+    """A step that is one request's portion of exactly the token budget replays a captured graph
+    from its third occurrence on. Two long prompts are cut into such portions (the last one of
+    each is shorter and runs eagerly), with decode steps, another request's short prompt and a
+    request ending in between; logits are wanted for the last token of some portions and for none
+    of others (two graph shapes). Every step is checked against a runner without graphs and
+    against the plain implementation."""
+    from clockwork_amd.config.engine import EngineConfig
+    from clockwork_amd.engine.model_runner import ModelRunner
+
+    name = "B"
+    cfg, _, block_size = TINY_CONFIGS[name]
+    budget = 72  # more rows than the narrow products take, and not a multiple of the page size
+    gen = torch.Generator().manual_seed(33)
+    toks = {k: torch.randint(0, cfg["vocab_size"], (n,), generator=gen).tolist() for k, n in
+            {"a": 6 * budget + 17, "b": 4 * budget + 5, "c": 30}.items()}
+    steps = []
+    at = {k: 0 for k in toks}
+
+    def portion(rid, n, want_last):
+        e = {"id": rid, "tokens": toks[rid][at[rid] : at[rid] + n], "want": [n - 1] if want_last else []}
+        at[rid] += n
+        return e
+
+    for i in range(6):
+        steps.append({"entries": [portion("a", budget, i % 2 == 0)], "end": []})
+        if i == 1:
+            steps.append({"entries": [portion("c", 29, True)], "end": []})
+        if i >= 1 and at["c"] < len(toks["c"]):
+            steps.append({"entries": [portion("c", 1, True)], "end": ["c"]})
+        if i < 4:
+            steps.append({"entries": [portion("b", budget, i % 2 == 1)], "end": []})
+    steps.append({"entries": [portion("a", 17, True), portion("b", 5, True)], "end": ["a", "b"]})
+    assert all(at[k] == len(v) for k, v in toks.items())
+
+    def runner(use_graphs):
+        ecfg = EngineConfig.defaults(
+            str(model_dirs[name]), dtype=dtype, block_size=block_size, num_blocks=160, enable_prefix_cache=False,
+            watermark=0.0, max_model_len=512, max_num_batched_tokens=budget,
+        )
+        return ModelRunner(ecfg, cache_fill=float("nan"), use_graphs=use_graphs)
+
+    with_graphs, eager = runner(True), runner(False)
+    got_g = replay.run_trace(with_graphs, [dict(s) for s in steps])
+    got_e = replay.run_trace(eager, [dict(s) for s in steps])
+    captured = [k for k, v in with_graphs._graphs.items() if isinstance(v, tuple) and k[0] == "portion"]
+    assert len(captured) == 2, f"portion graphs captured: {captured}"
+    assert got_g.keys() == got_e.keys() and len(got_g) >= 8
+    for key in got_e:  # the same kernels in the same order: the same numbers
+        torch.testing.assert_close(got_g[key], got_e[key], rtol=0, atol=0, msg=lambda m: f"portion graph differs from the eager step at {key}: {m}")
+    model = PlainQwen2(model_dirs[name])
+    ref = {k: model.logits(v) for k, v in toks.items()}
+    replay.compare(got_g, ref, **TOL[dtype])
+
+
 @pytest.mark.parametrize("tuned", [False, True])
 def test_wide_decode_batches_of_a_large_layer_replay_as_eager(tmp_path, tuned):
     """40 requests decoding together through one layer of the 7B shape: at this width some products
