@@ -153,15 +153,16 @@ def _need(cond: bool, msg: str) -> None:
 
 def _gpu(*tensors) -> None:
     for t in tensors:
-        if t is not None:
-            _need(t.is_cuda, "kernel arguments must live on the GPU")
-            _need(t.is_contiguous(), "kernel arguments must be contiguous")
+        if t is not None and not (t.is_cuda and t.is_contiguous()):
+            raise KernelError("kernel arguments must live on the GPU and be contiguous")
 
 
 def _i32(t, n: int | None, what: str) -> None:
-    _need(t.dtype == torch.int32 and t.dim() == 1, f"{what} must be a 1-d int32 tensor")
+    if not (t.dtype == torch.int32 and t.dim() == 1):
+        raise KernelError(f"{what} must be a 1-d int32 tensor")
     if n is not None:
-        _need(t.numel() >= n, f"{what} holds {t.numel()} entries, {n} needed")
+        if not (t.numel() >= n):
+            raise KernelError(f"{what} holds {t.numel()} entries, {n} needed")
 
 
 # ---------------------------------------------------------------------------------------------
@@ -171,7 +172,8 @@ def embedding(table: torch.Tensor, ids: torch.Tensor, out_resid: torch.Tensor) -
     T = ids.numel()
     V, H = table.shape
     _i32(ids, T, "ids")
-    _need(out_resid.dtype == torch.float32 and tuple(out_resid.shape) == (T, H), "residual must be [T, H] float32")
+    if not (out_resid.dtype == torch.float32 and tuple(out_resid.shape) == (T, H)):
+        raise KernelError("residual must be [T, H] float32")
     _check(
         _load("core").cw_embedding(_ptr(table), dtype_code(table.dtype), _ptr(ids), _ptr(out_resid), T, H, V, _stream()),
         "embedding",
@@ -258,18 +260,24 @@ def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_back: bo
         delta = delta.parts
     _gpu(resid, delta, delta0, weight, out, rows)
     T, H = resid.shape
-    _need(resid.dtype == torch.float32, "the residual stream is float32")
+    if not (resid.dtype == torch.float32):
+        raise KernelError("the residual stream is float32")
     if delta0 is not None:
-        _need(tuple(delta0.shape) == (T, H) and delta0.dtype == out.dtype, "the first pending delta must be [T, H] in the activation type")
+        if not (tuple(delta0.shape) == (T, H) and delta0.dtype == out.dtype):
+            raise KernelError("the first pending delta must be [T, H] in the activation type")
     n = T if rows is None else rows.numel()
     if rows is not None:
         _i32(rows, n, "rows")
-    _need(tuple(out.shape) == (n, H), f"out must be [{n}, {H}]")
-    _need(weight.numel() == H, "norm weight has the wrong size")
+    if not (tuple(out.shape) == (n, H)):
+        raise KernelError(f"out must be [{n}, {H}]")
+    if not (weight.numel() == H):
+        raise KernelError("norm weight has the wrong size")
     if parts:
-        _need(tuple(delta.shape) == (parts, T, H) and delta.dtype == torch.float32, "partial sums must be float32 [parts, T, H]")
+        if not (tuple(delta.shape) == (parts, T, H) and delta.dtype == torch.float32):
+            raise KernelError("partial sums must be float32 [parts, T, H]")
     elif delta is not None:
-        _need(tuple(delta.shape) == (T, H) and delta.dtype == out.dtype, "delta must be [T, H] in the activation type")
+        if not (tuple(delta.shape) == (T, H) and delta.dtype == out.dtype):
+            raise KernelError("delta must be [T, H] in the activation type")
     _check(
         _load("core").cw_add_rmsnorm(
             _ptr(resid), _ptr(delta0), _ptr(delta), parts, T, _ptr(weight), dtype_code(weight.dtype), float(eps), _ptr(out),
@@ -288,21 +296,28 @@ def rope_kv_write(qkv, bias, positions, slots, inv_freq, rotary_dim: int, nh: in
     _gpu(qkv, bias, positions, slots, inv_freq, k_cache, v_cache)
     T = qkv.shape[0]
     width = (nh + 2 * nkv) * hd
-    _need(qkv.dim() == 2 and qkv.shape[1] == width, f"qkv must be [T, {width}]")
+    if not (qkv.dim() == 2 and qkv.shape[1] == width):
+        raise KernelError(f"qkv must be [T, {width}]")
     _i32(positions, T, "positions")
     cache_rows = 0
     if slots is not None:
         _i32(slots, T, "slots")
-        _need(k_cache is not None and v_cache is not None, "slots without a cache")
-        _need(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype, "cache and activations differ in type")
-        _need(tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape, "cache must be [..., nkv, hd]")
+        if not (k_cache is not None and v_cache is not None):
+            raise KernelError("slots without a cache")
+        if not (k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype):
+            raise KernelError("cache and activations differ in type")
+        if not (tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape):
+            raise KernelError("cache must be [..., nkv, hd]")
         cache_rows = k_cache.numel() // (nkv * hd)
     else:
-        _need(nkv == 0, "keys and values need slots to be written to")
+        if not (nkv == 0):
+            raise KernelError("keys and values need slots to be written to")
     if bias is not None:
-        _need(bias.numel() == width, "qkv bias has the wrong size")
+        if not (bias.numel() == width):
+            raise KernelError("qkv bias has the wrong size")
     if inv_freq is not None:
-        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == rotary_dim // 2, "inv_freq must be float32 [rotary_dim / 2]")
+        if not (inv_freq.dtype == torch.float32 and inv_freq.numel() == rotary_dim // 2):
+            raise KernelError("inv_freq must be float32 [rotary_dim / 2]")
     else:
         rotary_dim = 0
     _check(
@@ -318,7 +333,8 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
     _gpu(gate_up, out)
     T, two_i = gate_up.shape
-    _need(two_i % 2 == 0 and tuple(out.shape) == (T, two_i // 2) and out.dtype == gate_up.dtype, "silu_mul shapes")
+    if not (two_i % 2 == 0 and tuple(out.shape) == (T, two_i // 2) and out.dtype == gate_up.dtype):
+        raise KernelError("silu_mul shapes")
     _check(_load("core").cw_silu_mul(_ptr(gate_up), _ptr(out), dtype_code(out.dtype), T, two_i // 2, _stream()), "silu_mul")
     return out
 
@@ -328,7 +344,8 @@ def copy_pages(pool: torch.Tensor, pairs: torch.Tensor) -> None:
     _gpu(pool, pairs)
     planes, num_blocks = pool.shape[0], pool.shape[1]
     block_bytes = pool[0, 0].numel() * pool.element_size()
-    _need(pairs.dtype == torch.int32 and pairs.dim() == 2 and pairs.shape[1] == 2, "pairs must be int32 [n, 2]")
+    if not (pairs.dtype == torch.int32 and pairs.dim() == 2 and pairs.shape[1] == 2):
+        raise KernelError("pairs must be int32 [n, 2]")
     _check(_load("core").cw_copy_pages(_ptr(pool), planes, num_blocks, block_bytes, _ptr(pairs), pairs.shape[0], _stream()), "copy_pages")
 
 
@@ -341,15 +358,19 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
     _gpu(x, weight, bias)
     M, K = x.shape
     N = weight.shape[0]
-    _need(weight.shape[1] == K, f"weight is {tuple(weight.shape)}, input has {K} columns")
+    if not (weight.shape[1] == K):
+        raise KernelError(f"weight is {tuple(weight.shape)}, input has {K} columns")
     if x.dtype == torch.float32:
-        _need(weight.dtype == torch.float32, "a float32 product needs float32 weights")
+        if not (weight.dtype == torch.float32):
+            raise KernelError("a float32 product needs float32 weights")
         out = torch.empty((M, N), dtype=torch.float32, device=x.device)
         if bias is not None:
-            _need(bias.dtype == torch.float32 and bias.numel() == N, "bias must be float32 [N]")
+            if not (bias.dtype == torch.float32 and bias.numel() == N):
+                raise KernelError("bias must be float32 [N]")
         _check(_load("gemm").cw_gemm_f32(_ptr(x), K, _ptr(weight), _ptr(bias), _ptr(out), N, M, N, K, _stream()), "gemm_f32")
         return out
-    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "a bfloat16 product needs bfloat16 operands")
+    if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16):
+        raise KernelError("a bfloat16 product needs bfloat16 operands")
     if M <= STREAM_MAX_ROWS and K % 8 == 0 and bias is None:
         lib = _load("gemm")
         if partial_ok and out_dtype is None:
@@ -401,14 +422,19 @@ def linear_tiled(x: torch.Tensor, weight: torch.Tensor, bias=None, swiglu: bool 
     [gate; up], through the LDS-tiled matrix-core kernel for many bfloat16 rows (csrc/gemm_tile.hip).
     The rows of x may have a stride (a slice of a wider buffer)."""
     _gpu(weight, bias)
-    _need(x.is_cuda and x.dim() == 2, "x must be a 2-d tensor on the GPU")
+    if not (x.is_cuda and x.dim() == 2):
+        raise KernelError("x must be a 2-d tensor on the GPU")
     M, K = x.shape
     N = weight.shape[0]
-    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "the tiled product is bfloat16")
-    _need(weight.shape[1] == K and K % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0, "rows of 16-byte multiples")
-    _need(not swiglu or (N % 2 == 0 and bias is None), "gate_up weight must be [2 I, K], without bias")
+    if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16):
+        raise KernelError("the tiled product is bfloat16")
+    if not (weight.shape[1] == K and K % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0):
+        raise KernelError("rows of 16-byte multiples")
+    if not (not swiglu or (N % 2 == 0 and bias is None)):
+        raise KernelError("gate_up weight must be [2 I, K], without bias")
     if bias is not None:
-        _need(bias.numel() == N and bias.dtype in (torch.bfloat16, torch.float32), "bias must be [N] bfloat16 or float32")
+        if not (bias.numel() == N and bias.dtype in (torch.bfloat16, torch.float32)):
+            raise KernelError("bias must be [N] bfloat16 or float32")
     out = torch.empty((M, N // 2 if swiglu else N), dtype=torch.bfloat16, device=x.device)
     _check(
         _load("gemm_tile").cw_gemm_bf16_tiled(
@@ -453,15 +479,19 @@ def qkv_rope_fused(x, weight, bias, positions, slots, inv_freq, nh: int, nkv: in
     to the cache rows ``slots``: one kernel for few bfloat16 rows (see csrc/gemm.hip)."""
     _gpu(x, weight, bias, positions, slots, inv_freq, k_cache, v_cache)
     M, K = x.shape
-    _need(qkv_rope_fused_supported(x, weight, hd, hd), "the fused q/k/v kernel does not take these operands")
-    _need(tuple(weight.shape) == ((nh + 2 * nkv) * hd, K), "qkv weight must be [(nh + 2 nkv) hd, K]")
+    if not (qkv_rope_fused_supported(x, weight, hd, hd)):
+        raise KernelError("the fused q/k/v kernel does not take these operands")
+    if not (tuple(weight.shape) == ((nh + 2 * nkv) * hd, K)):
+        raise KernelError("qkv weight must be [(nh + 2 nkv) hd, K]")
     _i32(positions, M, "positions")
     _i32(slots, M, "slots")
-    _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == hd // 2, "inv_freq must be float32 [hd / 2]")
+    if not (inv_freq.dtype == torch.float32 and inv_freq.numel() == hd // 2):
+        raise KernelError("inv_freq must be float32 [hd / 2]")
     _need(k_cache.dtype == torch.bfloat16 and tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape,
           "cache must be bfloat16 [..., nkv, hd]")
     if bias is not None:
-        _need(bias.numel() == weight.shape[0] and bias.dtype in (torch.bfloat16, torch.float32), "qkv bias")
+        if not (bias.numel() == weight.shape[0] and bias.dtype in (torch.bfloat16, torch.float32)):
+            raise KernelError("qkv bias")
     q = torch.empty((M, nh * hd), dtype=torch.bfloat16, device=x.device)
     _check(
         _load("gemm").cw_gemm_qkv_rope_bf16(
@@ -503,11 +533,13 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
     _gpu(x, gate_up_weight)
     M, K = x.shape
     two_i = gate_up_weight.shape[0]
-    _need(gate_up_weight.shape[1] == K and two_i % 2 == 0, "gate_up weight must be [2 I, K]")
+    if not (gate_up_weight.shape[1] == K and two_i % 2 == 0):
+        raise KernelError("gate_up weight must be [2 I, K]")
     out = torch.empty((M, two_i // 2), dtype=x.dtype, device=x.device)
     if (x.dtype == torch.bfloat16 and M <= STREAM_MAX_ROWS and K % 8 == 0
             and _load("gemm").cw_gemm_bf16_skinny_fast(2, M, two_i, K)):
-        _need(gate_up_weight.dtype == torch.bfloat16, "a bfloat16 product needs bfloat16 operands")
+        if not (gate_up_weight.dtype == torch.bfloat16):
+            raise KernelError("a bfloat16 product needs bfloat16 operands")
         _check(_load("gemm").cw_gemm_bf16_skinny(2, _ptr(x), K, _ptr(gate_up_weight), _ptr(out), two_i // 2, M, two_i, K, _stream()),
                "gemm_bf16_skinny(swiglu)")
         return out
@@ -537,16 +569,23 @@ def attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx
     """Portions of prompts through the bfloat16 matrix-core kernel; an item holds at most
     ``prefill_tokens_per_item(nh // nkv, row_blocks)`` tokens. ``row_blocks`` 2 instead of 4: smaller
     workgroups for launches with few items (head sizes up to 128). Other arguments as for ``attention``."""
-    _need(prefill_row_blocks_ok(hd, row_blocks), f"the kernel for head size {hd} does not take {row_blocks} row blocks")
+    if not (prefill_row_blocks_ok(hd, row_blocks)):
+        raise KernelError(f"the kernel for head size {hd} does not take {row_blocks} row blocks")
     _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items)
-    _need(q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16, "the kernel is bfloat16")
-    _need(out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd, "attention output must be [T, nh * hd]")
-    _need(q_stride >= nh * hd, "query rows overlap")
-    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= n_requests, "block_tables must be int32 [R, max_blocks]")
+    if not (q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16):
+        raise KernelError("the kernel is bfloat16")
+    if not (out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd):
+        raise KernelError("attention output must be [T, nh * hd]")
+    if not (q_stride >= nh * hd):
+        raise KernelError("query rows overlap")
+    if not (block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= n_requests):
+        raise KernelError("block_tables must be int32 [R, max_blocks]")
     _i32(ctx_lens, n_requests, "ctx_lens")
     _i32(cu_q, n_requests + 1, "cu_q")
-    _need(items.dtype == torch.int32 and items.numel() >= 4 * n_items, "items must be int32 [n_items, 4]")
-    _need(tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape, "cache must be [..., nkv, hd]")
+    if not (items.dtype == torch.int32 and items.numel() >= 4 * n_items):
+        raise KernelError("items must be int32 [n_items, 4]")
+    if not (tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape):
+        raise KernelError("cache must be [..., nkv, hd]")
     _check(
         _load("attention", hd).cw_attention_prefill_bf16(
             q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
@@ -587,18 +626,26 @@ def attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_
     with its token in row i (no other items). ``split_keys`` > 0: every split takes that many
     keys at a fixed place; no context may then be longer than ``max_ctx`` <= n_splits * split_keys."""
     _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, workspace)
-    _need(q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16, "the decode kernel is bfloat16")
-    _need(out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd, "attention output must be [T, nh * hd]")
-    _need(q_stride >= nh * hd, "query rows overlap")
-    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= n_requests, "block_tables must be int32 [R, max_blocks]")
+    if not (q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16):
+        raise KernelError("the decode kernel is bfloat16")
+    if not (out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd):
+        raise KernelError("attention output must be [T, nh * hd]")
+    if not (q_stride >= nh * hd):
+        raise KernelError("query rows overlap")
+    if not (block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= n_requests):
+        raise KernelError("block_tables must be int32 [R, max_blocks]")
     _i32(ctx_lens, n_requests, "ctx_lens")
     _i32(cu_q, n_requests + 1, "cu_q")
-    _need(items.dtype == torch.int32 and items.numel() >= 4 * n_items, "items must be int32 [n_items, 4]")
-    _need(tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape, "cache must be [..., nkv, hd]")
+    if not (items.dtype == torch.int32 and items.numel() >= 4 * n_items):
+        raise KernelError("items must be int32 [n_items, 4]")
+    if not (tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape):
+        raise KernelError("cache must be [..., nkv, hd]")
     if identity:
-        _need(n_items == n_requests == n_tokens, "identity items: one single-token item per request, nothing else")
+        if not (n_items == n_requests == n_tokens):
+            raise KernelError("identity items: one single-token item per request, nothing else")
     if split_keys:
-        _need(split_keys % 32 == 0 and split_keys * n_splits >= max_ctx > 0, "fixed key ranges do not cover the longest context")
+        if not (split_keys % 32 == 0 and split_keys * n_splits >= max_ctx > 0):
+            raise KernelError("fixed key ranges do not cover the longest context")
     lib = _load("attention", hd)
     need = lib.cw_attention_decode_workspace_floats(n_items, nh, nkv, n_splits)
     ws_floats = 0
@@ -625,14 +672,20 @@ def attention(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, c
     out [n_tokens, nh * hd]; caches [num_blocks * block_size, nkv, hd]; block_tables int32
     [n_requests, max_blocks]; items int32 [n_items, 4] = (request, first token, tokens, 0)."""
     _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, workspace)
-    _need(q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype, "attention operands differ in type or device")
-    _need(out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd, "attention output must be [T, nh * hd]")
-    _need(q_stride >= nh * hd, "query rows overlap")
-    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= n_requests, "block_tables must be int32 [R, max_blocks]")
+    if not (q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype):
+        raise KernelError("attention operands differ in type or device")
+    if not (out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd):
+        raise KernelError("attention output must be [T, nh * hd]")
+    if not (q_stride >= nh * hd):
+        raise KernelError("query rows overlap")
+    if not (block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= n_requests):
+        raise KernelError("block_tables must be int32 [R, max_blocks]")
     _i32(ctx_lens, n_requests, "ctx_lens")
     _i32(cu_q, n_requests + 1, "cu_q")
-    _need(items.dtype == torch.int32 and items.numel() >= 4 * n_items, "items must be int32 [n_items, 4]")
-    _need(tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape, "cache must be [..., nkv, hd]")
+    if not (items.dtype == torch.int32 and items.numel() >= 4 * n_items):
+        raise KernelError("items must be int32 [n_items, 4]")
+    if not (tuple(k_cache.shape[-2:]) == (nkv, hd) and k_cache.shape == v_cache.shape):
+        raise KernelError("cache must be [..., nkv, hd]")
     lib = _load("attention", hd)
     group = nh // nkv
     n_chunks = -(-group // gh)
@@ -658,7 +711,8 @@ def attention_workspace_floats(hd: int, rows: int, n_items: int, nkv: int, n_chu
 def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """First index of the maximum of every row of float32 ``logits`` [n, V] -> int32 [n]."""
     _gpu(logits, out)
-    _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be float32 [n, V]")
+    if not (logits.dtype == torch.float32 and logits.dim() == 2):
+        raise KernelError("logits must be float32 [n, V]")
     n, V = logits.shape
     lib = _load("sampling")
     chunks = lib.cw_argmax_chunks(V)
@@ -676,13 +730,18 @@ def sample(logits, temperature, top_k, top_p, seeds, draws, out=None, any_top_k:
     ``any_top_k`` / ``any_top_p`` off: the caller knows that no row has that option, and its
     kernels are not launched."""
     _gpu(logits, temperature, top_k, top_p, seeds, draws, out)
-    _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be float32 [n, V]")
+    if not (logits.dtype == torch.float32 and logits.dim() == 2):
+        raise KernelError("logits must be float32 [n, V]")
     n, V = logits.shape
-    _need(temperature.dtype == torch.float32 and temperature.numel() == n, "temperature must be float32 [n]")
-    _need(top_p.dtype == torch.float32 and top_p.numel() == n, "top_p must be float32 [n]")
+    if not (temperature.dtype == torch.float32 and temperature.numel() == n):
+        raise KernelError("temperature must be float32 [n]")
+    if not (top_p.dtype == torch.float32 and top_p.numel() == n):
+        raise KernelError("top_p must be float32 [n]")
     _i32(top_k, n, "top_k")
-    _need(seeds.dtype == torch.int64 and seeds.numel() == n, "seeds must be int64 [n]")
-    _need(draws.dtype == torch.int64 and draws.numel() == n, "draws must be int64 [n]")
+    if not (seeds.dtype == torch.int64 and seeds.numel() == n):
+        raise KernelError("seeds must be int64 [n]")
+    if not (draws.dtype == torch.int64 and draws.numel() == n):
+        raise KernelError("draws must be int64 [n]")
     if out is None:
         out = torch.empty(n, dtype=torch.int32, device=logits.device)
     _i32(out, n, "out")
