@@ -102,10 +102,14 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(AttnParams p) {
   const int kvh = blockIdx.y / p.n_chunks;
   const int chunk = blockIdx.y % p.n_chunks;
   const int split = blockIdx.z;
-  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1], ntok = p.items[4 * item + 2];
+  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1];
   const int ctx = p.ctx_lens[req];
   const int q_begin = p.cu_q[req];
   const int qlen = p.cu_q[req + 1] - q_begin;
+  // an item may reach past the request's tokens (work items laid out for a longer portion than
+  // the step brings): what lies past them is not computed
+  const int ntok = min(p.items[4 * item + 2], qlen - tok0);
+  if (ntok <= 0) return;
   const int group = p.nh / p.nkv;
   const int gh = p.gh;
   const int pos0 = ctx - qlen + tok0;  // absolute position of the item's first token
@@ -876,12 +880,16 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
   const int c = lane & 15, s = lane >> 4;
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / p.n_chunks, chunk = blockIdx.y % p.n_chunks;
-  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1], ntok = p.items[4 * item + 2];
+  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1];
   const int gh = p.gh;
   const int tpw = 32 / gh;  // tokens of a wave
   const int ctx = p.ctx_lens[req];
   const int q_begin = p.cu_q[req];
   const int qlen = p.cu_q[req + 1] - q_begin;
+  // an item may reach past the request's tokens (work items laid out for a longer portion than
+  // the step brings): what lies past them is not computed
+  const int ntok = min(p.items[4 * item + 2], qlen - tok0);
+  if (ntok <= 0) return;
   const int group = p.nh / p.nkv;
   const int pos0 = ctx - qlen + tok0;
   const int wg_last = pos0 + ntok - 1;

@@ -389,13 +389,16 @@ class StaticDecodeBatch:
 
 
 class StaticPortionBatch:
-    """One request's portion of a fixed number of tokens with fixed shapes, for a captured HIP graph.
+    """One request's portion of up to ``num_tokens`` tokens with fixed shapes, for a captured HIP graph.
 
-    A full-budget portion of a long prompt comes again and again with the same shape: its index
-    arrays live at fixed device addresses, refreshed by one host-to-device copy per step, and its
-    attention work items are made once. ``long_ranges`` only chooses the attention kernel's
-    workgroup shape, as the step's plan would (behind a long cached prefix or not); ``wanted``:
-    the logits of the portion's last token are made (else none).
+    A full-budget portion of a long prompt comes again and again with the same shape, and a short
+    prompt fits the next larger of a few sizes: the index arrays live at fixed device addresses,
+    refreshed by one host-to-device copy per step, and the attention work items are made once, for
+    ``num_tokens`` tokens. A shorter portion leaves rows at the end that belong to no request:
+    token 0, no cache slot, past the request's tokens as ``cu_q`` counts them, so no attention
+    item computes them and nothing reads what the other kernels make of them. ``long_ranges``
+    only chooses the attention kernel's workgroup shape, as the step's plan would (behind a long
+    cached prefix or not); ``wanted``: the logits of the portion's last token are made (else none).
     """
 
     def __init__(self, num_tokens: int, long_ranges: bool, wanted: bool, table_width: int, manager, device,
@@ -415,8 +418,9 @@ class StaticPortionBatch:
 
         take("token_ids", n)
         take("positions", n)
-        for name in ("ctx_lens", "starts", "state_slots"):
+        for name in ("ctx_lens", "starts", "state_slots", "logit_rows"):
             take(name, 1)
+        take("cu_q", 2)
         for g in range(n_groups):
             take(f"slots{g}", n)
             take(f"table{g}", table_width)
@@ -435,8 +439,8 @@ class StaticPortionBatch:
         ctx.num_tokens, ctx.num_requests, ctx.num_logit_rows = n, 1, int(wanted)
         ctx.token_ids, ctx.positions = view("token_ids"), view("positions")
         ctx.ctx_lens, ctx.starts, ctx.state_slots = view("ctx_lens"), view("starts"), view("state_slots")
-        ctx.cu_q = torch.tensor([0, n], dtype=torch.int32, device=device)
-        ctx.logit_rows = torch.tensor([n - 1] if wanted else [], dtype=torch.int32, device=device)
+        ctx.cu_q = view("cu_q")
+        ctx.logit_rows = view("logit_rows") if wanted else torch.empty(0, dtype=torch.int32, device=device)
         for g in range(n_groups):
             ctx.slots.append(view(f"slots{g}"))
             ctx.block_tables.append(view(f"table{g}").view(1, table_width))
@@ -455,7 +459,9 @@ class StaticPortionBatch:
 
     def fill(self, entry: StepEntry, manager) -> None:
         """This step's indices into the pinned buffer, then to the device."""
-        n, bs, width = self.num_tokens, self.block_size, self.table_width
+        n, width = len(entry.tokens), self.table_width
+        if not 0 < n <= self.num_tokens:
+            raise ValueError(f"request {entry.seq_id}: {n} tokens for a batch of {self.num_tokens}")
         a = self._np
         sent = getattr(self, "_sent", None)
         if sent is not None:
@@ -468,13 +474,20 @@ class StaticPortionBatch:
         ids = np.asarray(entry.tokens, dtype=np.int64)
         if ids.shape != (n,) or ids.min() < 0 or ids.max() >= self.vocab_size:
             raise ValueError(f"request {entry.seq_id}: a token id outside the vocabulary [0, {self.vocab_size})")
-        region("token_ids")[:] = ids
-        region("positions")[:] = np.arange(entry.start, entry.start + n, dtype=np.int32)
+        tok, pos = region("token_ids"), region("positions")
+        tok[:n] = ids
+        tok[n:] = 0
+        pos[:n] = np.arange(entry.start, entry.start + n, dtype=np.int32)
+        pos[n:] = 0
         region("ctx_lens")[0] = entry.start + n
         region("starts")[0] = entry.start
         region("state_slots")[0] = manager.state_slot(entry.seq_id)
+        region("logit_rows")[0] = n - 1
+        region("cu_q")[:] = (0, n)
         for g in range(len(manager.kv_groups)):
-            region(f"slots{g}")[:] = manager.slot_mapping(entry.seq_id, entry.start, entry.start + n, g)
+            slots = region(f"slots{g}")
+            slots[:n] = manager.slot_mapping(entry.seq_id, entry.start, entry.start + n, g)
+            slots[n:] = -1
             row = manager.block_table(entry.seq_id, g)
             if len(row) > width:
                 raise ValueError(f"request {entry.seq_id} holds {len(row)} pages, the graph was sized for {width}")

@@ -33,6 +33,9 @@ from clockwork_amd.weights.loader import load_parameters, read_config_json
 # padded batch sizes a decode graph is captured for, and the step in which the planned context grows
 GRAPH_BATCH_SIZES = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)
 GRAPH_KEY_BUCKET = 512
+# a step that is one request's portion replays a graph captured for the token budget or for the
+# next of these sizes (a step of 65 to 500 tokens is otherwise bound by the host's launches)
+PORTION_GRAPH_SIZES = (128, 256, 384, 512)
 # captured graphs kept at a time (each holds index buffers of its own): the least recently
 # replayed one goes when another shape is captured beyond this many
 GRAPH_LIMIT = 48
@@ -193,21 +196,25 @@ class ModelRunner:
         return out[torch.tensor(rows, device=self.device)]
 
     def _portion_graph_step(self, entry: StepEntry):
-        """A step that is one full-budget portion of one request (what a long prompt's prefill is
-        made of) replays a captured graph as the decode steps do: the first step of a shape runs
-        eagerly, the second is captured. Returns NotImplemented when the step has to take the
-        ordinary path."""
+        """A step that is one portion of one request, of the token budget (what a long prompt's
+        prefill is made of) or of up to 512 tokens (a short prompt), replays a captured graph as
+        the decode steps do: the first step of a shape runs eagerly, the second is captured.
+        Returns NotImplemented when the step has to take the ordinary path."""
         n = len(entry.tokens)
         want = [int(w) for w in entry.want]
         if want not in ([], [n - 1]) or entry.start + n > self._table_width * self.manager.block_size:
             return NotImplemented
-        key = ("portion", n, portion_has_long_ranges(entry.start, n), bool(want))
+        budget = self.cfg.scheduler.max_num_batched_tokens
+        size = n if n == budget else next((b for b in PORTION_GRAPH_SIZES if b >= n), None)
+        if size is None:
+            return NotImplemented
+        key = ("portion", size, portion_has_long_ranges(entry.start, n), bool(want))
         state = self._graphs.get(key)
         if state is None:
             self._graphs[key] = "seen"
             return NotImplemented
         if state == "seen":
-            batch = StaticPortionBatch(n, key[2], key[3], self._table_width, self.manager, self.device,
+            batch = StaticPortionBatch(size, key[2], key[3], self._table_width, self.manager, self.device,
                                        self.model.attention_geometries(), self.num_compute_units,
                                        self.spec.vocab_size)
             batch.fill(entry, self.manager)
@@ -294,7 +301,6 @@ class ModelRunner:
             if logits is not NotImplemented:
                 return logits
         if (self.use_graphs and not self.manager.state_groups and len(entries) == 1
-                and len(entries[0].tokens) == self.cfg.scheduler.max_num_batched_tokens
                 and len(entries[0].tokens) > ops.STREAM_MAX_ROWS):
             logits = self._portion_graph_step(entries[0])
             if logits is not NotImplemented:

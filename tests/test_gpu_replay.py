@@ -407,6 +407,55 @@ def test_full_budget_portions_replay_as_graphs(model_dirs, dtype):
     replay.compare(got_g, ref, **TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_short_prompts_replay_padded_graphs(model_dirs, dtype):
+    """A step that is one request's portion of 65 to 512 tokens replays a graph captured for the
+    next of a few sizes: the rows past the portion belong to no request. Prompts of many lengths
+    around those sizes, each followed by a second portion (so the padded step also runs behind
+    cached keys, and its own keys are read back) and a few single tokens; the pools are poisoned
+    with NaN, so a read past a request's tokens would show. Checked against a runner without
+    graphs and against the plain implementation."""
+    from clockwork_amd.config.engine import EngineConfig
+    from clockwork_amd.engine.model_runner import ModelRunner
+
+    name = "C"
+    cfg, _, block_size = TINY_CONFIGS[name]
+    gen = torch.Generator().manual_seed(44)
+    firsts = [65, 100, 128, 129, 127, 70, 200, 256, 257, 300, 384, 90, 500, 512, 260, 130]
+    toks, steps = {}, []
+    for i, n in enumerate(firsts):
+        rid = f"r{i}"
+        second = 66 + (i * 37) % 120
+        toks[rid] = torch.randint(0, cfg["vocab_size"], (n + second + 3,), generator=gen).tolist()
+        steps.append({"entries": [{"id": rid, "tokens": toks[rid][:n], "want": [n - 1]}], "end": []})
+        steps.append({"entries": [{"id": rid, "tokens": toks[rid][n : n + second], "want": [second - 1] if i % 2 else []}], "end": []})
+        for j in range(3):
+            at = n + second + j
+            steps.append({"entries": [{"id": rid, "tokens": toks[rid][at : at + 1], "want": [0]}], "end": [rid] if j == 2 else []})
+
+    def runner(use_graphs):
+        ecfg = EngineConfig.defaults(
+            str(model_dirs[name]), dtype=dtype, block_size=block_size, num_blocks=64, enable_prefix_cache=False,
+            watermark=0.0, max_model_len=1024,
+        )
+        return ModelRunner(ecfg, cache_fill=float("nan"), use_graphs=use_graphs)
+
+    with_graphs, eager = runner(True), runner(False)
+    got_g = replay.run_trace(with_graphs, [dict(s) for s in steps])
+    got_e = replay.run_trace(eager, [dict(s) for s in steps])
+    captured = sorted(k[1] for k, v in with_graphs._graphs.items() if isinstance(v, tuple) and k[0] == "portion")
+    assert set(captured) >= {128, 256, 384, 512}, f"portion graphs captured: {captured}"
+    assert got_g.keys() == got_e.keys()
+    # padded steps run products of more rows than the eager ones, so another kernel may take them,
+    # and the single tokens' graphs split their keys otherwise than eager steps: equal up to rounding
+    close = dict(rtol=2e-6, atol=2e-6) if dtype == "float32" else dict(rtol=2e-2, atol=2e-2)
+    for key in got_e:
+        torch.testing.assert_close(got_g[key], got_e[key], **close, msg=lambda m: f"padded graph differs from the eager step at {key}: {m}")
+    model = PlainQwen2(model_dirs[name])
+    ref = {k: model.logits(v) for k, v in toks.items()}
+    replay.compare(got_g, ref, **TOL[dtype])
+
+
 @pytest.mark.parametrize("tuned", [False, True])
 def test_wide_decode_batches_of_a_large_layer_replay_as_eager(tmp_path, tuned):
     """40 requests decoding together through one layer of the 7B shape: at this width some products
