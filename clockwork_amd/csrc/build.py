@@ -1,7 +1,7 @@
 """Compile the HIP sources for gfx950 into shared libraries, in-tree, on demand.
 
 Each source becomes one library ``_build/<name>-<hash>.so``; the hash covers the
-source text, the shared header and the compiler flags, so a changed source is
+source text, the headers beside it and the compiler flags, so a changed source is
 never served by a stale library. The attention source is built once per head
 size (``-DCW_HD=<n>``): a model compiles only the size it needs. Libraries are
 plain C ABI (no Python or torch headers), loaded with ctypes.
@@ -109,7 +109,8 @@ def _spec(name: str, head_dim: int | None) -> tuple[str, Path, list[str]]:
 def _digest(src: Path, defines: list[str]) -> str:
     h = hashlib.sha256()
     h.update(src.read_bytes())
-    h.update((CSRC / "common.h").read_bytes())
+    for header in sorted(CSRC.glob("*.h")):
+        h.update(header.read_bytes())
     h.update(" ".join([f"--offload-arch={target_arch()}"] + FLAGS + defines).encode())
     return h.hexdigest()[:12]
 

@@ -8,6 +8,9 @@
 // the first index whose running sum of weights, taken in index order, exceeds u * total. A row's
 // result depends on that row, its seed and its draw index only.
 #include "common.h"
+#include "sampling.h"
+
+#include <mutex>
 
 
 __device__ __forceinline__ uint32_t order_key(float x) {
@@ -86,6 +89,57 @@ CW_EXPORT int cw_argmax(const float* logits, int64_t row_stride, int n, int V, i
   if (workspace == nullptr || workspace_bytes < (int64_t)n * chunks * 8) return CW_ERR_ARG;
   float* pv = (float*)workspace;
   int* pi = (int*)(pv + (int64_t)n * chunks);
+  hipLaunchKernelGGL(argmax_partial_kernel, dim3(chunks, n), dim3(256), 0, stream, logits, row_stride, V, chunks, pv, pi);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(n), dim3(64), 0, stream, pv, pi, chunks, V, out);
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- arg-max without a workspace
+// For callers that cannot allocate (see sampling.h): the partial results live in this array, one
+// copy on every GPU that loads the library. In host code its name is only a handle for
+// hipGetSymbolAddress; the kernels get the address that call returned for the current GPU.
+static __device__ __align__(256) unsigned char scratch[CW_ARGMAX_STATIC_BYTES];
+static_assert(CW_ARGMAX_STATIC_BYTES == CW_ARGMAX_STATIC_MAX_ROWS * ARGMAX_MAX_CHUNKS * 8, "scratch holds a value and an index per row and chunk");
+
+#define ARGMAX_STATIC_MAX_DEVICES 64
+static void* scratch_of_device[ARGMAX_STATIC_MAX_DEVICES];
+static std::mutex scratch_lock;
+
+// The array's address on the current GPU, looked up at the first call on that GPU.
+static int argmax_static_scratch(void** out) {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) return CW_ERR_LAUNCH;
+  if (device < 0 || device >= ARGMAX_STATIC_MAX_DEVICES) return CW_ERR_SIZE;
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (scratch_of_device[device] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      return CW_ERR_LAUNCH;
+    }
+    scratch_of_device[device] = ptr;
+  }
+  *out = scratch_of_device[device];
+  return CW_OK;
+}
+
+CW_EXPORT int cw_argmax_static_init(void) {
+  void* ptr = nullptr;
+  return argmax_static_scratch(&ptr);
+}
+
+CW_EXPORT int cw_argmax_static(const float* logits, int64_t row_stride, int n, int V, int* out,
+                               hipStream_t stream) {
+  if (n < 0 || V <= 0 || row_stride < V || logits == nullptr || out == nullptr) return CW_ERR_ARG;
+  if (n == 0) return CW_OK;
+  if (n > CW_ARGMAX_STATIC_MAX_ROWS) return CW_ERR_SIZE;
+  void* ptr = nullptr;
+  const int status = argmax_static_scratch(&ptr);
+  if (status != CW_OK) return status;
+  const int chunks = cw_argmax_chunks(V);
+  // values in the first half of the array, indices in the second, wherever n and chunks end
+  float* pv = (float*)ptr;
+  int* pi = (int*)((unsigned char*)ptr + CW_ARGMAX_STATIC_BYTES / 2);
   hipLaunchKernelGGL(argmax_partial_kernel, dim3(chunks, n), dim3(256), 0, stream, logits, row_stride, V, chunks, pv, pi);
   hipLaunchKernelGGL(argmax_final_kernel, dim3(n), dim3(64), 0, stream, pv, pi, chunks, V, out);
   return cw_launch_status();

@@ -107,6 +107,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
         "sampling": {
             "cw_argmax_chunks": [I],
             "cw_argmax": [P, L, I, I, P, P, L, P],
+            "cw_argmax_static_init": [],
+            "cw_argmax_static": [P, L, I, I, P, P],
             "cw_sample": [P, L, I, I, P, P, P, P, P, P, P, L, I, P],
             "cw_sample_workspace_bytes": [I, I],
         },
