@@ -10,6 +10,8 @@ tokens (clockwork/engine/model_runner.py:48-132); here they are one batch.
 
 from __future__ import annotations
 
+import contextlib
+import gc
 from typing import Optional, Sequence
 
 import torch
@@ -39,6 +41,22 @@ PORTION_GRAPH_SIZES = (128, 256, 384, 512)
 # captured graphs kept at a time (each holds index buffers of its own): the least recently
 # replayed one goes when another shape is captured beyond this many
 GRAPH_LIMIT = 48
+
+
+@contextlib.contextmanager
+def capturing(graph: "torch.cuda.CUDAGraph", pool):
+    """Capture the launches made inside into ``graph``. The cyclic garbage collector is off
+    meanwhile: if it ran in the middle of a capture and found an unreachable runner, destroying
+    that runner's captured graphs and device memory would be HIP calls that a capturing stream
+    does not permit, and the error they raise inside a destructor ends the process."""
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph, pool=pool):
+            yield
+    finally:
+        if was_enabled:
+            gc.enable()
 
 
 def require_gpu() -> torch.device:
@@ -118,6 +136,29 @@ class ModelRunner:
         for g, pairs in by_group.items():
             self.pools.copy_pages(g, pairs)
 
+    def share_prefix(self, seq_id: str, source_id: str, num_tokens: int) -> None:
+        """Admit ``seq_id`` as a request whose first ``num_tokens`` tokens are the ones the live
+        request ``source_id`` has cached: it holds the same pages (what a prefix-cache hit gives
+        a request) and goes on at position ``num_tokens``. A last page that is only partly
+        covered is shared too; whoever writes to it first gets a copy of its own (``reserve``)."""
+        if self.manager.has(seq_id):
+            raise ValueError(f"request {seq_id} holds pages already")
+        blocks = -(-num_tokens // self.manager.block_size)
+        if num_tokens < 1 or any(blocks > len(self.manager.block_table(source_id, g))
+                                 for g in range(len(self.manager.kv_groups))):
+            raise ValueError(f"request {source_id} does not hold {num_tokens} tokens to share")
+        handles = self.manager.handles(source_id, blocks)
+        self.manager.admit(seq_id, num_tokens, prefix=handles)  # refuses models whose cache cannot be shared
+        for handle in handles:
+            self.manager.share_handle(handle)
+
+    def fork(self, parent_id: str, child_id: str) -> None:
+        """``child_id`` starts as a copy of the live request ``parent_id``: every page shared
+        (copied when either writes into it), fixed-size state copied now."""
+        slots = self.manager.fork(parent_id, child_id)
+        if slots is not None:
+            self.pools.copy_state(*slots)
+
     def release(self, seq_id: str) -> None:
         if self.manager.has(seq_id):
             self.manager.free(seq_id)
@@ -176,7 +217,7 @@ class ModelRunner:
             batch.fill(entries, self.manager)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
+            with capturing(graph, self._graph_pool):
                 out = self.model.forward(batch.ctx, self.caches)
             if self._graph_pool is None:
                 self._graph_pool = graph.pool()
@@ -220,7 +261,7 @@ class ModelRunner:
             batch.fill(entry, self.manager)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
+            with capturing(graph, self._graph_pool):
                 out = self.model.forward(batch.ctx, self.caches)
             if self._graph_pool is None:
                 self._graph_pool = graph.pool()

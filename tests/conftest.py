@@ -31,5 +31,11 @@ def model_dirs(tmp_path_factory):
     from tests.configs import TINY_CONFIGS
     from clockwork_amd.weights.random_init import write_random_model
 
+    from tests.replay import sharpen
+
     root = tmp_path_factory.mktemp("models")
-    return {name: write_random_model(root / name, cfg, seed) for name, (cfg, seed, _) in TINY_CONFIGS.items()}
+    dirs = {name: write_random_model(root / name, cfg, seed) for name, (cfg, seed, _) in TINY_CONFIGS.items()}
+    # the same models with peaked attention: a wrong key shows in their logits
+    for name in ("A", "B"):
+        dirs[name + "_peaked"] = sharpen(dirs[name], root / (name + "_peaked"))
+    return dirs

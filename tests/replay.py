@@ -19,19 +19,17 @@ def make_runner(model_dir, dtype: str, block_size: int, num_blocks: int, poison:
     return ModelRunner(cfg, cache_fill=poison, use_graphs=use_graphs)
 
 
-def run_trace(runner: ModelRunner, steps) -> dict:
-    """``steps``: list of dicts {"entries": [{"id", "tokens", "want"}], "end": [...]} as trace_run
-    reads them. Returns {(id, absolute position): float32 logits row on the CPU}."""
-    lengths: dict[str, int] = {}
+def run_trace(runner: ModelRunner, steps, usage: dict | None = None) -> dict:
+    """``steps``: list of dicts {"entries": [{"id", "tokens", "want"}], "end": [...], and the
+    optional "share" / "fork"} as trace_run reads them, run by the program's own ``TraceReplayer``.
+    Returns {(id, absolute position): float32 logits row on the CPU}. ``usage`` (a dict) receives
+    "peak_pages": the most pages of a pool that were held while a step ran."""
+    from clockwork_amd.engine.trace_run import TraceReplayer
+
+    replayer = TraceReplayer(runner)
     got = {}
     for step in steps:
-        entries = []
-        for e in step["entries"]:
-            start = lengths.get(e["id"], 0)
-            runner.reserve(e["id"], start, len(e["tokens"]))
-            entries.append(StepEntry(e["id"], start, e["tokens"], e.get("want", [])))
-            lengths[e["id"]] = start + len(e["tokens"])
-        logits = runner.step(entries)
+        entries, logits = replayer.run_step(step)
         if logits is not None:
             logits = logits.cpu()
             row = 0
@@ -40,9 +38,8 @@ def run_trace(runner: ModelRunner, steps) -> dict:
                     got[(e.seq_id, e.start + w)] = logits[row]
                     row += 1
             assert row == logits.shape[0]
-        for seq_id in step.get("end", []):
-            runner.release(seq_id)
-            lengths.pop(seq_id, None)
+    if usage is not None:
+        usage["peak_pages"] = replayer.peak_pages
     return got
 
 
@@ -113,6 +110,149 @@ def mixed(requests: dict, live: int = 4, decode_tail: int = 8, sizes=PORTIONS) -
         active = [rec for rec in active if rec[0] not in ended]
         tick += 1
     return steps
+
+
+def shared(a: list, vocab: int, block_size: int, seed: int = 0):
+    """Requests that hold the same pages. ``a`` is the tokens of request A, which runs throughout;
+    beside it, at most four live at a time:
+
+    * C is forked from A in the middle of a page; in that step A writes first, so A gets the copy;
+    * B begins with A's first two pages (a prefix-cache hit: the share ends at a page's edge);
+    * D begins with A's first page and three tokens of the second: it writes into a page that
+      A, B and C hold as well, behind tokens of A's that are not D's;
+    * G is forked from A later and writes first, so the child gets the copy;
+    * E and F are strangers that arrive when others have ended and take the pages given back,
+      among them pages that were copied from and copied to.
+
+    Every request goes on with tokens of its own, in portions and single tokens, and every
+    position's logits are wanted. Returns (steps, {id: the request's whole token sequence},
+    {id: the position at which the request's own steps begin})."""
+    import random
+
+    rng = random.Random(seed)
+    bs = block_size
+    fork_at = 2 * bs + bs // 2 + 1
+    assert len(a) >= fork_at + 3 * bs, "request A is too short for this trace"
+
+    def tail(n):
+        return [rng.randrange(vocab) for _ in range(n)]
+
+    seqs = {"A": list(a)}
+    at: dict[str, int] = {}
+    starts: dict[str, int] = {"A": 0}
+    live: list[str] = []
+    steps: list[dict] = []
+    sizes = [3, 1, 1, 5, 1, 2, 1, 1, 7, 1]
+
+    def join(step, rid, kind, count=None, own=0):
+        if kind == "fork":
+            seqs[rid] = seqs["A"][: at["A"]] + tail(own)
+            at[rid] = at["A"]
+            step.setdefault("fork", []).append({"id": rid, "from": "A"})
+        elif kind == "share":
+            seqs[rid] = seqs["A"][:count] + tail(own)
+            at[rid] = count
+            step.setdefault("share", []).append({"id": rid, "from": "A", "tokens": count})
+        else:
+            seqs[rid] = tail(own)
+            at[rid] = 0
+        starts[rid] = at[rid]
+        live.append(rid)
+
+    # who joins, as soon as fewer than four requests are live (A must still be there for a fork)
+    arrivals = [("C", "fork", None, 2 * bs + 3), ("B", "share", 2 * bs, bs + 5), ("D", "share", bs + 3, 6),
+                ("G", "fork", None, bs + 2), ("E", "new", None, 3 * bs + 1), ("F", "new", None, 2 * bs + 2)]
+    at["A"] = 0
+    live.append("A")
+    steps.append({"entries": [{"id": "A", "tokens": a[:fork_at], "want": list(range(fork_at))}], "end": []})
+    at["A"] = fork_at
+    tick = 0
+    while live:
+        step: dict = {"entries": [], "end": []}
+        joined = []
+        while arrivals and len(live) < 4 and (arrivals[0][1] == "new" or "A" in live):
+            rid, kind, count, own = arrivals.pop(0)
+            join(step, rid, kind, count, own)
+            joined.append(rid)
+        if arrivals and "A" not in live and arrivals[0][1] != "new":
+            raise AssertionError("request A ended before every fork and share was made")
+        # A first in the step of C's fork (A copies), the newcomer first in G's (the child copies)
+        order = list(live)
+        if "G" in joined:
+            order.remove("G")
+            order.insert(0, "G")
+        elif tick % 2 and not joined:
+            order.reverse()
+        for i, rid in enumerate(order):
+            toks = seqs[rid]
+            if rid == "A":
+                n = 1
+            elif rid in ("E", "F") and at[rid] == 0:
+                n = len(toks) - 4
+            else:
+                n = sizes[(tick + i) % len(sizes)]
+            n = min(n, len(toks) - at[rid])
+            step["entries"].append({"id": rid, "tokens": toks[at[rid] : at[rid] + n], "want": list(range(n))})
+            at[rid] += n
+            if at[rid] == len(toks):
+                step["end"].append(rid)
+        assert len(live) <= 4
+        live[:] = [rid for rid in live if rid not in step["end"]]
+        steps.append(step)
+        tick += 1
+    assert not arrivals
+    return steps, seqs, starts
+
+
+def compare_to_scale(got: dict, plain_logits: dict, rms_bound: float = 2e-2, worst_bound: float = 1e-1) -> tuple:
+    """For bfloat16, whose every activation is rounded to 8 bits: the errors relative to the
+    logits' own scale (their root mean square over everything compared). Their root mean square
+    must stay within ``rms_bound`` of it and the largest within ``worst_bound``: rounding gives
+    about one hundredth, a wrong key, mask or weight row moves logits by the scale itself.
+    Returns (scale, rms error, largest error)."""
+    assert got, "the replay produced no logits"
+    keys = sorted(got)
+    ref = torch.stack([plain_logits[rid][pos] for rid, pos in keys]).float()
+    rows = torch.stack([got[k] for k in keys])
+    bad = torch.isnan(rows).any(dim=1)
+    assert not bool(bad.any()), f"NaN in the logits of {keys[int(bad.nonzero()[0])]}"
+    errors = rows - ref
+    scale = ref.square().mean().sqrt().item()
+    rms = errors.square().mean().sqrt().item()
+    per_row = errors.abs().max(dim=1).values
+    worst = per_row.max().item()
+    assert rms < rms_bound * scale, f"rms error {rms:.3e} against a scale of {scale:.3e}"
+    assert worst < worst_bound * scale, (
+        f"request and position {keys[int(per_row.argmax())]}: error {worst:.3e} against a scale of {scale:.3e}")
+    return scale, rms, worst
+
+
+def sharpen(src_dir, dst_dir, score_std: float = 2.0):
+    """A copy of a random-weights model folder whose attention is peaked: query and key
+    projections scaled so that a score's standard deviation is about ``score_std`` instead of the
+    few hundredths that N(0, 0.02) weights give. Then a few keys carry most of each softmax, and a
+    key that is missed, read twice or read from a stale page moves the logits by their own scale
+    (with near-uniform attention over a hundred keys it would move them by a hundredth of it).
+    At 2.0 about one key in twenty of a hundred carries the softmax, and the rounding of bfloat16
+    queries and keys, which the exponential magnifies, still stays inside the bfloat16 bound
+    (measured: 1.2% root mean square, 8% at worst, of the logits' scale; 1.5% and 11% at 2.5)."""
+    import json
+    from pathlib import Path
+
+    from safetensors.torch import load_file, save_file
+
+    src_dir, dst_dir = Path(src_dir), Path(dst_dir)
+    cfg = json.loads((src_dir / "config.json").read_text())
+    # scores of unit-variance inputs through N(0, 0.02) projections: std = hidden * 0.02^2
+    factor = (score_std / (cfg["hidden_size"] * 0.02 ** 2)) ** 0.5
+    tensors = load_file(str(src_dir / "model.safetensors"))
+    for name in list(tensors):
+        if ".q_proj." in name or ".k_proj." in name:
+            tensors[name] = (tensors[name].float() * factor).to(tensors[name].dtype)
+    dst_dir.mkdir(parents=True, exist_ok=True)
+    (dst_dir / "config.json").write_text(json.dumps(cfg))
+    save_file(tensors, str(dst_dir / "model.safetensors"))
+    return dst_dir
 
 
 def pages_needed(requests: dict, live: int, block_size: int) -> int:

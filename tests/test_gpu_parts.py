@@ -277,8 +277,10 @@ def toy_dir(tmp_path_factory):
     return write_random_model(tmp_path_factory.mktemp("toy") / "toy", config, seed=3)
 
 
-def _toy_plain_logits(model_dir, tokens):
-    """The toy model from the plain formulas, whole sequence, no cache."""
+def _toy_plain_logits(model_dir, tokens, close_calls=None):
+    """The toy model from the plain formulas, whole sequence, no cache. ``close_calls`` (a list)
+    receives the positions whose second and third router logits lie within 0.1 of each other: a
+    rounding of the router's input can send such a token to another expert."""
     from safetensors.torch import load_file
 
     cfg = json.loads((model_dir / "config.json").read_text())
@@ -328,6 +330,9 @@ def _toy_plain_logits(model_dir, tokens):
             y = torch.zeros(T, H)
             for t in range(T):  # token by token, expert by expert
                 best = sorted(range(3), key=lambda e: -float(gates[t, e]))[:2]
+                ranked = sorted(float(g) for g in gates[t].log())  # logits up to a common shift
+                if close_calls is not None and ranked[1] - ranked[0] < 0.1:
+                    close_calls.append(t)
                 total = sum(float(gates[t, e]) for e in best)
                 for e in best:
                     hidden = torch.relu(w[p + "feed_forward.w_in"][e] @ x[t])
@@ -350,9 +355,23 @@ def test_a_toy_architecture_registers_builds_and_steps(toy_dir, dtype, mode):
     assert [(g.is_kv, g.window, g.entries) for g in runner.manager.groups] == [(True, None, (0, 5)), (True, 6, (1, 2)), (False, None, (3,))]
     assert not runner.manager.supports_prefix_sharing
     got = replay.run_trace(runner, getattr(replay, mode)(requests))
-    ref = {rid: _toy_plain_logits(toy_dir, toks) for rid, toks in requests.items()}
-    tol = dict(rtol=1e-5, atol=1e-5) if dtype == "float32" else dict(rtol=3e-2, atol=3e-2)
-    replay.compare(got, ref, **tol)
+    close = {rid: [] for rid in requests}
+    ref = {rid: _toy_plain_logits(toy_dir, toks, close[rid]) for rid, toks in requests.items()}
+    if dtype == "float32":
+        replay.compare(got, ref, rtol=1e-5, atol=1e-5)
+    else:
+        # Routing is a discrete choice: where two experts' gates nearly tie, the rounding of
+        # bfloat16 may choose the other one, which is no fault. Those positions are left out (the
+        # routed layer is the last, so a choice touches its own position only); float32 checks them.
+        sure = {key: row for key, row in got.items() if key[1] not in close[key[0]]}
+        assert len(sure) > 0.9 * len(got)
+        # The largest error allowed is 20% of the logits' scale here, not the 10% of the Qwen2
+        # models (the root mean square keeps its 2%): this toy's experts have weights five times
+        # as large as its other layers, so the last feed-forward decides the logits and passes on
+        # whatever rounding its input carries; at a sequence's first positions attention averages
+        # one to four values, its rounded output weighs most beside the exact embedding, and
+        # errors reach 15% of the scale there (2% elsewhere). float32 holds 1e-5 at every position.
+        replay.compare_to_scale(sure, ref, worst_bound=2e-1)
     assert not runner.manager.live_requests()
     assert [p.num_free for p in runner.manager.pools] == [64, 64]
 
