@@ -91,12 +91,14 @@ def _make_random(argv) -> int:
     p.add_argument("--config-json", required=True, help="a config.json of a supported architecture")
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--out", required=True)
+    p.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16",
+                   help="how the tensors are stored; float32 keeps the full mantissas of the drawn values")
     args = p.parse_args(argv)
     from clockwork_amd.weights.random_init import write_random_model
 
     with open(args.config_json, encoding="utf-8") as f:
         config = json.load(f)
-    print(write_random_model(args.out, config, args.seed))
+    print(write_random_model(args.out, config, args.seed, dtype=args.dtype))
     return 0
 
 

@@ -26,9 +26,12 @@ class RandomSource:
     """Stands in for a :class:`CheckpointIndex`: the same names and shapes, values drawn on demand."""
 
     def __init__(self, plan: list[WeightTarget], param_specs: dict[str, ParamSpec], seed: int,
-                 device="cpu", skip_optional: bool = True) -> None:
+                 device="cpu", skip_optional: bool = True, dtype: str = "bfloat16") -> None:
+        if dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"random weights come as bfloat16 or float32, not {dtype!r}")
         self.seed = int(seed)
         self.device = device
+        self.dtype = dtype
         self._init: dict[str, tuple] = {}
         shapes: dict[str, tuple[int, ...]] = {}
         for target in plan:
@@ -38,7 +41,8 @@ class RandomSource:
                 shapes[name] = tuple(shape)
                 self._init[name] = param_specs[target.param].init
         self._order = {name: i for i, name in enumerate(sorted(shapes))}
-        self.entries = {name: _Entry(shape, "BF16") for name, shape in shapes.items()}
+        tag = "BF16" if dtype == "bfloat16" else "F32"
+        self.entries = {name: _Entry(shape, tag) for name, shape in shapes.items()}
 
     def read(self, name: str):
         import torch
@@ -57,7 +61,8 @@ class RandomSource:
             t = torch.zeros(shape, dtype=torch.float32, device=self.device)
         else:
             raise ValueError(f"unknown init {init!r}")
-        return t.to(torch.bfloat16)
+        # float32: the values as drawn, with full mantissas (no bfloat16 number among them but by chance)
+        return t if self.dtype == "float32" else t.to(torch.bfloat16)
 
 
 def _describe(config: dict):
@@ -69,15 +74,17 @@ def _describe(config: dict):
     return arch, cfg, spec, arch.weight_plan(cfg, spec), model_param_specs(spec)
 
 
-def random_checkpoint_tensors(config: dict, seed: int, device="cpu") -> dict:
-    """``{checkpoint tensor name: bfloat16 tensor}`` for the architecture that ``config`` names."""
+def random_checkpoint_tensors(config: dict, seed: int, device="cpu", dtype: str = "bfloat16") -> dict:
+    """``{checkpoint tensor name: tensor}`` for the architecture that ``config`` names, bfloat16
+    or (``dtype="float32"``) float32 values that bfloat16 cannot hold."""
     _, _, _, plan, specs = _describe(config)
-    source = RandomSource(plan, specs, seed, device=device)
+    source = RandomSource(plan, specs, seed, device=device, dtype=dtype)
     return {name: source.read(name) for name in sorted(source.entries)}
 
 
-def write_random_model(out_dir: str | Path, config: dict, seed: int) -> Path:
-    """Write ``config.json`` and ``model.safetensors`` (bfloat16) into ``out_dir``."""
+def write_random_model(out_dir: str | Path, config: dict, seed: int, dtype: str = "bfloat16") -> Path:
+    """Write ``config.json`` and ``model.safetensors`` (bfloat16, or float32 tensors with full
+    mantissas for ``dtype="float32"``) into ``out_dir``."""
     from safetensors.torch import save_file
 
     out = Path(out_dir)
@@ -85,8 +92,8 @@ def write_random_model(out_dir: str | Path, config: dict, seed: int) -> Path:
     config = dict(config)
     arch, _, _, _, _ = _describe(config)
     config.setdefault("architectures", [arch.name])
-    config.setdefault("torch_dtype", "bfloat16")
-    tensors = random_checkpoint_tensors(config, seed)
+    config.setdefault("torch_dtype", dtype)
+    tensors = random_checkpoint_tensors(config, seed, dtype=dtype)
     (out / "config.json").write_text(json.dumps(config, indent=2) + "\n", encoding="utf-8")
     save_file({k: v.contiguous() for k, v in tensors.items()}, str(out / "model.safetensors"))
     return out

@@ -136,19 +136,50 @@ def test_eight_staggered_requests_equal_each_alone(model_dirs):
     assert e.manager.min_free_blocks() == 128
 
 
-def test_prefix_cache_second_pass_is_identical_and_counts_cached_tokens(model_dirs):
-    # tests/test_llm_engine.py:134-165: lengths [12, 10, 15, 8], pages of 4 -> cached [8, 8, 12, 4]
-    name = "A"
-    prompts = prompts_for(name, [12, 10, 15, 8], seed=5)
-    e = engine(model_dirs[name])
+def follows_plain(plain, prompt, tokens, stops=()) -> None:
+    """``tokens`` are the plain implementation's greedy tokens; in bfloat16, up to the first place
+    where rounding flips a near-tie: there the plain logits of the two tokens must lie within a
+    twentieth of the logits' scale (a wrong key or page moves them by the scale itself)."""
+    ids = list(prompt)
+    for i, token in enumerate(tokens):
+        row = plain.logits(ids)[-1]
+        best = int(row.argmax())
+        if token != best:
+            gap, scale = float(row[best] - row[token]), float(row.square().mean().sqrt())
+            assert gap < 0.05 * scale, f"token {i}: {token} instead of {best}, {gap:.3e} apart at a scale of {scale:.3e}"
+            return
+        ids.append(token)
+        if token in stops:
+            assert i == len(tokens) - 1
+            return
+
+
+# tests/test_llm_engine.py:134-165: lengths [12, 10, 15, 8], pages of 4 -> cached [8, 8, 12, 4];
+# the same with pages of 8 on the other model
+PREFIX_CASES = {"A": (4, [12, 10, 15, 8], [8, 8, 12, 4]), "B_peaked": (8, [24, 20, 30, 16], [16, 16, 24, 8])}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(PREFIX_CASES))
+def test_prefix_cache_second_pass_is_identical_and_counts_cached_tokens(model_dirs, name, dtype):
+    block_size, lengths, cached = PREFIX_CASES[name]
+    prompts = prompts_for(name[0], lengths, seed=5)
+    e = engine(model_dirs[name], dtype=dtype, block_size=block_size)
     first = e.generate(prompts, greedy(6))
     assert [o.num_cached_tokens for o in first] == [0, 0, 0, 0]
-    second = e.generate(prompts, greedy(6))
-    assert [o.num_cached_tokens for o in second] == [8, 8, 12, 4]
-    assert [o.token_ids for o in second] == [o.token_ids for o in first]
-    off = engine(model_dirs[name], enable_prefix_cache=False).generate(prompts, greedy(6))
-    assert [o.token_ids for o in off] == [o.token_ids for o in first]
-    assert e.stats()["prefix_cache_hit_tokens"] == 32
+    second = e.generate(prompts, greedy(6))   # reads pages that the first pass's requests wrote
+    assert [o.num_cached_tokens for o in second] == cached
+    assert e.stats()["prefix_cache_hit_tokens"] == sum(cached)
+    off = engine(model_dirs[name], dtype=dtype, block_size=block_size, enable_prefix_cache=False).generate(prompts, greedy(6))
+    plain = PlainQwen2(model_dirs[name])
+    if dtype == "float32":
+        assert [o.token_ids for o in second] == [o.token_ids for o in first] == [o.token_ids for o in off]
+        assert [o.token_ids for o in first] == [plain.greedy(p, 6) for p in prompts]
+    else:
+        # a hit runs the rest of the prompt as a step of another shape: other kernels, other rounding
+        for outs in (first, second, off):
+            for prompt, o in zip(prompts, outs):
+                follows_plain(plain, prompt, o.token_ids)
 
 
 def test_shared_prefix_accounting(model_dirs):
@@ -166,16 +197,22 @@ def test_shared_prefix_accounting(model_dirs):
     assert s["prefix_cache_hit_rate"] == 48 / 76
 
 
-def test_preemption_leaves_outputs_unchanged(model_dirs):
-    # tests/test_llm_engine.py:203-219: 8 pages of 4, three requests of 8 + 8 tokens
-    name = "A"
-    prompts = prompts_for(name, [8, 8, 8], seed=11)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,block_size", [("A", 4), ("B_peaked", 8)])
+def test_preemption_leaves_outputs_unchanged(model_dirs, name, block_size, dtype):
+    # tests/test_llm_engine.py:203-219: 8 pages of 4, three requests of 8 + 8 tokens (pages of 8: 16 + 16)
+    n = 2 * block_size
+    prompts = prompts_for(name[0], [n, n, n], seed=11)
     plain = PlainQwen2(model_dirs[name])
-    e = engine(model_dirs[name], num_blocks=8, enable_prefix_cache=False)
-    outs = e.generate(prompts, greedy(8))
+    e = engine(model_dirs[name], dtype=dtype, block_size=block_size, num_blocks=8, enable_prefix_cache=False)
+    outs = e.generate(prompts, greedy(n))
     assert e.stats()["num_preempted_total"] > 0
     for p, o in zip(prompts, outs):
-        assert o.token_ids == plain.greedy(p, 8)
+        if dtype == "float32":
+            assert o.token_ids == plain.greedy(p, n)
+        else:
+            assert len(o.token_ids) == n
+            follows_plain(plain, p, o.token_ids)
     assert e.manager.min_free_blocks() == 8
 
 
@@ -408,3 +445,17 @@ def test_long_random_session_equals_every_request_alone(model_dirs, seed):
         if rid not in aborted:
             out = alone.generate([prompt], params(n, stops))[0]
             assert (out.token_ids, out.finish_reason) == finals[rid], rid
+    # and the engine alone is right: a sample of the requests against the plain implementation
+    plain = PlainQwen2(model_dirs[name])
+    checked = 0
+    for rid, prompt, n, stops in requests:
+        if rid in aborted or n > 40 or checked == 12:
+            continue
+        want = []
+        for token in plain.greedy(prompt, n):
+            want.append(token)
+            if token in stops:
+                break
+        assert finals[rid][0] == want, rid
+        checked += 1
+    assert checked == 12

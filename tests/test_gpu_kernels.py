@@ -64,6 +64,76 @@ def test_add_rmsnorm(dtype, wdtype, T, H, eps):
     torch.testing.assert_close(out2.float(), want[rows.long()], **tol(dtype))
 
 
+def _norm_cast_orders(v: torch.Tensor, weight: torch.Tensor, eps: float):
+    """rmsnorm of float32 rows ``v`` with a bfloat16 ``weight``, rounded the reference's way,
+    weight * bfloat16(x / rms) (clockwork/engine/model.py:49: the cast comes before the weight),
+    and the other way, bfloat16(weight * x / rms). Both bfloat16."""
+    xhat = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    first = weight.to(torch.bfloat16) * xhat.to(torch.bfloat16)          # a bfloat16 product: rounded once more
+    other = (weight.float() * xhat).to(torch.bfloat16)
+    return first, other
+
+
+@pytest.mark.parametrize("T,H", [(6, 1536), (5, 100), (3, 4104), (4, 70)])
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
+def test_rmsnorm_rounds_before_the_weight_multiplies(T, H, wdtype):
+    """The order of the two roundings of a bfloat16 norm, which a tolerance cannot see: weights far
+    from 1 with full mantissas make weight * bfloat16(x) and bfloat16(weight * x) differ in the last
+    bit of about a third of the elements. The kernel (both its vector and its scalar form, with a
+    delta and with selected rows) must give the first, bit for bit; one element in a thousand is
+    allowed to differ, where the float32 statistic's own last bit decides a rounding."""
+    from clockwork_amd import ops
+
+    resid = torch.randn(T, H, device=DEV) * 2
+    delta = torch.randn(T, H, device=DEV).to(torch.bfloat16)
+    weight = (1.37 + 0.41 * torch.randn(H, device=DEV)).to(torch.bfloat16)   # bfloat16 values either way
+    first, other = _norm_cast_orders((resid + delta.float()).cpu(), weight.cpu(), 1e-6)
+    assert float((first != other).float().mean()) > 0.15, "the inputs do not tell the two orders apart"
+    out = torch.empty(T, H, device=DEV, dtype=torch.bfloat16)
+    ops.add_rmsnorm(resid.clone(), delta, weight.to(wdtype), 1e-6, out)
+    assert float((out.cpu() != first).float().mean()) < 1e-3
+    rows = torch.tensor([T - 1, 1], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, H, device=DEV, dtype=torch.bfloat16)
+    ops.add_rmsnorm(resid.clone(), delta, weight.to(wdtype), 1e-6, out2, rows)
+    assert float((out2.cpu() != first[rows.long().cpu()]).float().mean()) < 1e-3
+
+
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
+def test_norm_inside_the_gate_up_product_rounds_before_the_weight_multiplies(wdtype):
+    """The same pin for the norm that the gate/up product makes for itself. Its normed row is not
+    written anywhere, so the weights are chosen to show it: up row j is the unit vector of element
+    j % K and gate row j four times the unit vector of another element, so that (products with 1
+    and 4 and sums with zeros being exact) output j is silu(4 n[a]) * n[b] for two elements of the
+    normed row n. The expected outputs are made from the row rounded the reference's way and from
+    the row rounded the other way; the kernel must follow the first."""
+    from clockwork_amd import ops
+
+    M, K, I = 7, 1024, 4096
+    resid = torch.randn(M, K, device=DEV) * 2
+    delta = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    weight = (1.37 + 0.41 * torch.randn(K, device=DEV)).to(torch.bfloat16)
+    j = torch.arange(I)
+    gate_at, up_at = (7 * j + 3) % K, j % K
+    w = torch.zeros(2 * I, K)
+    w[j, gate_at] = 4.0
+    w[I + j, up_at] = 1.0
+    w = w.to(torch.bfloat16).to(DEV)
+    assert ops.swiglu_norm_fusable(M, 2 * I, K, torch.bfloat16, w, delta)
+    got = ops.linear_swiglu(ops.LazyAddNorm(resid, delta, weight.to(wdtype), 1e-6, torch.bfloat16), w).cpu()
+    first, other = _norm_cast_orders((resid + delta.float()).cpu(), weight.cpu(), 1e-6)
+
+    def outputs(n):
+        n = n.double()
+        g = 4.0 * n[:, gate_at]
+        return (g / (1.0 + torch.exp(-g)) * n[:, up_at]).to(torch.bfloat16)
+
+    want, wrong = outputs(first), outputs(other)
+    assert float((want != wrong).float().mean()) > 0.15, "the inputs do not tell the two orders apart"
+    # the kernel's float32 exponential may decide a rounding otherwise now and then
+    assert float((got != want).float().mean()) < 5e-3
+    assert float((got != wrong).float().mean()) > 0.15
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1536, 8960), (8, 1536, 8960), (16, 96, 4096), (3, 1000, 5000 * 8)])
 def test_split_k_partial_sums_feed_the_norm(M, N, K):
     """A narrow product with a long K comes back as float32 partial sums; the norm kernel adds them

@@ -210,6 +210,33 @@ def test_odd_sizes_replay_like_the_plain_implementation(tmp_path, name, dtype):
         assert runner.manager.min_free_blocks() == runner.manager.num_blocks
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("mode", ["prefill_then_decode", "mixed"])
+def test_float32_weights_with_full_mantissas(tmp_path, name, mode):
+    """The other tests' checkpoints are bfloat16, so their "float32" weights have 8-bit mantissas
+    and every product of two of them is exact in float32. Here the folder holds float32 tensors as
+    drawn: a float32 path that dropped low bits of its operands anywhere would miss the 1e-5 bar."""
+    from clockwork_amd.weights.random_init import write_random_model
+
+    cfg, seed, block_size = TINY_CONFIGS[name]
+    model_dir = write_random_model(tmp_path / name, cfg, seed, dtype="float32")
+    from safetensors.torch import load_file
+
+    stored = load_file(str(model_dir / "model.safetensors"))
+    assert all(t.dtype == torch.float32 for t in stored.values())
+    some = stored["model.layers.0.mlp.down_proj.weight"]
+    assert float((some.to(torch.bfloat16).float() != some).float().mean()) > 0.9
+    requests = _requests(name)
+    plain = PlainQwen2(model_dir)
+    ref = {rid: plain.logits(toks) for rid, toks in requests.items()}
+    live = 4 if mode == "mixed" else 1
+    runner = replay.make_runner(model_dir, "float32", block_size, replay.pages_needed(requests, live, block_size))
+    assert all(p.dtype == torch.float32 for p in runner.model.params.values())
+    got = replay.run_trace(runner, getattr(replay, mode)(requests))
+    worst = _check(got, ref, "float32")
+    print(f"{name} float32 weights {mode}: largest error {worst:.3e}")
+
+
 def test_wide_layers_in_float32(tmp_path):
     """The same wide model in true float32, mixed batches: the 1e-5 bar at layer sizes that the
     tiny models do not reach (a feed-forward 4360 wide, 1024-element rows, head size 128)."""

@@ -173,6 +173,106 @@ def test_shifting_all_positions_changes_nothing(tiny):
     torch.testing.assert_close(run(0), run(77), rtol=1e-9, atol=1e-9)
 
 
+def _layer_setup(tiny, eps=None):
+    """Layer 1 of model B in float64, a random stream h and its rotary tables."""
+    model = plain.PlainQwen2(tiny["B"], dtype=torch.float64)
+    if eps is not None:
+        model.eps = eps
+    T = 7
+    h = torch.randn(T, 192, dtype=torch.float64, generator=torch.Generator().manual_seed(4)) * 0.3
+    cos, sin = plain.rope_tables(torch.arange(T), model.hd, model.theta, torch.float64)
+    return model, h, cos, sin
+
+
+def _without(model, *names):
+    """The same model with the named matrices of layer 1 zeroed."""
+    import copy
+
+    other = copy.copy(model)
+    other.w = dict(model.w)
+    for name in names:
+        key = f"model.layers.1.{name}.weight"
+        other.w[key] = torch.zeros_like(model.w[key])
+    return other
+
+
+def test_a_layer_with_both_output_matrices_zeroed_is_the_identity(tiny):
+    """clockwork/engine/model.py:147-154: out = h + attn(...) + mlp(...). Both branches end in a
+    matrix without bias, so zeroing o_proj and down_proj must leave the stream untouched; a norm
+    applied to the stream itself (post-norm: h = norm(h + branch)) would not."""
+    model, h, cos, sin = _layer_setup(tiny)
+    still = _without(model, "self_attn.o_proj", "mlp.down_proj")
+    assert torch.equal(still.layer(1, h, cos, sin), h)
+
+
+def test_each_branch_reads_the_normed_stream_and_adds_to_the_raw_one(tiny):
+    """Pre-norm wiring: a branch sees norm(stream), which does not change when the stream is
+    scaled (eps aside: it is set to nothing here), and its output is added to the unscaled
+    stream. With the other branch switched off, layer(c h) - c h == layer(h) - h for each of the
+    two; a branch fed the raw stream, or a norm after the sum, breaks this."""
+    model, h, cos, sin = _layer_setup(tiny, eps=1e-300)
+    for off in ("mlp.down_proj", "self_attn.o_proj"):
+        one = _without(model, off)
+        branch = one.layer(1, h, cos, sin) - h
+        assert float(branch.abs().max()) > 1e-3  # the branch that is left does something
+        for c in (0.25, 9.0):
+            torch.testing.assert_close(one.layer(1, c * h, cos, sin) - c * h, branch, rtol=1e-9, atol=1e-12)
+
+
+def test_the_feed_forward_reads_the_stream_after_attention_was_added(tiny):
+    """model.py:150-154: the second residual is h + attn, and the second norm reads it. Putting
+    the layer together from its two branches, each measured alone, must give the layer; a
+    feed-forward that read the layer's input, or the attention output alone, would not."""
+    model, h, cos, sin = _layer_setup(tiny)
+    a = _without(model, "mlp.down_proj").layer(1, h, cos, sin) - h          # attention branch
+    only_ffn = _without(model, "self_attn.o_proj")
+    m = only_ffn.layer(1, h + a, cos, sin) - (h + a)                        # feed-forward on h + a
+    whole = model.layer(1, h, cos, sin)
+    torch.testing.assert_close(whole, h + a + m, rtol=1e-12, atol=1e-12)
+    m_wrong = only_ffn.layer(1, h, cos, sin) - h                            # feed-forward on h
+    assert not torch.allclose(whole, h + a + m_wrong, atol=1e-5)
+
+
+def test_each_norm_weight_feeds_its_own_branch(tiny):
+    """input_layernorm scales what attention reads, post_attention_layernorm what the
+    feed-forward reads (model.py:148, 152): with one branch off, the other norm's weight has no
+    effect and the branch's own norm weight does; swapped weights change the layer."""
+    model, h, cos, sin = _layer_setup(tiny)
+
+    def with_norms(m, first, second):
+        import copy
+
+        other = copy.copy(m)
+        other.w = dict(m.w)
+        other.w["model.layers.1.input_layernorm.weight"] = first
+        other.w["model.layers.1.post_attention_layernorm.weight"] = second
+        return other
+
+    w1 = model.w["model.layers.1.input_layernorm.weight"]
+    w2 = model.w["model.layers.1.post_attention_layernorm.weight"]
+    assert not torch.allclose(w1, w2)
+    attn_only = _without(model, "mlp.down_proj")
+    base = attn_only.layer(1, h, cos, sin)
+    assert torch.equal(with_norms(attn_only, w1, 3 * w2).layer(1, h, cos, sin), base)
+    assert not torch.allclose(with_norms(attn_only, 3 * w1, w2).layer(1, h, cos, sin), base, atol=1e-4)
+    ffn_only = _without(model, "self_attn.o_proj")
+    base = ffn_only.layer(1, h, cos, sin)
+    assert torch.equal(with_norms(ffn_only, 3 * w1, w2).layer(1, h, cos, sin), base)
+    assert not torch.allclose(with_norms(ffn_only, w1, 3 * w2).layer(1, h, cos, sin), base, atol=1e-4)
+    assert not torch.allclose(with_norms(model, w2, w1).layer(1, h, cos, sin), model.layer(1, h, cos, sin), atol=1e-5)
+
+
+def test_final_norm_comes_before_the_head_and_after_the_last_layer(tiny):
+    """model.py:204, 228-233: logits = head(norm(h_L)). Scaling model.norm's weight scales every
+    logit by the same factor (the head has no bias); a head applied to the raw stream would not
+    notice, a norm per layer output would compound."""
+    model = plain.PlainQwen2(tiny["B"], dtype=torch.float64)
+    toks = [5, 900, 31, 7]
+    before = model.logits(toks)
+    model.w["model.norm.weight"] = 2.5 * model.w["model.norm.weight"]
+    torch.testing.assert_close(model.logits(toks), 2.5 * before, rtol=1e-12, atol=1e-12)
+
+
 def test_tied_head_is_the_embedding(tiny):
     model = plain.PlainQwen2(tiny["A"])
     assert model.w["lm_head.weight"] is model.w["model.embed_tokens.weight"]
