@@ -290,75 +290,82 @@ def test_wide_layers_take_the_streaming_and_fused_paths(tmp_path, mode):
     assert not runner.manager.live_requests()
 
 
-def test_a_layer_of_the_benchmark_model_in_both_precisions(tmp_path):
-    """One layer with exactly the sizes of the benchmark's model, the full vocabulary of 151,936
-    and the tied head, mixed batches: float32 at the 1e-5 bar (25 million logits), bfloat16 within
-    the rounding of its 8-bit mantissas."""
+MODES = ["whole", "prefill_then_decode", "portions", "mixed"]
+
+
+def _benchmark_shape(tmp_path_factory, layers: int):
+    """A folder with ``layers`` layers of exactly the benchmark's model (random weights, the full
+    vocabulary of 151,936, the tied head), three requests and their logits from the plain
+    implementation in float64. Sums of 1,536 and 8,960 float32 products carry rounding of about
+    1e-5 themselves, in the engine and in a float32 plain implementation alike (two such
+    implementations differ by up to 1.3e-5 after one layer), so the plain side runs in float64:
+    what is measured is the engine's own rounding."""
     from clockwork_amd.weights.random_init import write_random_model
     from tests.configs import LAYER_1P5B
 
-    model_dir = write_random_model(tmp_path / "layer1p5b", LAYER_1P5B, 2)
+    config = dict(LAYER_1P5B, num_hidden_layers=layers)
+    model_dir = write_random_model(tmp_path_factory.mktemp(f"benchmark_shape_{layers}") / "model", config, 2)
     gen = torch.Generator().manual_seed(11)
-    requests = {f"w{i}": torch.randint(0, LAYER_1P5B["vocab_size"], (n,), generator=gen).tolist()
+    requests = {f"w{i}": torch.randint(0, config["vocab_size"], (n,), generator=gen).tolist()
                 for i, n in enumerate([40, 70, 55])}
-    # Sums of 1,536 and 8,960 float32 products carry rounding of about 1e-5 themselves, in the
-    # engine and in a float32 plain implementation alike (they differ by up to 1.3e-5 here), so
-    # the plain side runs in float64: what is measured is the engine's own rounding.
     plain = PlainQwen2(model_dir, dtype=torch.float64)
     want = {rid: plain.logits(toks).float() for rid, toks in requests.items()}
-    scale = torch.cat([w.flatten() for w in want.values()]).square().mean().sqrt().item()
-    pages = replay.pages_needed(requests, 3, 16)
-    got = replay.run_trace(replay.make_runner(model_dir, "float32", 16, pages), replay.mixed(requests))
-    worst = replay.compare(got, want, **TOL["float32"])
-    print(f"benchmark layer float32 mixed: largest error {worst:.3e}")
-    got = replay.run_trace(replay.make_runner(model_dir, "bfloat16", 16, pages), replay.mixed(requests))
-    errors = torch.stack([row - want[rid][pos] for (rid, pos), row in sorted(got.items())])
-    assert not torch.isnan(errors).any()
-    rms, worst = errors.square().mean().sqrt().item(), errors.abs().max().item()
-    print(f"benchmark layer bfloat16 mixed: logits' scale {scale:.3f}, rms error {rms:.3e}, largest {worst:.3e}")
-    # as for the layers of the larger models below: relative to the logits' own scale
-    assert rms < 2e-2 * scale and worst < 1e-1 * scale
+    return model_dir, requests, want
 
 
-def test_the_whole_benchmark_model_against_the_plain_implementation(tmp_path):
-    """All 28 layers of the benchmark's model (random weights: a 3 GB folder, 1.5 billion
-    parameters), three requests in mixed batches, against the plain implementation on the CPU.
-    float32: the same arg-max at every position and errors of float32 rounding carried through 28
-    layers (measured: rms 2.5e-6, largest 1.5e-5 among 25 million logits). bfloat16: errors of
-    about 2 % of the logits' scale, and wherever the arg-max differs the plain logits of the two
-    tokens lie closer than that (random weights give many near-ties)."""
-    from clockwork_amd.weights.random_init import write_random_model
-    from tests.configs import LAYER_1P5B
+@pytest.fixture(scope="module")
+def benchmark_layer(tmp_path_factory):
+    return _benchmark_shape(tmp_path_factory, 1)
 
-    config = dict(LAYER_1P5B, num_hidden_layers=28)
-    model_dir = write_random_model(tmp_path / "qwen2.5-1.5b-shape", config, 2)
-    gen = torch.Generator().manual_seed(11)
-    requests = {f"w{i}": torch.randint(0, config["vocab_size"], (n,), generator=gen).tolist() for i, n in enumerate([40, 70, 55])}
-    plain = PlainQwen2(model_dir)
-    want = {rid: plain.logits(toks) for rid, toks in requests.items()}
-    del plain
-    scale = torch.cat([w.flatten() for w in want.values()]).square().mean().sqrt().item()
-    pages = replay.pages_needed(requests, 3, 16)
-    for dtype in ("float32", "bfloat16"):
-        runner = replay.make_runner(model_dir, dtype, 16, pages)
-        got = replay.run_trace(runner, replay.mixed(requests))
-        del runner
-        assert len(got) == 165
-        errors = torch.stack([row - want[rid][pos] for (rid, pos), row in sorted(got.items())])
-        assert not torch.isnan(errors).any()
-        rms, worst = errors.square().mean().sqrt().item(), errors.abs().max().item()
-        gaps = []
-        for (rid, pos), row in got.items():
-            ref = want[rid][pos]
-            a, b = int(row.argmax()), int(ref.argmax())
-            if a != b:
-                gaps.append(float(ref[b] - ref[a]))
-        print(f"whole model {dtype}: scale {scale:.3f}, rms {rms:.3e}, largest {worst:.3e}, arg-max differs at {len(gaps)} of 165")
-        if dtype == "float32":
-            assert not gaps and rms < 5e-6 and worst < 5e-5
-        else:
-            assert rms < 4e-2 * scale and worst < 2.5e-1 * scale
-            assert all(g < 1e-1 * scale for g in gaps) and len(gaps) < 30
+
+@pytest.fixture(scope="module")
+def benchmark_model(tmp_path_factory):
+    return _benchmark_shape(tmp_path_factory, 28)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", MODES)
+def test_a_layer_of_the_benchmark_model(benchmark_layer, mode, dtype):
+    """One layer with exactly the sizes of the benchmark's model, in every way of cutting the
+    work: float32 at the 1e-5 bar (25 million logits), bfloat16 within its bound."""
+    model_dir, requests, want = benchmark_layer
+    live = 3 if mode == "mixed" else 1
+    runner = replay.make_runner(model_dir, dtype, 16, replay.pages_needed(requests, live, 16))
+    got = replay.run_trace(runner, getattr(replay, mode)(requests))
+    assert len(got) == 165
+    worst = _check(got, want, dtype)
+    print(f"benchmark layer {dtype} {mode}: largest error {worst:.3e}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", MODES)
+def test_the_whole_benchmark_model(benchmark_model, mode, dtype):
+    """All 28 layers of the benchmark's model (a 3 GB folder, 1.5 billion random parameters), in
+    every way of cutting the work, against the plain implementation in float64 on the CPU.
+    float32: the 1e-5 bar and the same arg-max at every position. bfloat16: the rounding of 28
+    layers adds up to about 2% of the logits' scale (root mean square; bound 4%, the largest of 25
+    million within 25%), and wherever the arg-max differs the plain logits of the two tokens lie
+    closer than a tenth of the scale (random weights give many near-ties)."""
+    model_dir, requests, want = benchmark_model
+    live = 3 if mode == "mixed" else 1
+    runner = replay.make_runner(model_dir, dtype, 16, replay.pages_needed(requests, live, 16))
+    got = replay.run_trace(runner, getattr(replay, mode)(requests))
+    del runner
+    assert len(got) == 165
+    gaps = []
+    for (rid, pos), row in got.items():
+        ref = want[rid][pos]
+        a, b = int(row.argmax()), int(ref.argmax())
+        if a != b:
+            gaps.append(float(ref[b] - ref[a]))
+    if dtype == "float32":
+        worst = replay.compare(got, want, **TOL["float32"])
+        assert not gaps
+        print(f"whole model float32 {mode}: largest error {worst:.3e}")
+    else:
+        scale, rms, worst = replay.compare_to_scale(got, want, rms_bound=4e-2, worst_bound=2.5e-1)
+        print(f"whole model bfloat16 {mode}: scale {scale:.3f}, rms {rms:.3e}, largest {worst:.3e}, arg-max differs at {len(gaps)} of 165")
+        assert all(g < 1e-1 * scale for g in gaps) and len(gaps) < 30
 
 
 @pytest.mark.parametrize("which", ["LAYER_7B", "LAYER_32B"])
