@@ -20,6 +20,7 @@ from clockwork_amd import ops
 from clockwork_amd.cache.manager import CacheManager, cache_needs_of, plan_groups
 from clockwork_amd.cache.pools import CachePools, pages_that_fit
 from clockwork_amd.config.engine import EngineConfig
+from clockwork_amd.engine.graph_nodes import node_kinds, only_kernels
 from clockwork_amd.engine.batch import (
     StaticDecodeBatch,
     StaticPortionBatch,
@@ -113,6 +114,7 @@ class ModelRunner:
         # decode-only steps replay captured HIP graphs: one per (padded batch size, context bucket)
         self.use_graphs = use_graphs and self.model.graph_safe()
         self._graphs: dict = {}
+        self.graph_nodes: dict = {}  # per captured shape: how many nodes of each kind its graph held
         self._graph_pool = None
         self._table_width = -(-cfg.model.max_model_len // cfg.cache.block_size)
 
@@ -206,6 +208,8 @@ class ModelRunner:
         if state is None:
             self._graphs[key] = "seen"
             return NotImplemented
+        if state == "eager":
+            return NotImplemented
         for e in entries:
             if not 0 <= int(e.tokens[0]) < self.spec.vocab_size:
                 raise ValueError(f"request {e.seq_id}: token id {e.tokens[0]} outside the vocabulary")
@@ -216,13 +220,9 @@ class ModelRunner:
                                       self.model.attention_geometries(), self.num_compute_units)
             batch.fill(entries, self.manager)
             torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with capturing(graph, self._graph_pool):
-                out = self.model.forward(batch.ctx, self.caches)
-            if self._graph_pool is None:
-                self._graph_pool = graph.pool()
-            state = self._graphs[key] = (batch, graph, out)
-            self._drop_old_graphs()
+            state = self._capture(key, batch)
+            if state is None:
+                return NotImplemented
         self._graphs[key] = self._graphs.pop(key)  # most recently used last
         batch, graph, out = state
         batch.fill(entries, self.manager)
@@ -254,25 +254,45 @@ class ModelRunner:
         if state is None:
             self._graphs[key] = "seen"
             return NotImplemented
+        if state == "eager":
+            return NotImplemented
         if state == "seen":
             batch = StaticPortionBatch(size, key[2], key[3], self._table_width, self.manager, self.device,
                                        self.model.attention_geometries(), self.num_compute_units,
                                        self.spec.vocab_size)
             batch.fill(entry, self.manager)
             torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with capturing(graph, self._graph_pool):
-                out = self.model.forward(batch.ctx, self.caches)
-            if self._graph_pool is None:
-                self._graph_pool = graph.pool()
-            state = self._graphs[key] = (batch, graph, out)
-            self._drop_old_graphs()
+            state = self._capture(key, batch)
+            if state is None:
+                return NotImplemented
         self._graphs[key] = self._graphs.pop(key)  # most recently used last
         batch, graph, out = state
         batch.fill(entry, self.manager)
         graph.replay()
         self.manager.release_behind_window(entry.seq_id, entry.start + n)
         return out if want else None
+
+    def _capture(self, key, batch):
+        """Capture the model's step on ``batch`` (filled, its copy done) as the graph of ``key``.
+        A graph that holds anything but kernel nodes is not kept (a library product may record a
+        memset of its workspace, and such nodes have replayed wrongly): its shape is marked to
+        run eagerly from now on and None is returned."""
+        graph = torch.cuda.CUDAGraph(keep_graph=True)
+        with capturing(graph, self._graph_pool):
+            out = self.model.forward(batch.ctx, self.caches)
+        kinds = node_kinds(graph)
+        self.graph_nodes[key] = dict(kinds)
+        if not only_kernels(kinds):
+            torch.cuda.synchronize()
+            graph.reset()
+            self._graphs[key] = "eager"
+            return None
+        graph.instantiate()
+        if self._graph_pool is None:
+            self._graph_pool = graph.pool()
+        state = self._graphs[key] = (batch, graph, out)
+        self._drop_old_graphs()
+        return state
 
     def _drop_old_graphs(self) -> None:
         captured = [k for k, v in self._graphs.items() if isinstance(v, tuple)]
@@ -305,7 +325,8 @@ class ModelRunner:
     @torch.no_grad()
     def step_prepared(self, handle, tokens) -> torch.Tensor:
         """Run the step that ``prepare_decode`` got ready, now that its tokens are known; every
-        entry's logits are returned, float32 [entries, vocab]. ``tokens``: a sequence of ids, or
+        entry's logits are returned, float32 [entries, vocab], a view of the graph's output buffer
+        that the next step of this shape overwrites. ``tokens``: a sequence of ids, or
         an int32 device tensor (what the sampling kernels of the step before wrote, possibly
         still being computed: the tokens then never visit the host)."""
         key, entries = handle
@@ -333,7 +354,9 @@ class ModelRunner:
     @torch.no_grad()
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Run the entries as one batch; float32 logits [wanted, vocab] in the order of the
-        entries and of each entry's ``want`` (None when nothing is wanted)."""
+        entries and of each entry's ``want`` (None when nothing is wanted). The tensor may be a
+        view of a replayed graph's own output buffer: it holds this step's logits until the next
+        step runs, so a caller that keeps logits across steps copies them."""
         if not entries:
             return None
         if (self.use_graphs and not self.manager.state_groups and len(entries) <= GRAPH_BATCH_SIZES[-1]

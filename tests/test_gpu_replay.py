@@ -615,8 +615,8 @@ def test_short_prompts_replay_padded_graphs(model_dirs, dtype):
 @pytest.mark.parametrize("tuned", [False, True])
 def test_wide_decode_batches_of_a_large_layer_replay_as_eager(tmp_path, tuned):
     """40 requests decoding together through one layer of the 7B shape: at this width some products
-    are library products inside the captured graph (also a kernel the library's tuning picked,
-    which may clear a workspace before it runs). Every replay, with eager steps of another batch
+    are library products inside the captured graph (also a kernel the library's tuning picked;
+    the runner keeps a graph only if it holds kernel nodes alone). Every replay, with eager steps of another batch
     size and synchronisations in between, must equal the same step of a runner without graphs."""
     from clockwork_amd.weights.random_init import write_random_model
     from tests import configs
@@ -644,6 +644,7 @@ def test_wide_decode_batches_of_a_large_layer_replay_as_eager(tmp_path, tuned):
     got_e = replay.run_trace(eager, [dict(s) for s in fixed])
     captured = [k for k, v in with_graphs._graphs.items() if isinstance(v, tuple)]
     assert {size for size, _ in captured} == {48, 24}
+    assert all(set(with_graphs.graph_nodes[k]) == {"kernel"} for k in captured)
     assert got_g.keys() == got_e.keys() and len(got_g) > 200
     scale = torch.stack(list(got_e.values())).square().mean().sqrt().item()
     for key in got_e:
@@ -656,6 +657,86 @@ def test_wide_decode_batches_of_a_large_layer_replay_as_eager(tmp_path, tuned):
         diff = (got_g[key] - got_e[key]).abs()
         bound = 2e-2 * scale + 2.0 ** -7 * got_e[key].abs()
         assert bool((diff <= bound).all()), f"graph replay differs from the eager step at {key}: {diff.max().item()}"
+
+
+@pytest.mark.parametrize("tuned", [False, True])
+def test_captured_graphs_hold_kernel_nodes_only(tmp_path, tuned):
+    """One layer of the 7B shape: a decode batch of 96 rows and a portion of 2048 tokens, the two
+    kinds of step whose graphs capture library products (also the kernels the library's tuning
+    picks). The runner walks every graph it captures and keeps it only if all its nodes are kernel
+    launches; here both graphs must be kept, i.e. the library recorded no memset or copy node."""
+    from clockwork_amd.config.engine import EngineConfig
+    from clockwork_amd.engine.batch import StepEntry
+    from clockwork_amd.engine.model_runner import ModelRunner
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests import configs
+
+    config = configs.LAYER_7B
+    model_dir = write_random_model(tmp_path / "layer7b", config, 3)
+    cfg = EngineConfig.defaults(str(model_dir), dtype="bfloat16", block_size=16, num_blocks=96 + 3 * 128 + 8,
+                                enable_prefix_cache=False, watermark=0.0, max_model_len=8192,
+                                max_num_batched_tokens=2048, max_num_seqs=128)
+    runner = ModelRunner(cfg)
+    if tuned:
+        assert runner.tune_products([2048, 96]) == [2048, 96]
+    gen = torch.Generator().manual_seed(5)
+    long_prompt = torch.randint(0, config["vocab_size"], (3 * 2048,), generator=gen).tolist()
+    runner.reserve("long", 0, 3 * 2048)
+    for i in range(3):  # seen, captured, replayed
+        runner.step([StepEntry("long", 2048 * i, long_prompt[2048 * i : 2048 * (i + 1)], [2047])])
+    for r in range(96):
+        runner.reserve(f"r{r}", 0, 3)
+    for i in range(3):
+        runner.step([StepEntry(f"r{r}", i, [int(long_prompt[r + i])], [0]) for r in range(96)])
+    torch.cuda.synchronize()
+    kept = {k: v for k, v in runner._graphs.items() if isinstance(v, tuple)}
+    print({k: runner.graph_nodes[k] for k in runner.graph_nodes})
+    assert set(kept) == set(runner.graph_nodes)
+    assert (96, 512) in kept and any(k[0] == "portion" and k[1] == 2048 for k in kept)
+    for key, kinds in runner.graph_nodes.items():
+        assert set(kinds) == {"kernel"} and kinds["kernel"] > 10, f"graph {key} holds {kinds}"
+
+
+def test_a_graph_with_a_memset_node_is_not_kept(model_dirs):
+    """A part whose step clears a buffer with a memset (torch's zero_ of a large tensor is one):
+    the captured graph holds a node that is no kernel, so the runner drops it and runs that
+    batch shape eagerly from then on, with the same logits."""
+    from clockwork_amd.engine.graph_nodes import node_kinds
+
+    name = "B"
+    cfg, _, block_size = TINY_CONFIGS[name]
+    # what the walk reports for a capture with a memset in it
+    scratch = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+    import ctypes
+
+    from clockwork_amd.engine import graph_nodes
+
+    hip = graph_nodes._runtime()
+    hip.hipMemsetAsync.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p]
+    graph = torch.cuda.CUDAGraph(keep_graph=True)
+    with torch.cuda.graph(graph):
+        scratch.add_(1)
+        assert hip.hipMemsetAsync(scratch.data_ptr(), 0, scratch.numel(), torch.cuda.current_stream().cuda_stream) == 0
+    kinds = node_kinds(graph)
+    assert kinds["kernel"] >= 1 and kinds["memset"] == 1
+    graph.reset()   # never replayed
+
+    toks = torch.randint(0, cfg["vocab_size"], (40,), generator=torch.Generator().manual_seed(2)).tolist()
+    steps = [{"entries": [{"id": "x", "tokens": [t], "want": [0]}], "end": []} for t in toks]
+    clean = replay.run_trace(replay.make_runner(model_dirs[name], "float32", block_size, 8), [dict(s) for s in steps])
+    runner = replay.make_runner(model_dirs[name], "float32", block_size, 8)
+    norm = runner.model.final_norm
+    real = norm.forward
+
+    def with_memset(resid, delta, rows=None):
+        hip.hipMemsetAsync(scratch.data_ptr(), 0, scratch.numel(), torch.cuda.current_stream().cuda_stream)
+        return real(resid, delta, rows)
+
+    norm.forward = with_memset
+    got = replay.run_trace(runner, [dict(s) for s in steps])
+    assert runner._graphs[(1, 512)] == "eager" and runner.graph_nodes[(1, 512)].get("memset") == 1
+    for key in clean:
+        torch.testing.assert_close(got[key], clean[key], rtol=2e-6, atol=2e-6)
 
 
 def test_negative_control_a_small_weight_change_breaks_the_match(model_dirs, tmp_path):
