@@ -101,6 +101,9 @@ class CacheManager:
         self.watermark_blocks = int(watermark * num_blocks)
         self.max_num_seqs = max_num_seqs
         self._free_slots = list(range(max_num_seqs - 1, -1, -1))
+        # what a row that holds no request carries as its state slot: the pools' spare slot when
+        # the model keeps state, else -1
+        self.idle_state_slot = max_num_seqs if self.state_groups else -1
         self._requests: dict[str, RequestPages] = {}
         self._epochs = 0
 

@@ -5,7 +5,9 @@ kv_heads, head_dim] in the engine's dtype: an entry's keys (or values) are the
 reference's paged layout [num_blocks, block_size, kv_heads, head_dim]
 (clockwork/kvcache/kv_cache.py:24-30), one page id addresses the same page in
 every entry of the group, and a copy-on-write copies all of them with one kernel.
-Per state group one tensor [entries, max_num_seqs, *shape].
+Per state group one tensor [entries, max_num_seqs + 1, *shape]: a slot per live request and a
+spare one at the end that belongs to nobody (rows of a fixed-shape batch that hold no request
+point there, so a part may read and write "its" slot for every row without asking).
 """
 
 from __future__ import annotations
@@ -66,8 +68,11 @@ class CachePools:
                 self.kv.append(pool)
             else:
                 need = group.need
-                shape = (len(group.entries), max_num_seqs, *need.shape)
+                shape = (len(group.entries), max_num_seqs + 1, *need.shape)
                 pool = torch.zeros(shape, dtype=getattr(torch, need.dtype), device=device)
+                if (pool[0, 0].numel() * pool.element_size()) % 4:
+                    raise ValueError(f"a state of shape {tuple(need.shape)} {need.dtype} is not a whole number of "
+                                     "32-bit words: the kernel that clears a fresh request's state takes words")
                 for row, entry in enumerate(group.entries):
                     self._state_index[entry] = (len(self.state), row)
                 self.state.append(pool)
@@ -113,6 +118,9 @@ class CachePools:
         for pool in self.state:
             pool[:, dst_slot].copy_(pool[:, src_slot])
 
-    def zero_state(self, slot: int) -> None:
+    def zero_fresh_state(self, state_slots: torch.Tensor, starts: torch.Tensor, n: int) -> None:
+        """Clear the state of the step's requests that begin at position 0 (device int32 arrays of
+        the step: each request's slot and first position). One kernel per state group; part of
+        every step of a model with state, captured or not."""
         for pool in self.state:
-            pool[:, slot].zero_()
+            ops.zero_state_rows(pool, state_slots, starts, n)

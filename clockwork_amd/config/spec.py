@@ -70,16 +70,32 @@ class LayerSpec:
     """One block: which parts it is made of and how they are wired.
 
     ``arrangement`` names an entry of the arrangement registry ("prenorm":
-    x + mixer(norm(x)), then x + ffn(norm(x))). ``mixer``, ``feed_forward`` and
-    the norms are specs of registered part kinds; different layers of one model
-    may hold different kinds.
+    x + mixer(norm(x)), then x + ffn(norm(x))). The parts are specs of registered
+    part kinds under the names the arrangement expects: the four that most blocks
+    have can be given by keyword (any of them may be left out), others in
+    ``extra`` as (name, spec) pairs; the arrangement's factory receives them all
+    as keyword arguments. Different layers of one model may hold different kinds.
+    The part named ``mixer`` is the one that owns the block's cache.
     """
 
     arrangement: str
-    mixer: Any
-    feed_forward: Any
-    mixer_norm: Any
-    ffn_norm: Any
+    mixer: Any = None
+    feed_forward: Any = None
+    mixer_norm: Any = None
+    ffn_norm: Any = None
+    extra: tuple = ()
+
+    def named_parts(self) -> dict:
+        """{name: spec} of every part of the block, in a fixed order."""
+        parts = {}
+        for name in ("mixer", "feed_forward", "mixer_norm", "ffn_norm"):
+            if getattr(self, name) is not None:
+                parts[name] = getattr(self, name)
+        for name, spec in self.extra:
+            if name in parts:
+                raise ValueError(f"a block has two parts named {name!r}")
+            parts[name] = spec
+        return parts
 
 
 @dataclass(frozen=True)
@@ -105,6 +121,11 @@ class ModelSpec:
     final_norm: Any
     tie_embeddings: bool = False
     eos_token_ids: tuple[int, ...] = ()
+    # specs of the part that turns token ids into the residual stream and of the part that turns
+    # the final norm's rows into logits; None: a plain table lookup and a plain product with a
+    # [vocab, hidden] matrix (the embedding table itself when ``tie_embeddings`` is set)
+    embedding: Any = None
+    head: Any = None
     # free-form facts for reporting (bench config lines and the like), never read by parts
     info: dict = field(default_factory=dict)
 

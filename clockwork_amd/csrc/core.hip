@@ -432,6 +432,32 @@ CW_EXPORT int cw_copy_pages(void* pool, int planes, int64_t num_blocks, int64_t 
   return cw_launch_status();
 }
 
+// ---------------------------------------------------------------- fresh state slots
+// The state pool of a group is [entries, slots, row_bytes]. A request whose first token runs in
+// this step (starts[r] == 0) begins from an empty state: its slot's row is cleared in every
+// entry, by a kernel (no memset: the launch is part of steps that are captured as graphs).
+// slots[r] < 0 or >= num_slots: the row belongs to no request, nothing is cleared.
+__global__ void zero_state_rows_kernel(uint32_t* __restrict__ pool, int64_t entry_words, int64_t row_words,
+                                       int num_slots, const int* __restrict__ slots,
+                                       const int* __restrict__ starts) {
+  const int r = blockIdx.x, entry = blockIdx.y;
+  const int slot = slots[r];
+  if (starts[r] != 0 || slot < 0 || slot >= num_slots) return;
+  uint32_t* row = pool + entry * entry_words + (int64_t)slot * row_words;
+  for (int64_t i = threadIdx.x; i < row_words; i += blockDim.x) row[i] = 0u;
+}
+
+CW_EXPORT int cw_zero_state_rows(void* pool, int entries, int num_slots, int64_t row_bytes, const int* slots,
+                                 const int* starts, int n, hipStream_t stream) {
+  if (entries <= 0 || num_slots <= 0 || row_bytes <= 0 || (row_bytes & 3) || n < 0 || !pool || !slots || !starts)
+    return CW_ERR_ARG;
+  if (n == 0) return CW_OK;
+  if (entries > 65535) return CW_ERR_SIZE;
+  hipLaunchKernelGGL(zero_state_rows_kernel, dim3(n, entries), dim3(256), 0, stream, (uint32_t*)pool,
+                     (int64_t)num_slots * (row_bytes / 4), row_bytes / 4, num_slots, slots, starts);
+  return cw_launch_status();
+}
+
 // ---------------------------------------------------------------- casts
 // out[i] = float(in[i]) for bfloat16 input (logits of a bfloat16 product to float32).
 __global__ void bf16_to_f32_kernel(const bf16_t* __restrict__ in, float* __restrict__ out, int64_t n) {

@@ -25,30 +25,6 @@ class StepEntry:
     want: Sequence[int] = ()
 
 
-@dataclass
-class AttentionPlan:
-    """Work items of the attention kernels for one head geometry (see csrc/attention.hip).
-
-    Requests with one token go to the 16-row kernel, cut over their keys into
-    ``single_splits`` parts; longer portions are cut into tiles of the 64-row kernel."""
-
-    wide_items: Optional[torch.Tensor] = None
-    n_wide: int = 0
-    gh_wide: int = 1
-    mfma_items: Optional[torch.Tensor] = None   # the same portions cut for the bfloat16 matrix-core kernel
-    n_mfma: int = 0
-    mfma_row_blocks: int = 4   # row blocks of that kernel's workgroups: 2 when 4 would leave compute units idle
-    single_items: Optional[torch.Tensor] = None
-    n_single: int = 0
-    gh_single: int = 1
-    chunks_single: int = 1
-    single_splits: int = 1
-    decode_splits: int = 1   # splits of the bfloat16 decode kernel (finer: it walks 16-key tiles)
-    decode_split_keys: int = 0    # keys of each of those splits, at fixed places (a multiple of 32)
-    decode_max_ctx: int = 0       # the longest context the fixed places were planned for
-    single_identity: bool = False  # a batch of single tokens only: item i is request i, token row i
-
-
 class _Packer:
     def __init__(self) -> None:
         self.parts: list[np.ndarray] = []
@@ -100,91 +76,19 @@ class StepContext:
         self.h_starts: list[int] = []
         self.h_state_slots: list[int] = []
         self.seq_ids: list[str] = []
-        self._plans: dict = {}
+        self.plans: dict = {}     # what parts have planned for this step, under keys of their own
         self._pinned: list = []   # host buffers of the plans' uploads, alive as long as the step
         self.num_compute_units = 256
 
-    def attention_plan(self, nh: int, nkv: int, narrow_ok: bool = False) -> AttentionPlan:
-        """``narrow_ok``: the matrix-core kernel for portions also comes with two row blocks a
-        workgroup (see ``ops.prefill_row_blocks_ok``)."""
-        # a batch of single tokens has no portions: one plan, whatever the kernel for portions offers
-        narrow_ok = bool(narrow_ok) and any(q > 1 for q in self.h_q_lens)
-        key = (nh, nkv, narrow_ok)
-        plan = self._plans.get(key)
-        if plan is None:
-            plan = self._plans[key] = self._make_plan(nh, nkv, narrow_ok)
-        return plan
-
-    def _make_plan(self, nh: int, nkv: int, narrow_ok: bool = False) -> AttentionPlan:
-        group = nh // nkv
-        gh_wide = min(group, 64)
-        tokens_per_tile = 64 // gh_wide
-        gh_single = min(group, 16)
-        wide: list = []   # one array of items per portion
-        mfma: list = []
-        # Workgroups of four row blocks share each key among the most rows, but a launch has to
-        # fill the compute units, and the workgroup with the longest key range decides its time:
-        # with fewer than 1.5 workgroups a compute unit, halve them. Behind a long cached prefix
-        # every workgroup's key range is long and about the same, and sharing the keys among more
-        # rows wins again (2048 tokens of the 1.5B shape: 46 against 52 us with no prefix, 94
-        # against 96 us behind 2048 tokens, 197 against 182 us behind 6144).
-        tokens_of_four = 4 * (32 // min(group, 32))
-        workgroups = sum(-(-q // tokens_of_four) for q in self.h_q_lens if q > 1) * nkv * -(-group // 32)
-        portion_tokens = sum(q for q in self.h_q_lens if q > 1)
-        keys = sum(q * (c - q / 2.0) for q, c in zip(self.h_q_lens, self.h_ctx_lens) if q > 1)
-        short_ranges = portion_tokens > 0 and keys / portion_tokens < 3072  # portion_has_long_ranges says the same of one portion
-        row_blocks = 2 if narrow_ok and short_ranges and 2 * workgroups < 3 * self.num_compute_units else 4
-        tokens_per_mfma_item = row_blocks * (32 // min(group, 32))
-        single: list[int] = []
-        longest_single = 0
-
-        def items_of(r: int, q_len: int, step: int, longest_first: bool) -> np.ndarray:
-            """(request, first token, tokens, 0) for runs of ``step`` tokens of one portion."""
-            tok0 = np.arange(0, q_len, step, dtype=np.int32)
-            if longest_first:
-                tok0 = tok0[::-1]
-            out = np.zeros((tok0.size, 4), dtype=np.int32)
-            out[:, 0] = r
-            out[:, 1] = tok0
-            out[:, 2] = np.minimum(step, q_len - tok0)
-            return out.reshape(-1)
-
-        for r, q_len in enumerate(self.h_q_lens):
-            if q_len == 1:
-                single += [r, 0, 1, 0]
-                longest_single = max(longest_single, self.h_ctx_lens[r])
-            else:
-                wide.append(items_of(r, q_len, tokens_per_tile, False))
-                # longest key ranges first: the last tokens of a portion have the most work
-                mfma.append(items_of(r, q_len, tokens_per_mfma_item, True))
-        wide = np.concatenate(wide) if wide else np.zeros(0, dtype=np.int32)
-        mfma = np.concatenate(mfma) if mfma else np.zeros(0, dtype=np.int32)
-        plan = AttentionPlan(gh_wide=gh_wide, gh_single=gh_single, mfma_row_blocks=row_blocks)
-        plan.n_wide, plan.n_single, plan.n_mfma = len(wide) // 4, len(single) // 4, len(mfma) // 4
-        plan.chunks_single = -(-group // gh_single)
-        if plan.n_single:
-            groups_running = plan.n_single * nkv * plan.chunks_single
-            by_occupancy = -(-4 * self.num_compute_units // groups_running)
-            by_length = max(1, longest_single // 256)
-            plan.single_splits = max(1, min(by_occupancy, by_length, 64))
-            # decode kernel: a workgroup per (request, kv head, split); a split is at least 128 keys
-            # (one 32-key tile for each of its four waves), and about two workgroups per compute
-            # unit are enough to keep memory busy. More than 64 splits never paid: one request
-            # with 30000 keys takes 16 us with 64 to 128 splits and 19 us with 235.
-            base = plan.n_single * nkv * -(-group // min(group, 16))
-            plan.decode_splits = max(1, min(-(-2 * self.num_compute_units // base), longest_single // 128, 64))
-            # fixed places for the splits: a workgroup then knows its pages before it knows the
-            # request's length, which saves it a trip to memory
-            plan.decode_split_keys = 32 * -(-(-(-longest_single // plan.decode_splits)) // 32)
-            plan.decode_max_ctx = longest_single
-            plan.single_identity = plan.n_single == len(self.h_q_lens)
+    def upload(self, arrays) -> list:
+        """int32 arrays to the device in one copy; returns a device view of each. For a part
+        that plans its kernels' work items for this step (kept in ``plans``)."""
         packer = _Packer()
-        packer.add(wide)
-        packer.add(single)
-        packer.add(mfma)
-        plan.wide_items, plan.single_items, plan.mfma_items = packer.upload(self.device)
+        for a in arrays:
+            packer.add(a)
+        views = packer.upload(self.device)
         self._pinned.append(packer)
-        return plan
+        return views
 
 
 def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int) -> StepContext:
@@ -256,12 +160,12 @@ class StaticDecodeBatch:
 
     ``size`` requests of one token each; every index array lives at a fixed device address and
     is refreshed by one host-to-device copy per step. Rows past the live requests are padding:
-    token 0 at position 0, no cache slot (-1) and no pages, so they write nothing and read
-    nothing. ``key_capacity`` (the longest context the graph is planned for) only fixes how
+    token 0 at position 0, no cache slot (-1), no pages and the state pools' spare slot, so they
+    write nothing that anyone reads and read nothing. ``key_capacity`` (the longest context the graph is planned for) only fixes how
     finely the attention kernel splits its keys.
     """
 
-    def __init__(self, size: int, key_capacity: int, table_width: int, manager, device, geometries,
+    def __init__(self, size: int, key_capacity: int, table_width: int, manager, device, prepare,
                  num_compute_units: int) -> None:
         self.size = size
         self.table_width = table_width
@@ -304,11 +208,10 @@ class StaticDecodeBatch:
         ctx.h_q_lens = [1] * size
         ctx.h_ctx_lens = [key_capacity] * size
         ctx.h_starts = [0] * size
-        ctx.h_state_slots = [-1] * size
+        ctx.h_state_slots = [manager.idle_state_slot] * size
         ctx.seq_ids = [""] * size
         ctx.num_compute_units = num_compute_units
-        for nh, nkv in geometries:  # work items are the same every step: made once, outside the graph
-            ctx.attention_plan(nh, nkv)
+        prepare(ctx)  # the parts' work items are the same every step: made once, outside the graph
         self.ctx = ctx
 
     def fill(self, entries: Sequence[StepEntry], manager, upload: bool = True) -> None:
@@ -336,7 +239,7 @@ class StaticDecodeBatch:
         pos[n:] = 0
         ctx_lens[n:] = 1
         starts[n:] = 0
-        state[n:] = -1
+        state[n:] = manager.idle_state_slot
         tok[:n] = [e.tokens[0] for e in entries]
         st = [e.start for e in entries]
         pos[:n] = st
@@ -396,13 +299,14 @@ class StaticPortionBatch:
     refreshed by one host-to-device copy per step, and the attention work items are made once, for
     ``num_tokens`` tokens. A shorter portion leaves rows at the end that belong to no request:
     token 0, no cache slot, past the request's tokens as ``cu_q`` counts them, so no attention
-    item computes them and nothing reads what the other kernels make of them. ``long_ranges``
-    only chooses the attention kernel's workgroup shape, as the step's plan would (behind a long
-    cached prefix or not); ``wanted``: the logits of the portion's last token are made (else none).
+    item computes them and nothing reads what the other kernels make of them. ``typical_start``
+    is the position of a portion of the class of steps this batch serves (the parts choose their
+    kernels' shapes by it, as they would for that step; any step's results are right under any
+    such choice); ``wanted``: the logits of the portion's last token are made (else none).
     """
 
-    def __init__(self, num_tokens: int, long_ranges: bool, wanted: bool, table_width: int, manager, device,
-                 geometries, num_compute_units: int, vocab_size: int) -> None:
+    def __init__(self, num_tokens: int, typical_start: int, wanted: bool, table_width: int, manager, device,
+                 prepare, num_compute_units: int, vocab_size: int) -> None:
         self.num_tokens = n = num_tokens
         self.vocab_size = vocab_size
         self.table_width = table_width
@@ -444,17 +348,14 @@ class StaticPortionBatch:
         for g in range(n_groups):
             ctx.slots.append(view(f"slots{g}"))
             ctx.block_tables.append(view(f"table{g}").view(1, table_width))
-        # what the attention plan looks at: the portion's length and whether its key ranges are long
-        behind = PORTION_LONG_RANGE if long_ranges else 0
+        # what the parts' plans look at: the portion's length and where it starts
         ctx.h_q_lens = [n]
-        ctx.h_ctx_lens = [behind + n]
-        ctx.h_starts = [behind]
-        ctx.h_state_slots = [-1]
+        ctx.h_ctx_lens = [typical_start + n]
+        ctx.h_starts = [typical_start]
+        ctx.h_state_slots = [manager.idle_state_slot]
         ctx.seq_ids = [""]
         ctx.num_compute_units = num_compute_units
-        for nh, nkv in geometries:  # work items are the same every step: made once, outside the graph
-            for narrow_ok in (False, True):
-                ctx.attention_plan(nh, nkv, narrow_ok=narrow_ok)
+        prepare(ctx)  # the parts' work items are the same every step: made once, outside the graph
         self.ctx = ctx
 
     def fill(self, entry: StepEntry, manager) -> None:
@@ -498,12 +399,3 @@ class StaticPortionBatch:
         self.device_buf.copy_(self.host, non_blocking=True)
         self._sent = torch.cuda.Event()
         self._sent.record()
-
-
-# keys a portion has before it when its key ranges count as long (see StepContext._make_plan)
-PORTION_LONG_RANGE = 1 << 16
-
-
-def portion_has_long_ranges(start: int, num_tokens: int) -> bool:
-    """The plan's rule for one portion: its tokens see 3072 keys or more on average."""
-    return start + num_tokens / 2.0 >= 3072

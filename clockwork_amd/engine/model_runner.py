@@ -26,7 +26,6 @@ from clockwork_amd.engine.batch import (
     StaticPortionBatch,
     StepEntry,
     build_context,
-    portion_has_long_ranges,
 )
 from clockwork_amd.parts.model import DecoderModel
 from clockwork_amd.registry import resolve_architecture
@@ -83,7 +82,7 @@ class ModelRunner:
         self.model_config = self.arch.parse_config(self.config_dict)
         self.spec = self.arch.build_spec(self.model_config)
         self.model = DecoderModel(self.spec)
-        ops.preload(self.model.head_dims(), tiled_products=cfg.model.hip_products)
+        ops.preload(self.model.kernel_libraries(), tiled_products=cfg.model.hip_products)
         plan = self.arch.weight_plan(self.model_config, self.spec)
         params = load_parameters(
             cfg.model.model, plan, self.model.param_specs(), self.dtype, self.device, source=weight_source
@@ -217,7 +216,7 @@ class ModelRunner:
                 raise ValueError(f"request {e.seq_id}: wanted index outside its 1 token")
         if state == "seen":
             batch = StaticDecodeBatch(size, capacity, self._table_width, self.manager, self.device,
-                                      self.model.attention_geometries(), self.num_compute_units)
+                                      self.model.prepare, self.num_compute_units)
             batch.fill(entries, self.manager)
             torch.cuda.synchronize()
             state = self._capture(key, batch)
@@ -249,7 +248,9 @@ class ModelRunner:
         size = n if n == budget else next((b for b in PORTION_GRAPH_SIZES if b >= n), None)
         if size is None:
             return NotImplemented
-        key = ("portion", size, portion_has_long_ranges(entry.start, n), bool(want))
+        # the parts may run other kernels for a portion behind many cached keys than for an early
+        # one: a graph serves the portions of its own class (judged for the padded size)
+        key = ("portion", size, self.model.shape_class([size], [entry.start + size]), bool(want))
         state = self._graphs.get(key)
         if state is None:
             self._graphs[key] = "seen"
@@ -257,9 +258,8 @@ class ModelRunner:
         if state == "eager":
             return NotImplemented
         if state == "seen":
-            batch = StaticPortionBatch(size, key[2], key[3], self._table_width, self.manager, self.device,
-                                       self.model.attention_geometries(), self.num_compute_units,
-                                       self.spec.vocab_size)
+            batch = StaticPortionBatch(size, entry.start, bool(want), self._table_width, self.manager, self.device,
+                                       self.model.prepare, self.num_compute_units, self.spec.vocab_size)
             batch.fill(entry, self.manager)
             torch.cuda.synchronize()
             state = self._capture(key, batch)
@@ -279,7 +279,7 @@ class ModelRunner:
         run eagerly from now on and None is returned."""
         graph = torch.cuda.CUDAGraph(keep_graph=True)
         with capturing(graph, self._graph_pool):
-            out = self.model.forward(batch.ctx, self.caches)
+            out = self._forward(batch.ctx)
         kinds = node_kinds(graph)
         self.graph_nodes[key] = dict(kinds)
         if not only_kernels(kinds):
@@ -308,7 +308,7 @@ class ModelRunner:
         ``step_prepared``, or None when the step cannot simply replay a captured graph (then
         ``step`` runs it as usual). Everything but the tokens is written to the pinned buffer."""
         n = len(positions)
-        if not (self.use_graphs and not self.manager.state_groups and 0 < n <= GRAPH_BATCH_SIZES[-1]):
+        if not (self.use_graphs and 0 < n <= GRAPH_BATCH_SIZES[-1]):
             return None
         size = next(b for b in GRAPH_BATCH_SIZES if b >= n)
         longest = max(start + 1 for _, start in positions)
@@ -351,6 +351,14 @@ class ModelRunner:
         return out[: len(entries)]
 
     # ------------------------------------------------------------------ the step
+    def _forward(self, ctx):
+        """The model's step on a laid-out batch: requests that begin in it start from an empty
+        fixed-size state (cleared on the device, by the step's own first positions, so that a
+        captured step does it too), then the parts run."""
+        if self.pools.state:
+            self.pools.zero_fresh_state(ctx.state_slots, ctx.starts, ctx.num_requests)
+        return self.model.forward(ctx, self.caches)
+
     @torch.no_grad()
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Run the entries as one batch; float32 logits [wanted, vocab] in the order of the
@@ -359,23 +367,19 @@ class ModelRunner:
         step runs, so a caller that keeps logits across steps copies them."""
         if not entries:
             return None
-        if (self.use_graphs and not self.manager.state_groups and len(entries) <= GRAPH_BATCH_SIZES[-1]
+        if (self.use_graphs and len(entries) <= GRAPH_BATCH_SIZES[-1]
                 and all(len(e.tokens) == 1 for e in entries)):
             logits = self._graph_step(entries)
             if logits is not NotImplemented:
                 return logits
-        if (self.use_graphs and not self.manager.state_groups and len(entries) == 1
+        if (self.use_graphs and len(entries) == 1
                 and len(entries[0].tokens) > ops.STREAM_MAX_ROWS):
             logits = self._portion_graph_step(entries[0])
             if logits is not NotImplemented:
                 return logits
-        if self.manager.state_groups:
-            for e in entries:
-                if e.start == 0:
-                    self.pools.zero_state(self.manager.state_slot(e.seq_id))
         ctx = build_context(entries, self.manager, self.device, self.spec.vocab_size)
         ctx.num_compute_units = self.num_compute_units
-        logits = self.model.forward(ctx, self.caches)
+        logits = self._forward(ctx)
         for e in entries:
             self.manager.release_behind_window(e.seq_id, e.start + len(e.tokens))
         return logits

@@ -62,16 +62,20 @@ def _load(name: str, head_dim: int | None = None) -> ctypes.CDLL:
     return lib
 
 
-def preload(head_dims=(), tiled_products: bool = False, sampling: bool = False) -> None:
-    """Build (side by side, if several are missing) and load what a model with these head sizes
-    runs: the common kernels, the products and one attention library per head size; the tiled
-    product and the sampling kernels only for a caller that uses them."""
+def preload(libraries=(), tiled_products: bool = False, sampling: bool = False) -> None:
+    """Build (side by side, if several are missing) and load what a model runs: the common
+    kernels, the products and the ``libraries`` its parts name, as (name, head size or None)
+    pairs, e.g. ("attention", 128); the tiled product and the sampling kernels only for a caller
+    that uses them."""
     jobs = [("core", None), ("gemm", None)]
     if tiled_products:
         jobs.append(("gemm_tile", None))
     if sampling:
         jobs.append(("sampling", None))
-    jobs += [("attention", int(hd)) for hd in sorted(set(head_dims))]
+    for name, head_dim in libraries:
+        job = (str(name), None if head_dim is None else int(head_dim))
+        if job not in jobs:
+            jobs.append(job)
     build.ensure_many(jobs)
     for name, hd in jobs:
         _load(name, hd)
@@ -90,6 +94,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_rope_kv_write": [P, I, P, I, P, P, P, I, I, I, I, I, P, P, L, P],
             "cw_silu_mul": [P, P, I, I, I, P],
             "cw_copy_pages": [P, I, L, L, P, I, P],
+            "cw_zero_state_rows": [P, I, I, L, P, P, I, P],
             "cw_bf16_to_f32": [P, P, L, P],
         },
         "gemm": {
@@ -349,6 +354,20 @@ def copy_pages(pool: torch.Tensor, pairs: torch.Tensor) -> None:
     if not (pairs.dtype == torch.int32 and pairs.dim() == 2 and pairs.shape[1] == 2):
         raise KernelError("pairs must be int32 [n, 2]")
     _check(_load("core").cw_copy_pages(_ptr(pool), planes, num_blocks, block_bytes, _ptr(pairs), pairs.shape[0], _stream()), "copy_pages")
+
+
+def zero_state_rows(pool: torch.Tensor, slots: torch.Tensor, starts: torch.Tensor, n: int) -> None:
+    """pool [entries, num_slots, ...]: for each of the first ``n`` requests of a step that starts at
+    position 0 (``starts[r] == 0``), clear row ``slots[r]`` in every entry; a slot outside
+    [0, num_slots) clears nothing. A kernel, so a captured step may hold it."""
+    _gpu(pool, slots, starts)
+    _i32(slots, n, "slots")
+    _i32(starts, n, "starts")
+    if pool.dim() < 2:
+        raise KernelError("a state pool is [entries, slots, ...]")
+    row_bytes = (pool[0, 0].numel() if pool.dim() > 2 else 1) * pool.element_size()
+    _check(_load("core").cw_zero_state_rows(_ptr(pool), pool.shape[0], pool.shape[1], row_bytes, _ptr(slots),
+                                            _ptr(starts), int(n), _stream()), "zero_state_rows")
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, partial_ok: bool = False):

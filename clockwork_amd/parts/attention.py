@@ -8,6 +8,10 @@ portions and single tokens in the same step; output product.
 
 from __future__ import annotations
 
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
 import torch
 
 from clockwork_amd import ops
@@ -16,6 +20,120 @@ from clockwork_amd.parts.base import EntryCache, Part
 from clockwork_amd.parts.rope import NoPosition
 from clockwork_amd.parts.specs import AttentionSpec
 from clockwork_amd.registry import build_part
+
+
+@dataclass
+class AttentionPlan:
+    """Work items of the attention kernels for one head geometry (see csrc/attention.hip).
+
+    Requests with one token go to the 16-row kernel, cut over their keys into
+    ``single_splits`` parts; longer portions are cut into tiles of the 64-row kernel."""
+
+    wide_items: Optional[torch.Tensor] = None
+    n_wide: int = 0
+    gh_wide: int = 1
+    mfma_items: Optional[torch.Tensor] = None   # the same portions cut for the bfloat16 matrix-core kernel
+    n_mfma: int = 0
+    mfma_row_blocks: int = 4   # row blocks of that kernel's workgroups: 2 when 4 would leave compute units idle
+    single_items: Optional[torch.Tensor] = None
+    n_single: int = 0
+    gh_single: int = 1
+    chunks_single: int = 1
+    single_splits: int = 1
+    decode_splits: int = 1   # splits of the bfloat16 decode kernel (finer: it walks 16-key tiles)
+    decode_split_keys: int = 0    # keys of each of those splits, at fixed places (a multiple of 32)
+    decode_max_ctx: int = 0       # the longest context the fixed places were planned for
+    single_identity: bool = False  # a batch of single tokens only: item i is request i, token row i
+
+
+# a portion's key ranges count as long when its tokens see this many keys or more on average
+LONG_RANGE_KEYS = 3072
+
+
+def portions_have_short_ranges(q_lens, ctx_lens) -> bool:
+    """The rule by which a step's portions (entries of more than one token) choose the shape of
+    the matrix-core kernel's workgroups: True while their tokens see fewer than 3072 keys on
+    average. Behind a long cached prefix every workgroup's key range is long and about the same,
+    and sharing the keys among more rows wins (2048 tokens of the 1.5B shape: 46 against 52 us
+    with no prefix, 94 against 96 us behind 2048 tokens, 197 against 182 us behind 6144)."""
+    tokens = sum(q for q in q_lens if q > 1)
+    keys = sum(q * (c - q / 2.0) for q, c in zip(q_lens, ctx_lens) if q > 1)
+    return tokens > 0 and keys / tokens < LONG_RANGE_KEYS
+
+
+def attention_plan(ctx, nh: int, nkv: int, narrow_ok: bool = False) -> AttentionPlan:
+    """The step's work items for heads of this geometry, made once a step and kept in
+    ``ctx.plans``. ``narrow_ok``: the matrix-core kernel for portions also comes with two row
+    blocks a workgroup (see ``ops.prefill_row_blocks_ok``)."""
+    # a batch of single tokens has no portions: one plan, whatever the kernel for portions offers
+    narrow_ok = bool(narrow_ok) and any(q > 1 for q in ctx.h_q_lens)
+    key = ("attention", nh, nkv, narrow_ok)
+    plan = ctx.plans.get(key)
+    if plan is None:
+        plan = ctx.plans[key] = _make_plan(ctx, nh, nkv, narrow_ok)
+    return plan
+
+
+def _make_plan(ctx, nh: int, nkv: int, narrow_ok: bool) -> AttentionPlan:
+    group = nh // nkv
+    gh_wide = min(group, 64)
+    tokens_per_tile = 64 // gh_wide
+    gh_single = min(group, 16)
+    wide: list = []   # one array of items per portion
+    mfma: list = []
+    # Workgroups of four row blocks share each key among the most rows, but a launch has to
+    # fill the compute units, and the workgroup with the longest key range decides its time:
+    # with fewer than 1.5 workgroups a compute unit, halve them (unless the key ranges are long).
+    tokens_of_four = 4 * (32 // min(group, 32))
+    workgroups = sum(-(-q // tokens_of_four) for q in ctx.h_q_lens if q > 1) * nkv * -(-group // 32)
+    short_ranges = portions_have_short_ranges(ctx.h_q_lens, ctx.h_ctx_lens)
+    row_blocks = 2 if narrow_ok and short_ranges and 2 * workgroups < 3 * ctx.num_compute_units else 4
+    tokens_per_mfma_item = row_blocks * (32 // min(group, 32))
+    single: list[int] = []
+    longest_single = 0
+
+    def items_of(r: int, q_len: int, step: int, longest_first: bool) -> np.ndarray:
+        """(request, first token, tokens, 0) for runs of ``step`` tokens of one portion."""
+        tok0 = np.arange(0, q_len, step, dtype=np.int32)
+        if longest_first:
+            tok0 = tok0[::-1]
+        out = np.zeros((tok0.size, 4), dtype=np.int32)
+        out[:, 0] = r
+        out[:, 1] = tok0
+        out[:, 2] = np.minimum(step, q_len - tok0)
+        return out.reshape(-1)
+
+    for r, q_len in enumerate(ctx.h_q_lens):
+        if q_len == 1:
+            single += [r, 0, 1, 0]
+            longest_single = max(longest_single, ctx.h_ctx_lens[r])
+        else:
+            wide.append(items_of(r, q_len, tokens_per_tile, False))
+            # longest key ranges first: the last tokens of a portion have the most work
+            mfma.append(items_of(r, q_len, tokens_per_mfma_item, True))
+    wide = np.concatenate(wide) if wide else np.zeros(0, dtype=np.int32)
+    mfma = np.concatenate(mfma) if mfma else np.zeros(0, dtype=np.int32)
+    plan = AttentionPlan(gh_wide=gh_wide, gh_single=gh_single, mfma_row_blocks=row_blocks)
+    plan.n_wide, plan.n_single, plan.n_mfma = len(wide) // 4, len(single) // 4, len(mfma) // 4
+    plan.chunks_single = -(-group // gh_single)
+    if plan.n_single:
+        groups_running = plan.n_single * nkv * plan.chunks_single
+        by_occupancy = -(-4 * ctx.num_compute_units // groups_running)
+        by_length = max(1, longest_single // 256)
+        plan.single_splits = max(1, min(by_occupancy, by_length, 64))
+        # decode kernel: a workgroup per (request, kv head, split); a split is at least 128 keys
+        # (one 32-key tile for each of its four waves), and about two workgroups per compute
+        # unit are enough to keep memory busy. More than 64 splits never paid: one request
+        # with 30000 keys takes 16 us with 64 to 128 splits and 19 us with 235.
+        base = plan.n_single * nkv * -(-group // min(group, 16))
+        plan.decode_splits = max(1, min(-(-2 * ctx.num_compute_units // base), longest_single // 128, 64))
+        # fixed places for the splits: a workgroup then knows its pages before it knows the
+        # request's length, which saves it a trip to memory
+        plan.decode_split_keys = 32 * -(-(-(-longest_single // plan.decode_splits)) // 32)
+        plan.decode_max_ctx = longest_single
+        plan.single_identity = plan.n_single == len(ctx.h_q_lens)
+    plan.wide_items, plan.single_items, plan.mfma_items = ctx.upload([wide, single, mfma])
+    return plan
 
 
 class PagedAttention(Part):
@@ -46,11 +164,30 @@ class PagedAttention(Part):
     def cache_need(self):
         return KVPagesSpec(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)
 
+    def kernel_libraries(self) -> list:
+        return [("attention", int(self.spec.head_dim))]
+
+    def _plan(self, ctx, dtype) -> AttentionPlan:
+        hd = self.spec.head_dim
+        narrow_ok = ops.prefill_attention_supported(hd, dtype) and ops.prefill_row_blocks_ok(hd, 2)
+        return attention_plan(ctx, self.spec.num_heads, self.spec.num_kv_heads, narrow_ok=narrow_ok)
+
+    def prepare(self, ctx) -> None:
+        """The step's work items, before ``forward`` (a captured step must not make them)."""
+        self._plan(ctx, self.dtype)
+
+    def shape_class(self, q_lens, ctx_lens):
+        """Portions behind a long cached prefix run another workgroup shape than early ones."""
+        if not any(q > 1 for q in q_lens):
+            return "single tokens"
+        return "short key ranges" if portions_have_short_ranges(q_lens, ctx_lens) else "long key ranges"
+
     def bind(self, params, device, dtype) -> None:
         self.qkv_weight = params["qkv_weight"]
         self.qkv_bias = params.get("qkv_bias")
         self.out_weight = params["out_weight"]
         self.out_bias = params.get("out_bias")
+        self.dtype = dtype
         self.position.bind({}, device, dtype)
 
     def forward(self, x: torch.Tensor, ctx, cache: EntryCache) -> torch.Tensor:
@@ -75,7 +212,7 @@ class PagedAttention(Part):
             self.position.rotate_and_store(qkv, bias, ctx.positions, None, nh, 0, hd, None, None)
         out = torch.empty((T, self.q_width), dtype=x.dtype, device=x.device)
         mfma = ops.prefill_attention_supported(hd, x.dtype)
-        plan = ctx.attention_plan(nh, nkv, narrow_ok=mfma and ops.prefill_row_blocks_ok(hd, 2))
+        plan = self._plan(ctx, x.dtype)
         common = dict(
             q=qkv, q_stride=qkv.shape[1], out=out, k_cache=cache.k, v_cache=cache.v,
             block_tables=ctx.block_tables[cache.group], ctx_lens=ctx.ctx_lens, cu_q=ctx.cu_q,

@@ -1,4 +1,4 @@
-"""Interfaces of the parts a layer is put together from.
+"""Interfaces of the parts a model is put together from.
 
 A part is built from its spec alone (sizes and constants are parameters; no part
 knows which model it is in) and goes through three stages:
@@ -6,10 +6,13 @@ knows which model it is in) and goes through three stages:
 1. ``param_specs()`` - the tensors it owns: ``{local name: ParamSpec}``. Needs no GPU.
 2. ``bind(params, device, dtype)`` - receives ``{local name: device tensor}`` and
    prepares whatever else it needs on the device (tables, constants).
-3. its run method, called by the block arrangement during a step.
+3. its run method, called during a step.
 
 Roles and their run methods:
 
+* embedding:     ``forward(ctx) -> resid``: the float32 residual stream [T, H] of the step's
+                 tokens (``ctx.token_ids``, ``ctx.positions``). May offer ``table()``, the
+                 [vocab, H] matrix a tied head uses.
 * norm:          ``forward(resid, delta, rows=None) -> normed`` - ``resid`` is the
                  float32 residual stream [T, H]; ``delta`` (activation type, an
                  ``ops.PartialSums`` of that shape, or None)
@@ -25,9 +28,32 @@ Roles and their run methods:
                  uses ``project_rotate_store(x, weight, bias, positions, slots, nh, nkv, hd,
                  k, v) -> q or None`` when the part offers it (product, encoding and cache
                  write in one kernel).
-* arrangement:   ``forward(resid, delta, ctx, cache) -> delta`` - wires norms,
-                 mixer and feed-forward around the residual stream; the returned
-                 ``delta`` is the last branch output, not yet added.
+* arrangement:   built by its factory from the block's parts as keyword arguments, under
+                 the names the ``LayerSpec`` gives them (``mixer``, ``feed_forward``,
+                 ``mixer_norm``, ``ffn_norm`` or any others). ``parts() -> {name: part}``;
+                 ``forward(resid, delta, ctx, cache) -> delta`` wires norms, mixer and
+                 feed-forward around the residual stream; the returned ``delta`` is the last
+                 branch output, not yet added. The part named ``mixer`` owns the block's
+                 cache; the part named ``mixer_norm`` is the first to take the delta handed on.
+* head:          ``forward(rows, ctx) -> logits``: float32 [n, vocab] for the final norm's rows.
+                 A head whose spec has ``tied`` set gets ``use_embedding(embedding part)``
+                 before ``bind``. ``matrices()``: what a step streams through it (byte counts).
+
+What any part may add:
+
+* ``graph_safe = True``: its step is a fixed sequence of launches on the device (no host
+  reads, no shapes that depend on data), so a step may be captured as a HIP graph.
+* ``prepare(ctx)``: make, before ``forward``, what depends on the step's shape alone (work
+  items, uploaded through ``ctx.upload``) and keep it in ``ctx.plans``; a captured step is
+  prepared once, outside the capture.
+* ``shape_class(q_lens, ctx_lens)``: a label for what of a step's shape decides which kernels
+  the part launches; a captured graph serves steps of its own class.
+* ``kernel_libraries()``: the HIP libraries it runs, as (name, head size or None).
+
+Fixed-size state: ``cache.state`` is [slots, *shape] of the run entry; a request's row is
+``ctx.state_slots[r]`` (``ctx.h_state_slots`` on the host). Rows of a fixed-shape batch that
+hold no request carry the pool's spare last slot, so a part may read and write every row's
+slot; the state of a request whose first token runs in the step is cleared before the parts run.
 """
 
 from __future__ import annotations

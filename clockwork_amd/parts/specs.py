@@ -64,3 +64,21 @@ class SwiGLUSpec:
 
     hidden_size: int
     intermediate_size: int
+
+
+@dataclass(frozen=True)
+class TokenEmbeddingSpec:
+    """The residual stream starts as row ``id`` of a [vocab, hidden] table: no scaling, nothing added."""
+
+    vocab_size: int
+    hidden_size: int
+
+
+@dataclass(frozen=True)
+class LinearHeadSpec:
+    """logits = rows @ W^T with W [vocab, hidden], no bias, float32 logits. ``tied``: W is the
+    embedding's table (one buffer, two uses) unless the checkpoint brings a head of its own."""
+
+    vocab_size: int
+    hidden_size: int
+    tied: bool = False

@@ -50,8 +50,9 @@ def unregister_architecture(names: list[str]) -> None:
 def resolve_architecture(config: dict) -> Architecture:
     """Pick the architecture by ``architectures[0]``, else by ``model_type``.
 
-    Anything unknown is refused the way the reference refuses it
-    (clockwork/engine/loader.py:70-71).
+    Anything unknown is refused (the reference refuses every model_type but its own,
+    clockwork/engine/loader.py:70-71; an architecture's ``parse_config`` repeats that check
+    for its own name).
     """
     keys = []
     archs = config.get("architectures")
@@ -66,7 +67,7 @@ def resolve_architecture(config: dict) -> Architecture:
             return _ARCHITECTURES[key]
     known = sorted(set(_ARCHITECTURES) | set(_BUILTIN_ARCHITECTURES))
     raise ValueError(
-        f"expected a qwen2 model, got model_type={config.get('model_type')!r} "
+        f"no architecture is registered for model_type={config.get('model_type')!r} "
         f"architectures={config.get('architectures')!r}; registered: {known}"
     )
 
@@ -81,6 +82,8 @@ _BUILTIN_PARTS = {
     "RopeNeoxSpec": ("clockwork_amd.parts.rope", "RopeNeox"),
     "AttentionSpec": ("clockwork_amd.parts.attention", "PagedAttention"),
     "SwiGLUSpec": ("clockwork_amd.parts.mlp", "SwiGLU"),
+    "TokenEmbeddingSpec": ("clockwork_amd.parts.embedding", "TokenEmbedding"),
+    "LinearHeadSpec": ("clockwork_amd.parts.embedding", "LinearHead"),
 }
 _ARRANGEMENTS: dict[str, Callable[..., Any]] = {}
 _BUILTIN_ARRANGEMENTS = {"prenorm": ("clockwork_amd.parts.block", "PreNormBlock")}

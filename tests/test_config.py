@@ -111,9 +111,13 @@ def test_qwen2_config_refuses_what_is_not_built():
 def test_registry_picks_by_architecture_or_model_type_and_rejects_the_rest():
     assert resolve_architecture({"architectures": ["Qwen2ForCausalLM"]}).name == "Qwen2ForCausalLM"
     assert resolve_architecture({"model_type": "qwen2"}).name == "Qwen2ForCausalLM"
-    # clockwork/engine/loader.py:70-71
-    with pytest.raises(ValueError, match="expected a qwen2 model, got model_type='llama'"):
+    # clockwork/engine/loader.py:70-71: whatever is not the built architecture is refused; the
+    # registry names what it was given and what it knows, the architecture itself keeps the
+    # reference's words for a config that reaches it under a wrong model_type
+    with pytest.raises(ValueError, match="no architecture is registered for model_type='llama'.*Qwen2ForCausalLM"):
         resolve_architecture({"model_type": "llama", "architectures": ["LlamaForCausalLM"]})
+    with pytest.raises(ValueError, match="expected a qwen2 model, got model_type='llama'"):
+        Qwen2Config.from_dict(dict(TINY_A, model_type="llama"))
 
 
 def test_spec_carries_the_config_layer_by_layer():

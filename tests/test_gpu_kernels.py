@@ -556,6 +556,7 @@ def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs,
                    decode_kernel=False, prefill_kernel=False, fixed_ranges=False):
     from clockwork_amd import ops
     from clockwork_amd.engine.batch import StepContext
+    from clockwork_amd.parts.attention import attention_plan
 
     ctx = StepContext()
     ctx.device = torch.device(DEV)
@@ -563,7 +564,7 @@ def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs,
     # prefill_kernel: True or 4 for workgroups of four row blocks, 2 for two (few work items here,
     # so the plan takes the small workgroups whenever it may)
     narrow = prefill_kernel == 2 and not isinstance(prefill_kernel, bool)
-    plan = ctx.attention_plan(nh, nkv, narrow_ok=narrow)
+    plan = attention_plan(ctx, nh, nkv, narrow_ok=narrow)
     assert plan.mfma_row_blocks == (2 if narrow else 4)
     if splits is not None:
         plan.single_splits = splits

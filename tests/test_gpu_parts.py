@@ -1,7 +1,9 @@
-"""Each part alone against the plain formulas, and the framework's openness: toy parts and a toy
-architecture defined here are registered, built from a model folder and stepped without any
+"""Each part alone against the plain formulas, and the framework's openness: toy parts and toy
+architectures defined here are registered, built from a model folder and stepped without any
 change to the framework's files (a mixer with state of its own, windowed attention in a group
-of its own, a layer that runs twice, a layer that reads another layer's cache)."""
+of its own, a layer that runs twice, a layer that reads another layer's cache; a second toy with
+an embedding and an output head of its own, a block with one norm, and a mixer with state whose
+decode steps replay as HIP graphs)."""
 
 import json
 from dataclasses import dataclass
@@ -376,6 +378,233 @@ def test_a_toy_architecture_registers_builds_and_steps(toy_dir, dtype, mode):
     assert [p.num_free for p in runner.manager.pools] == [64, 64]
 
 
+# ---------------------------------------------------------------------------------- a second toy
+@dataclass(frozen=True)
+class ScaledEmbeddingSpec:
+    """The stream starts as multiplier * table[id]."""
+
+    vocab_size: int
+    hidden_size: int
+    multiplier: float
+
+
+class ScaledEmbedding:
+    graph_safe = True
+
+    def __init__(self, spec):
+        self.spec = spec
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.spec.vocab_size, self.spec.hidden_size))}
+
+    def bind(self, params, device, dtype):
+        self.weight = params["weight"]
+
+    def table(self):
+        return self.weight
+
+    def forward(self, ctx):
+        return self.weight[ctx.token_ids.long()].float() * self.spec.multiplier
+
+
+@dataclass(frozen=True)
+class CappedHeadSpec:
+    """logits = cap * tanh(rows @ table^T / cap), the table being the embedding's."""
+
+    cap: float
+    tied: bool = True
+
+
+class CappedHead:
+    graph_safe = True
+
+    def __init__(self, spec):
+        self.spec = spec
+
+    def param_specs(self):
+        return {}
+
+    def use_embedding(self, embedding):
+        self.embedding = embedding
+
+    def bind(self, params, device, dtype):
+        pass
+
+    def forward(self, rows, ctx):
+        from clockwork_amd import ops
+
+        logits = ops.linear(rows, self.embedding.table(), out_dtype=torch.float32)
+        return self.spec.cap * torch.tanh(logits / self.spec.cap)
+
+
+class OneNormBlock:
+    """h = h + mixer(norm(h)) + ffn(norm(h)): one norm feeds both branches."""
+
+    def __init__(self, mixer, feed_forward, mixer_norm):
+        self.mixer, self.feed_forward, self.mixer_norm = mixer, feed_forward, mixer_norm
+
+    def parts(self):
+        return {"mixer": self.mixer, "feed_forward": self.feed_forward, "mixer_norm": self.mixer_norm}
+
+    def forward(self, resid, delta, ctx, cache):
+        from clockwork_amd import ops
+
+        x = self.mixer_norm.forward(resid, delta)
+        a = self.mixer.forward(x, ctx, cache)
+        f = self.feed_forward.forward(x, ctx)
+        a = a.sum(x.dtype) if isinstance(a, ops.PartialSums) else a
+        f = f.sum(x.dtype) if isinstance(f, ops.PartialSums) else f
+        return (a.float() + f.float()).to(x.dtype)
+
+
+@dataclass(frozen=True)
+class DecayMixerSpec:
+    """s_t = decay * s_{t-1} + x_t, y_t = s_t W: a state per request, kept in float32."""
+
+    hidden_size: int
+    decay: float
+
+
+class DecayMixer:
+    """Steps of single tokens run on the device alone (a gather and a scatter by the step's state
+    slots), so they can be captured as graphs; portions walk their tokens from the host."""
+
+    graph_safe = True
+
+    def __init__(self, spec):
+        self.spec = spec
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.spec.hidden_size, self.spec.hidden_size), init=("normal", 0.05))}
+
+    def cache_need(self):
+        return StateSpec((self.spec.hidden_size,), "float32")
+
+    def bind(self, params, device, dtype):
+        self.weight = params["weight"]
+
+    def forward(self, x, ctx, cache):
+        xf = x.float()
+        if all(n == 1 for n in ctx.h_q_lens):
+            slots = ctx.state_slots.long()       # rows that hold no request carry the spare slot
+            s = self.spec.decay * cache.state[slots] + xf
+            cache.state[slots] = s
+        else:
+            s = torch.empty_like(xf)
+            at = 0
+            for r, n in enumerate(ctx.h_q_lens):
+                state = cache.state[ctx.h_state_slots[r]].clone()
+                for t in range(at, at + n):
+                    state = self.spec.decay * state + xf[t]
+                    s[t] = state
+                cache.state[ctx.h_state_slots[r]] = state
+                at += n
+        return (s @ self.weight.float().t()).to(x.dtype)
+
+
+@dataclass(frozen=True)
+class Toy2Config:
+    vocab: int
+    hidden: int
+    multiplier: float
+    cap: float
+    decay: float
+    eps: float
+
+
+def _toy2_spec(cfg: Toy2Config) -> ModelSpec:
+    norm = RMSNormSpec(cfg.hidden, cfg.eps)
+    ffn = SwiGLUSpec(cfg.hidden, 3 * cfg.hidden)
+    attn = AttentionSpec(cfg.hidden, 4, 1, 16, True, False, 0.25, position=RopeNeoxSpec(rotary_dim=16, theta=500.0))
+    layers = [
+        LayerSpec("one_norm", mixer=attn, feed_forward=ffn, mixer_norm=norm),      # no second norm
+        LayerSpec("prenorm", DecayMixerSpec(cfg.hidden, cfg.decay), ffn, norm, norm),
+    ]
+    return ModelSpec("Toy2ForCausalLM", cfg.vocab, cfg.hidden, layers, [RunEntry(0), RunEntry(1)], norm,
+                     embedding=ScaledEmbeddingSpec(cfg.vocab, cfg.hidden, cfg.multiplier), head=CappedHeadSpec(cfg.cap))
+
+
+@pytest.fixture(scope="module")
+def toy2_dir(tmp_path_factory):
+    from clockwork_amd.registry import register_arrangement
+    from clockwork_amd.weights.random_init import write_random_model
+
+    register_part(ScaledEmbeddingSpec, ScaledEmbedding)
+    register_part(CappedHeadSpec, CappedHead)
+    register_part(DecayMixerSpec, DecayMixer)
+    register_arrangement("one_norm", OneNormBlock)
+    register_architecture(
+        ["Toy2ForCausalLM"],
+        Architecture(
+            "Toy2ForCausalLM",
+            parse_config=lambda d: Toy2Config(d["vocab"], d["hidden"], d["multiplier"], d["cap"], d["decay"], d["eps"]),
+            build_spec=_toy2_spec,
+            weight_plan=_toy_plan,
+        ),
+    )
+    config = {"architectures": ["Toy2ForCausalLM"], "vocab": 211, "hidden": 64, "multiplier": 3.0, "cap": 0.4,
+              "decay": 0.8, "eps": 1e-5}
+    return write_random_model(tmp_path_factory.mktemp("toy2") / "toy2", config, seed=8)
+
+
+def _toy2_plain_logits(model_dir, tokens):
+    from safetensors.torch import load_file
+
+    cfg = json.loads((model_dir / "config.json").read_text())
+    w = {k: v.float() for k, v in load_file(str(model_dir / "model.safetensors")).items()}
+    assert not any(k.startswith("lm_head.") for k in w)
+    T, H = len(tokens), cfg["hidden"]
+    h = cfg["multiplier"] * plain.embedding(w["embed.weight"], torch.tensor(tokens))
+    # block 0: one norm, attention and feed-forward side by side
+    x = plain.rmsnorm(h, w["layers.0.mixer_norm.weight"], cfg["eps"])
+    qkv = plain.linear(x, w["layers.0.mixer.qkv_weight"], w["layers.0.mixer.qkv_bias"])
+    cos, sin = plain.rope_tables(torch.arange(T), 16, 500.0)
+    q = plain.apply_rope(qkv[:, :64].view(T, 4, 16), cos, sin)
+    k = plain.apply_rope(qkv[:, 64:80].view(T, 1, 16), cos, sin)
+    v = qkv[:, 80:].view(T, 1, 16)
+    a = plain.linear(plain.attention_dense(q, k, v, 0.25).reshape(T, 64), w["layers.0.mixer.out_weight"])
+    gu = w["layers.0.feed_forward.gate_up_weight"]
+    h = h + a + plain.swiglu(x, gu[: 3 * H], gu[3 * H :], w["layers.0.feed_forward.down_weight"])
+    # block 1: the recurrence, then a feed-forward behind a norm of its own
+    x = plain.rmsnorm(h, w["layers.1.mixer_norm.weight"], cfg["eps"])
+    s, rows = torch.zeros(H), []
+    for t in range(T):
+        s = cfg["decay"] * s + x[t]
+        rows.append(s)
+    h = h + torch.stack(rows) @ w["layers.1.mixer.weight"].t()
+    x = plain.rmsnorm(h, w["layers.1.ffn_norm.weight"], cfg["eps"])
+    gu = w["layers.1.feed_forward.gate_up_weight"]
+    h = h + plain.swiglu(x, gu[: 3 * H], gu[3 * H :], w["layers.1.feed_forward.down_weight"])
+    logits = plain.linear(plain.rmsnorm(h, w["final_norm.weight"], cfg["eps"]), w["embed.weight"])
+    return cfg["cap"] * torch.tanh(logits / cfg["cap"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["whole", "prefill_then_decode", "portions", "mixed"])
+def test_a_second_toy_with_its_own_embedding_head_and_block(toy2_dir, dtype, mode):
+    """An embedding with a multiplier, a capped head tied to it, a block with one norm and a mixer
+    with state, all registered from this file. Its single-token steps replay as HIP graphs although
+    it keeps state: a fresh request's state is cleared by a kernel inside the step."""
+    gen = torch.Generator().manual_seed(6)
+    requests = {f"u{i}": torch.randint(0, 211, (n,), generator=gen).tolist() for i, n in enumerate([50, 9, 77, 1, 64])}
+    runner = replay.make_runner(toy2_dir, dtype, 8, 40)
+    assert [(g.is_kv, g.entries) for g in runner.manager.groups] == [(True, (0,)), (False, (1,))]
+    assert runner.use_graphs and runner.manager.idle_state_slot == runner.manager.max_num_seqs
+    got = replay.run_trace(runner, getattr(replay, mode)(requests))
+    ref = {rid: _toy2_plain_logits(toy2_dir, toks) for rid, toks in requests.items()}
+    if dtype == "float32":
+        replay.compare(got, ref, rtol=1e-5, atol=1e-5)
+    else:
+        replay.compare_to_scale(got, ref)
+    captured = [k for k, v in runner._graphs.items() if isinstance(v, tuple)]
+    if mode in ("prefill_then_decode", "mixed"):
+        assert captured, "no single-token step was replayed as a graph"
+        assert all(set(runner.graph_nodes[k]) == {"kernel"} for k in captured)
+    assert not runner.manager.live_requests()
+    # slots come back, and a slot that another request used is cleared for the next one
+    assert len(runner.manager._free_slots) == runner.manager.max_num_seqs
+
+
 def test_windowed_group_uses_few_pages_for_a_long_request(toy_dir):
     runner = replay.make_runner(toy_dir, "float32", 8, 64)
     toks = torch.randint(0, 300, (200,), generator=torch.Generator().manual_seed(6)).tolist()
@@ -400,5 +629,5 @@ def test_unknown_parts_and_architectures_are_refused():
         build_part(Unknown())
     from clockwork_amd.registry import resolve_architecture
 
-    with pytest.raises(ValueError, match="expected a qwen2 model"):
+    with pytest.raises(ValueError, match="no architecture is registered"):
         resolve_architecture({"architectures": ["NopeForCausalLM"], "model_type": "nope"})
