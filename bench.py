@@ -68,7 +68,7 @@ def build_runner(args, prefix_cache: bool = False, max_batch: int = 0):
     max_batch = max(args.batch, 64, max_batch)
     context = context_of(args)
     cfg = EngineConfig.defaults(
-        "random:qwen2.5-1.5b", dtype=args.dtype, max_model_len=context, block_size=BLOCK,
+        f"random:{SHAPES[args.shape][0].lower()}", dtype=args.dtype, max_model_len=context, block_size=BLOCK,
         num_blocks=max_batch * context // BLOCK, enable_prefix_cache=prefix_cache, watermark=0.0,
         max_num_seqs=max_batch, max_num_batched_tokens=max(PROMPT_LEN, max_batch),
     )
@@ -106,16 +106,28 @@ def time_decode(cfg, runner, batch: int, steps: int, warmup: int, sampling=None,
     seqs = list(engine.scheduler.running)
     assert len(seqs) == batch and all(s.num_uncomputed_tokens() == 1 for s in seqs)
     ctx_begin = sum(len(s) for s in seqs) / batch
+    # the host's clock around the whole loop is the measurement; events on the GPU's queue after
+    # every step give the steps' own times beside it (the notebook's method, bench_t4.ipynb:236-250)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    marks[0].record()
     t0 = time.perf_counter()
-    for _ in range(steps):
+    for i in range(steps):
         outs = engine.step()
+        marks[i + 1].record()
         assert len(outs) == batch
     _sync()
     elapsed = time.perf_counter() - t0
     for i in range(batch):
         engine.abort_request(f"b{batch}-{i}")
     mean_ctx = ctx_begin + (steps - 1) / 2.0  # keys a request reads in the middle step
+    gaps = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    LAST_STEP_TIMES.clear()
+    LAST_STEP_TIMES.update(mean=round(sum(gaps) / steps, 4), p50=round(gaps[steps // 2], 4), max=round(gaps[-1], 4))
     return elapsed, mean_ctx
+
+
+# per-step times of the last ``time_decode`` run, from events on the GPU's queue (milliseconds)
+LAST_STEP_TIMES: dict = {}
 
 
 def time_prefill(cfg, runner, repeats: int = 6, total: int = PROMPT_LEN):
@@ -320,6 +332,7 @@ def main() -> int:
     elapsed, mean_ctx = time_decode(cfg, runner, args.batch, args.steps, args.warmup, sampling, args.prompt_len)
     value = args.batch * args.steps / elapsed
     ms = 1e3 * elapsed / args.steps
+    step_times = dict(LAST_STEP_TIMES)
     step_bytes = runner.model.weight_bytes_per_step() + args.batch * mean_ctx * runner.pools.kv_bytes_per_token()
     achieved = step_bytes / (elapsed / args.steps) / 1e9
 
@@ -331,6 +344,7 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms, 4),
+        "ms_per_step_by_gpu_events": step_times,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

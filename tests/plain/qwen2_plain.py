@@ -1,7 +1,7 @@
 """A plain, slow Qwen2: whole sequences, no cache, one function per part.
 
-Written from the reference's formulas (each function cites file:line under
-/root/reference); it shares no code with ``clockwork_amd``: it parses config.json
+Written from the reference's formulas (each function cites file:line in the reference's
+source tree); it shares no code with ``clockwork_amd``: it parses config.json
 and reads the safetensors file itself. Everything runs on the CPU in ``dtype``
 (float32 by default, float64 for invariants).
 """

@@ -95,6 +95,42 @@ def test_tied_head_may_be_absent_untied_may_not(tmp_path):
     assert err.value.missing == ["lm_head.weight"]
 
 
+def test_a_tied_checkpoint_that_carries_its_head_keeps_one_table(tmp_path):
+    """clockwork/engine/model.py:217-218: a tied head is the embedding's parameter, so a head
+    tensor in the file can only be that table again. It is checked and let go (one matrix in
+    memory, one in the step's byte count); a head that differs from the table is an error."""
+    from clockwork_amd.models.qwen2 import Qwen2Config, build_spec
+    from clockwork_amd.parts.model import DecoderModel
+
+    d = write_random_model(tmp_path / "tied", TINY_A, seed=0)
+    tensors = load_file(str(d / "model.safetensors"))
+    tensors["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    save_file(tensors, str(d / "model.safetensors"))
+    spec = build_spec(Qwen2Config.from_dict(TINY_A))
+    model = DecoderModel(spec)
+    params = _load(d, TINY_A)
+    assert "lm_head.weight" in params
+    model.bind(params, torch.device("cpu"), torch.float32)
+    assert model.head.weight is model.embedding.weight and "lm_head.weight" not in model.params
+    alone = DecoderModel(spec)
+    without = {k: v for k, v in params.items() if k != "lm_head.weight"}
+    alone.bind(without, torch.device("cpu"), torch.float32)
+    assert model.weight_bytes_per_step() == alone.weight_bytes_per_step()
+    params["lm_head.weight"] = params["lm_head.weight"].clone()
+    params["lm_head.weight"][3, 5] += 1.0
+    with pytest.raises(ValueError, match="differs from the embedding table"):
+        DecoderModel(spec).bind(params, torch.device("cpu"), torch.float32)
+    # an untied model keeps a head of its own and counts it
+    from tests.configs import TINY_B as B
+
+    spec_b = build_spec(Qwen2Config.from_dict(B))
+    model_b = DecoderModel(spec_b)
+    model_b.bind(_load(write_random_model(tmp_path / "untied", B, seed=1), B), torch.device("cpu"), torch.float32)
+    assert model_b.head.weight is not model_b.embedding.weight
+    assert model_b.weight_bytes_per_step() == sum(
+        t.numel() * t.element_size() for k, t in model_b.params.items() if k != "embed.weight")
+
+
 def test_dtype_rules(tmp_path):
     """Matrices take the engine's dtype; small vectors that the file holds in 32-bit stay 32-bit."""
     d = write_random_model(tmp_path / "m", TINY_A, seed=0)
