@@ -183,7 +183,7 @@ class CacheManager:
         for g, pool in enumerate(self.pools):
             need = max(0, self._blocks_for(self._admission_extent(g, total_len, portion_end)) - len(prefix))
             if need > pool.num_free:
-                raise OutOfPages(f"group {g}: requested {need} blocks, {pool.num_free} free")
+                raise OutOfPages(f"layer group {g}: {need} pages wanted, {pool.num_free} free")
             needs.append(need)
         if self.state_groups and not self._free_slots:
             raise OutOfPages("no free state slot")
@@ -220,7 +220,7 @@ class CacheManager:
             if upto > len(table) * size:
                 return False
             page = table[logical]
-            if page != NO_PAGE and pool._refs[page] > 1:
+            if page != NO_PAGE and pool._holders[page] > 1:
                 return False
         return True
 

@@ -10,7 +10,6 @@ mode; text (prompts, stop strings, ``RequestOutput.text``) needs a tokenizer wit
 from __future__ import annotations
 
 import itertools
-from dataclasses import dataclass
 from typing import Optional
 
 import torch
@@ -24,11 +23,41 @@ from clockwork_amd.engine.sequence import RequestOutput, SamplingParams, Sequenc
 from clockwork_amd.sampling.sampler import Sampler
 
 
-@dataclass
-class _TextState:
-    prefix_offset: int = 0
-    read_offset: int = 0
-    text: str = ""
+class _RequestText:
+    """The text a request has produced so far, grown token by token.
+
+    A token's text can depend on the tokens around it (a character spread over several tokens,
+    a leading space that depends on what came before), so new text is never decoded from the
+    new token alone: the tokens from ``anchor`` on are decoded with and without the newcomers
+    and the difference is what they added (clockwork/engine/llm_engine.py:187-198). While the
+    decoded tail ends in U+FFFD a character is still incomplete and nothing is shown."""
+
+    __slots__ = ("shown", "anchor", "rendered")
+
+    def __init__(self) -> None:
+        self.shown = ""      # text handed out so far (cut where a stop string began)
+        self.anchor = 0      # first output token of the decoding window
+        self.rendered = 0    # output tokens whose text has been handed out
+
+    def grow(self, decode, output_ids: list) -> str:
+        """Text that the tokens past ``rendered`` add; "" while they end inside a character."""
+        with_new = decode(output_ids[self.anchor:])
+        if with_new.endswith("\ufffd"):
+            return ""
+        known = decode(output_ids[self.anchor:self.rendered])
+        self.anchor, self.rendered = self.rendered, len(output_ids)
+        return with_new[len(known):]
+
+    def accept(self, addition: str, stop_strings) -> tuple[str, bool]:
+        """Append ``addition``, unless a stop string shows up: then the text ends where the
+        earliest one begins (llm_engine.py:211-221). Returns (what was really added, stopped)."""
+        text = self.shown + addition
+        starts = [at for at in map(text.find, stop_strings) if at >= 0]
+        if starts:
+            text = text[: min(starts)]
+        added = text[len(self.shown):]  # nothing if the stop string began in text already shown
+        self.shown = text
+        return added, bool(starts)
 
 
 class LLMEngine:
@@ -55,7 +84,7 @@ class LLMEngine:
         self.sampler = Sampler(self.runner.device, cfg.model.seed)
         self._eos_ids = self._resolve_eos()
         self._seqs: dict[str, Sequence] = {}
-        self._text: dict[str, _TextState] = {}
+        self._text: dict[str, _RequestText] = {}
         # arrival "times" are a counter, so order never depends on the clock (llm_engine.py:57-59)
         self._arrivals = itertools.count()
         self._generate_ids = itertools.count()
@@ -119,7 +148,7 @@ class LLMEngine:
             raise ValueError("stop strings need a tokenizer; use stop_token_ids instead")
         seq = Sequence(request_id, prompt_token_ids, params, arrival_time=float(next(self._arrivals)))
         self._seqs[request_id] = seq
-        self._text[request_id] = _TextState()
+        self._text[request_id] = _RequestText()
         self.scheduler.add_seq(seq)
 
     def abort_request(self, request_id: str) -> None:
@@ -264,95 +293,75 @@ class LLMEngine:
     def generate(self, prompts, sampling_params: Optional[SamplingParams] = None) -> list[RequestOutput]:
         """Run prompts (strings or lists of token ids) to completion; final outputs in prompt order
         (llm_engine.py:135-159)."""
-        ids = []
+        finals: dict[str, Optional[RequestOutput]] = {}
         for prompt in prompts:
             request_id = f"generate-{next(self._generate_ids)}"
-            ids.append(request_id)
-            if isinstance(prompt, str):
-                self.add_request(request_id, prompt=prompt, sampling_params=sampling_params)
-            else:
-                self.add_request(request_id, prompt_token_ids=prompt, sampling_params=sampling_params)
-        finals: dict[str, RequestOutput] = {}
-        pending = set(ids)
-        while pending:
+            key = "prompt" if isinstance(prompt, str) else "prompt_token_ids"
+            self.add_request(request_id, sampling_params=sampling_params, **{key: prompt})
+            finals[request_id] = None
+        unfinished = len(finals)
+        while unfinished:
             outputs = self.step()
             for output in outputs:
-                if output.finished and output.request_id in pending:
+                if output.finished and finals.get(output.request_id, output) is None:
                     finals[output.request_id] = output
-                    pending.discard(output.request_id)
-            if not outputs and not self.scheduler.has_unfinished() and pending:
-                raise RuntimeError(f"engine drained with unfinished requests: {sorted(pending)}")
-        return [finals[i] for i in ids]
+                    unfinished -= 1
+            if unfinished and not outputs and not self.scheduler.has_unfinished():
+                lost = sorted(rid for rid, out in finals.items() if out is None)
+                raise RuntimeError(f"the engine has nothing left to run, yet these requests never finished: {lost}")
+        return list(finals.values())
 
     def stats(self) -> dict:
-        sched, cache = self.scheduler.stats, self.prefix_cache.stats
-        return {
-            "num_waiting": sched.num_waiting,
-            "num_running": sched.num_running,
-            "num_preempted_total": sched.num_preempted_total,
-            "num_scheduled_batches": sched.num_scheduled_batches,
-            "total_prompt_tokens": sched.total_prompt_tokens,
-            "total_cached_tokens": sched.total_cached_tokens,
-            "prefix_cache_queries": cache.queries,
-            "prefix_cache_hit_tokens": cache.hit_tokens,
-            "prefix_cache_prompt_tokens": cache.prompt_tokens,
-            "prefix_cache_hit_rate": cache.hit_rate,
-            "num_free_blocks": self.manager.min_free_blocks(),
-            "lookahead_steps": self.lookahead_steps,
-        }
+        """Counters of the scheduler and the prefix cache under the reference's names
+        (llm_engine.py:161-177), and two of this engine's own."""
+        report = dict(vars(self.scheduler.stats))
+        cache = self.prefix_cache.stats
+        for name in ("queries", "hit_tokens", "prompt_tokens", "hit_rate"):
+            report[f"prefix_cache_{name}"] = getattr(cache, name)
+        report["num_free_blocks"] = self.manager.min_free_blocks()
+        report["lookahead_steps"] = self.lookahead_steps
+        return report
 
     # ------------------------------------------------------------------ text and finishing
     def _decode(self, ids: list[int]) -> str:
         return self.tokenizer.decode(ids, skip_special_tokens=True)
 
-    def _text_step(self, seq: Sequence, state: _TextState) -> str:
-        """Incremental detokenisation; text that ends in U+FFFD is an unfinished multi-token
-        character and is held back (llm_engine.py:187-198)."""
-        ids = seq.output_token_ids
-        new_text = self._decode(ids[state.prefix_offset:])
-        if new_text.endswith("\ufffd"):
-            return ""
-        prefix_text = self._decode(ids[state.prefix_offset:state.read_offset])
-        state.prefix_offset, state.read_offset = state.read_offset, len(ids)
-        return new_text[len(prefix_text):]
+    def _ends_with_a_stop_token(self, seq: Sequence) -> bool:
+        params, token = seq.sampling_params, seq.output_token_ids[-1]
+        return token in params.stop_token_ids or (token in self._eos_ids and not params.ignore_eos)
+
+    def _is_out_of_room(self, seq: Sequence) -> bool:
+        return (len(seq.output_token_ids) >= seq.sampling_params.max_tokens
+                or len(seq) >= self.cfg.model.max_model_len)
 
     def _process(self, seq: Sequence) -> RequestOutput:
-        """Finish rules (llm_engine.py:200-242): a stop token (EOS unless ignore_eos, or one of
-        stop_token_ids) stays in the ids and adds no text; a stop string cuts the text; then
-        max_tokens and max_model_len give "length"."""
-        params = seq.sampling_params
-        state = self._text[seq.seq_id]
-        token = seq.output_token_ids[-1]
-        reason = None
-        delta = ""
-        if (not params.ignore_eos and token in self._eos_ids) or token in params.stop_token_ids:
-            reason = "stop"
-        elif self.tokenizer is not None:
-            delta = self._text_step(seq, state)
-            candidate = state.text + delta
-            hits = [pos for pos in (candidate.find(s) for s in params.stop) if pos >= 0]
-            if hits:
-                candidate = candidate[: min(hits)]
-                delta = candidate[len(state.text):] if len(candidate) > len(state.text) else ""
-                reason = "stop"
-            state.text = candidate
-        if reason is None and (
-            len(seq.output_token_ids) >= params.max_tokens or len(seq) >= self.cfg.model.max_model_len
-        ):
-            reason = "length"
-        if reason == "stop":
+        """What the request's newest token means for it (llm_engine.py:200-242). The rules, in
+        order: a stop token (end of sequence unless ``ignore_eos``, or one of ``stop_token_ids``)
+        ends it, stays in the ids and adds no text; otherwise the token's text is added and a
+        stop string in it ends the request with the text cut there; otherwise ``max_tokens`` or
+        the model length end it with reason "length"."""
+        text = self._text[seq.seq_id]
+        added = ""
+        if self._ends_with_a_stop_token(seq):
             seq.status = SequenceStatus.FINISHED_STOPPED
-        elif reason == "length":
-            seq.status = SequenceStatus.FINISHED_LENGTH
+        else:
+            stopped = False
+            if self.tokenizer is not None:
+                added, stopped = text.accept(text.grow(self._decode, seq.output_token_ids), seq.sampling_params.stop)
+            if stopped:
+                seq.status = SequenceStatus.FINISHED_STOPPED
+            elif self._is_out_of_room(seq):
+                seq.status = SequenceStatus.FINISHED_LENGTH
+        reasons = {SequenceStatus.FINISHED_STOPPED: "stop", SequenceStatus.FINISHED_LENGTH: "length"}
         return RequestOutput(
             request_id=seq.seq_id,
             prompt_token_ids=seq.prompt_token_ids,  # shared, not copied: a prompt never changes
             token_ids=list(seq.output_token_ids),
-            text=state.text,
+            text=text.shown,
             finished=seq.is_finished(),
-            finish_reason=reason,
+            finish_reason=reasons.get(seq.status),
             num_cached_tokens=seq.num_cached_tokens,
             num_prompt_tokens=len(seq.prompt_token_ids),
             num_generated_tokens=len(seq.output_token_ids),
-            delta_text=delta,
+            delta_text=added,
         )

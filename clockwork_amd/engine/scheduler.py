@@ -26,6 +26,7 @@ error raised by the engine.
 
 from __future__ import annotations
 
+from collections import deque
 from dataclasses import dataclass, field
 from typing import Optional
 
@@ -113,16 +114,20 @@ class Scheduler:
         self.manager.free(seq.seq_id)
 
     def _preempt(self, seq: Sequence) -> None:
+        """Take a running request's pages away. It keeps its tokens, loses its progress and waits
+        again, ahead of every request that was never admitted and, among the preempted ones, in
+        order of arrival (clockwork/scheduler/scheduler.py:79-96)."""
         self._release(seq)
         seq.reset_for_recompute()
         seq.num_cached_tokens = 0
         seq.status = SequenceStatus.PREEMPTED
-        key = self._priority(seq)
-        i = 0
-        while (i < len(self.waiting) and self.waiting[i].status is SequenceStatus.PREEMPTED
-               and self._priority(self.waiting[i]) < key):
-            i += 1
-        self.waiting.insert(i, seq)
+        mine = self._priority(seq)
+        ahead = 0
+        for other in self.waiting:
+            if other.status is not SequenceStatus.PREEMPTED or self._priority(other) > mine:
+                break
+            ahead += 1
+        self.waiting.insert(ahead, seq)
         self.stats.num_preempted_total += 1
         self.version += 1
 
@@ -139,37 +144,43 @@ class Scheduler:
             n = min(n, self.cfg.max_prefill_chunk)
         return n
 
+    def _make_room(self, seq: Sequence, start: int, n: int, unserved: deque, out: SchedulerOutput) -> bool:
+        """Free pages until ``seq`` can write positions [start, start + n): idle blocks of the
+        prefix cache first; then running requests are preempted, the latest arrival among those
+        not served yet in this step first, the request itself when no other is left
+        (scheduler.py:98-113). False if ``seq`` itself had to go."""
+        while not self.manager.can_extend(seq.seq_id, start, start + n):
+            if self._evict_for(1):
+                continue
+            victim = unserved.pop() if unserved else seq
+            self._preempt(victim)
+            out.preempted.append(victim)
+            if victim is seq:
+                return False
+        return True
+
     def _serve_running(self, out: SchedulerOutput) -> None:
-        ordered = sorted(self.running, key=self._priority)
+        """Every running request, in order of arrival, gets its next tokens: one if it decodes
+        (always served), else a portion of what it still has to run, as the budget allows."""
+        unserved = deque(sorted(self.running, key=self._priority))
         budget = self.cfg.max_num_batched_tokens
-        served: list[Sequence] = []
-        while ordered:
-            seq = ordered.pop(0)
+        kept: list[Sequence] = []
+        while unserved:
+            seq = unserved.popleft()
             remaining = seq.num_uncomputed_tokens()
-            if remaining == 1:
-                n = 1  # decoding requests are always served (scheduler.py:98-118)
-            else:
-                n = self._chunk(remaining, budget - out.num_batched_tokens)
-                if not self.cfg.enable_chunked_prefill and n < remaining:
-                    n = 0
-                if n <= 0:
-                    served.append(seq)  # stays running, contributes nothing this step
-                    continue
+            n = 1 if remaining == 1 else self._chunk(remaining, budget - out.num_batched_tokens)
+            if remaining > 1 and not self.cfg.enable_chunked_prefill and n < remaining:
+                n = 0  # a prompt runs whole or not at all
+            if n <= 0:
+                kept.append(seq)  # stays running, contributes nothing this step
+                continue
             start = seq.num_computed_tokens
-            while not self.manager.can_extend(seq.seq_id, start, start + n):
-                if self._evict_for(1):
-                    continue
-                victim = ordered.pop() if ordered else seq
-                self._preempt(victim)
-                out.preempted.append(victim)
-                if victim is seq:
-                    break
-            if seq.status is SequenceStatus.PREEMPTED:
+            if not self._make_room(seq, start, n, unserved, out):
                 continue
             out.copies += self.manager.extend(seq.seq_id, start, start + n)
-            served.append(seq)
+            kept.append(seq)
             self._emit(out, seq, start, n)
-        self.running = served
+        self.running = kept
 
     def _emit(self, out: SchedulerOutput, seq: Sequence, start: int, n: int, admitted: bool = False) -> None:
         samples = start + n == len(seq)
@@ -216,12 +227,10 @@ class Scheduler:
     def schedule(self) -> SchedulerOutput:
         out = SchedulerOutput()
         self._serve_running(out)
-        while self.waiting and len(self.running) < self.cfg.max_num_seqs:
-            seq = self.waiting[0]
-            if not self._try_admit(seq, out):
-                break
-            self.waiting.pop(0)
-            self.running.append(seq)
+        # the head of the queue or nobody: a request that does not fit holds back those behind it
+        while (self.waiting and len(self.running) < self.cfg.max_num_seqs
+               and self._try_admit(self.waiting[0], out)):
+            self.running.append(self.waiting.pop(0))
         if not out.is_empty():
             self.stats.num_scheduled_batches += 1
         self._refresh()

@@ -31,10 +31,12 @@ def test_pool_refuses_double_free_and_bad_ids():
     pool = PagePool(4, BS)
     page = pool.take()
     pool.drop(page)
-    with pytest.raises(ValueError, match="not allocated"):
+    with pytest.raises(ValueError, match="has no holder"):
         pool.drop(page)
-    with pytest.raises(ValueError, match="out of range"):
+    with pytest.raises(ValueError, match="outside this pool"):
         pool.share(4)
+    with pytest.raises(ValueError, match="one at a time"):
+        pool.hold(pool.take(), 2)
     with pytest.raises(ValueError):
         PagePool(0, BS)
 
