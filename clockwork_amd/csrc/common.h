@@ -68,6 +68,18 @@ __device__ __forceinline__ float cw_wave_max(float v) {
   return v;
 }
 
+// A workgroup barrier for data that waves hand each other through LDS: LDS writes made before it
+// are visible after it. __syncthreads() also orders global memory, and for that it waits until
+// every global store the wave has issued is done; the counter it waits on counts loads as well, in
+// order, so a wave that has prefetched its next tile and then stored a result waits at the barrier
+// for the prefetch too, and the loop loses the overlap it was built for. Kernels whose global
+// stores nobody in the workgroup reads back use this barrier in such loops.
+__device__ __forceinline__ void cw_lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 static inline int cw_launch_status() {
   return hipGetLastError() == hipSuccess ? CW_OK : CW_ERR_LAUNCH;
 }

@@ -348,45 +348,40 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
 #pragma unroll
       for (int e = 0; e < 8; ++e) xf[u][0][e] = (__bf16)(wv[u][e] * (float)(__bf16)(v[u][e] * inv));
   } else {
+    // Token tile by token tile, a row's k-steps one after the other: a lane's 16 bytes of step u
+    // and of step u + 1 are halves of one 128-byte line, and asked for back to back the second
+    // finds the line in the compute unit's own cache (step by step over all token tiles, every
+    // finds the line in the compute unit's own cache. The loads are unconditional, from clamped
+    // addresses; what lies past M or K is zeroed afterwards. (Every workgroup pulls all of x from
+    // L2: with 64 rows that is 44 MB beside the 55 MB of a gate/up matrix, and the two share what
+    // L2 delivers, about 5.7 TB/s: 13 us with 8 rows, 19 us with 64.)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const bf16_t* xrow = X + (int64_t)min(mt * 16 + r, M - 1) * ldx;
+#pragma unroll
+      for (int u = 0; u < SPW; ++u)
+        xf[u][mt] = *reinterpret_cast<const bf16x8_t*>(xrow + koff[u]);
+    }
 #pragma unroll
     for (int u = 0; u < SPW; ++u) {
-      const int k = ((blockIdx.y * WAVES + wave) * SPW + u) * 32 + s * 8;
-      const bool kok = k + 8 <= K;
+      const bool kok = ((blockIdx.y * WAVES + wave) * SPW + u) * 32 + s * 8 + 8 <= K;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
+      for (int mt = 0; mt < MT; ++mt)
+        if (!kok || mt * 16 + r >= M) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) xf[u][mt][e] = (__bf16)0.0f;
-        if (kok && mt * 16 + r < M) xf[u][mt] = *reinterpret_cast<const bf16x8_t*>(X + (int64_t)(mt * 16 + r) * ldx + k);
-      }
+          for (int e = 0; e < 8; ++e) xf[u][mt][e] = (__bf16)0.0f;
+        }
     }
   }
-  int buf = 0;
-  for (; tile < n_tiles; tile += gridDim.x) {
-    const bf16_t* w_next = wrow(min(tile + (int)gridDim.x, n_tiles - 1));
-    f32x4_t acc[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      // the chunk after this one: of this tile, or the first of the workgroup's next tile
-#pragma unroll
-      for (int u = 0; u < CH; ++u)
-        nxt[u] = *reinterpret_cast<const bf16x8_t*>((c + 1 < NC ? w_tile + koff[(c + 1) * CH + u] : w_next + koff[u]));
-#pragma unroll
-      for (int u = 0; u < CH; ++u)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], xf[c * CH + u][mt], acc[mt], 0, 0, 0);
-#pragma unroll
-      for (int u = 0; u < CH; ++u) cur[u] = nxt[u];
-    }
-    w_tile = w_next;
+  // what the waves' partial tiles of ``tile`` (in red[buf]) become: summed over the waves, then
+  // stored as the mode says. One barrier before; a second after, when the buffer is not doubled.
+  auto finish_tile = [&](const f32x4_t (&acc)[MT], int tile, int buf) __attribute__((always_inline)) {
     // lane (r, s) holds weight rows 4s..4s+3 of token r of tile mt -> red[buf][wave][mt][token][row]:
     // one 16-byte store a lane, the lanes of a wave side by side (no bank is hit twice)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
       *reinterpret_cast<f32x4_t*>(&red[buf][wave][mt * 256 + r * 16 + 4 * s]) = acc[mt];
-    __syncthreads();
+    cw_lds_barrier();  // not __syncthreads(): the next tile's weights stay in flight across it
     if (MODE == 2) {
       if (threadIdx.x < MT * 128) {  // (token, j): the gate and the up value of output j are neighbours
         const int j = threadIdx.x & 7, m = threadIdx.x >> 3;
@@ -414,8 +409,70 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
         }
       }
     }
-    if (NBUF == 1) __syncthreads();
-    buf = (buf + 1) % NBUF;
+    if (NBUF == 1) cw_lds_barrier();
+  };
+  int buf = 0;
+  if constexpr (NC == 1) {
+    // A wave's whole share of a tile is one set of fragments. Two sets take turns, without a
+    // copy between them (a copy has to wait for the loads it copies): the loads of the tile
+    // after this one are issued before this tile's products and are waited for only when their
+    // own products begin, so they are in flight during the whole of this tile's products,
+    // reduction and stores. Past the last tile a valid address is read and dropped.
+    auto load_set = [&](bf16x8_t (&dst)[CH], int t) __attribute__((always_inline)) {
+      const bf16_t* w = wrow(min(t, n_tiles - 1));
+#pragma unroll
+      for (int u = 0; u < CH; ++u) dst[u] = *reinterpret_cast<const bf16x8_t*>(w + koff[u]);
+    };
+    auto products = [&](const bf16x8_t (&w)[CH], f32x4_t (&acc)[MT]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int u = 0; u < CH; ++u)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], xf[u][mt], acc[mt], 0, 0, 0);
+    };
+    const int stride = (int)gridDim.x;
+    while (tile < n_tiles) {
+      f32x4_t acc[MT];
+      load_set(nxt, tile + stride);
+      __builtin_amdgcn_sched_barrier(0);  // the loads stay in front of the products
+      products(cur, acc);
+      finish_tile(acc, tile, buf);
+      buf = (buf + 1) % NBUF;
+      tile += stride;
+      if (tile >= n_tiles) break;
+      load_set(cur, tile + stride);
+      __builtin_amdgcn_sched_barrier(0);
+      products(nxt, acc);
+      finish_tile(acc, tile, buf);
+      buf = (buf + 1) % NBUF;
+      tile += stride;
+    }
+  } else {
+    for (; tile < n_tiles; tile += gridDim.x) {
+      const bf16_t* w_next = wrow(min(tile + (int)gridDim.x, n_tiles - 1));
+      f32x4_t acc[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        // the chunk after this one: of this tile, or the first of the workgroup's next tile
+#pragma unroll
+        for (int u = 0; u < CH; ++u)
+          nxt[u] = *reinterpret_cast<const bf16x8_t*>((c + 1 < NC ? w_tile + koff[(c + 1) * CH + u] : w_next + koff[u]));
+#pragma unroll
+        for (int u = 0; u < CH; ++u)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], xf[c * CH + u][mt], acc[mt], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < CH; ++u) cur[u] = nxt[u];
+      }
+      w_tile = w_next;
+      finish_tile(acc, tile, buf);
+      buf = (buf + 1) % NBUF;
+    }
   }
 }
 
