@@ -838,6 +838,30 @@ def test_decode_attention_kernel_window_and_mixed_batch(window, fixed_ranges):
         at += q_len
 
 
+def test_decode_attention_many_requests_with_splits():
+    """Fifty requests of lengths from 1 to 400 keys with 5 to 7 splits each (many of them empty),
+    three launches in a row over the same pages."""
+    dtype = torch.bfloat16
+    nh, nkv, hd, bs = 12, 2, 128, 16
+    gen = torch.Generator().manual_seed(5)
+    ctx_lens = [int(c) for c in torch.randint(1, 400, (50,), generator=gen)]
+    num_blocks = sum(-(-c // bs) for c in ctx_lens) + 5
+    perm = torch.randperm(num_blocks, generator=gen).tolist()
+    tables, at = [], 0
+    for c in ctx_lens:
+        n = -(-c // bs)
+        tables.append(perm[at : at + n])
+        at += n
+    kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens, poison=float("nan"))
+    for launch in range(3):
+        qs = [torch.randn(1, nh, hd, device=DEV).to(dtype) for _ in ctx_lens]
+        out = _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, [1] * len(ctx_lens), kc, vc, qs, splits=5 + launch,
+                             decode_kernel=True, fixed_ranges=launch == 1)
+        for r in range(len(ctx_lens)):
+            want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5)
+            torch.testing.assert_close(out[r : r + 1].float().cpu(), want, **tol(dtype))
+
+
 def test_decode_attention_far_key_stands_out():
     nh, nkv, hd, bs = 12, 2, 128, 16
     ctx = 700
