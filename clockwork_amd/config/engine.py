@@ -12,8 +12,6 @@ from pathlib import Path
 
 import yaml
 
-_DTYPES = ("float32", "bfloat16")
-
 
 @dataclass
 class ModelConfig:
@@ -33,15 +31,17 @@ class ModelConfig:
     hip_products: bool = False
 
     def torch_dtype(self):
+        """The torch dtype of ``dtype``; the reference's float16 is named so that a user of it
+        knows why it is refused (clockwork/config.py:26-31)."""
         import torch
 
+        names = {"float32": torch.float32, "bfloat16": torch.bfloat16}
         if self.dtype == "float16":
-            raise ValueError(
-                "dtype 'float16' is not built in this engine; use 'bfloat16' or 'float32'"
-            )
-        if self.dtype not in _DTYPES:
-            raise ValueError(f"unknown dtype {self.dtype!r}, expected one of {_DTYPES}")
-        return getattr(torch, self.dtype)
+            raise ValueError("dtype 'float16' is not built in this engine; use 'bfloat16' or 'float32'")
+        try:
+            return names[self.dtype]
+        except KeyError:
+            raise ValueError(f"unknown dtype {self.dtype!r}, expected one of {tuple(names)}") from None
 
 
 @dataclass
@@ -78,30 +78,33 @@ class SchedulerConfig:
     lookahead: bool = True
 
 
-_SECTIONS = ("model", "cache", "scheduler")
-
-
 @dataclass
 class EngineConfig:
     model: ModelConfig
     cache: CacheConfig = field(default_factory=CacheConfig)
     scheduler: SchedulerConfig = field(default_factory=SchedulerConfig)
 
+    def sections(self) -> dict:
+        """Section name -> its dataclass instance, in the order a key is looked up."""
+        return {"model": self.model, "cache": self.cache, "scheduler": self.scheduler}
+
     @classmethod
     def from_yaml(cls, path: str | Path) -> "EngineConfig":
-        """Read sections ``model:``, ``cache:``, ``scheduler:`` (clockwork/config.py:57-68)."""
-        data = yaml.safe_load(Path(path).read_text(encoding="utf-8")) or {}
-        model = data.get("model")
-        if not isinstance(model, dict) or "model" not in model:
+        """A file with the sections ``model:`` (which must name the model), ``cache:`` and
+        ``scheduler:`` (clockwork/config.py:57-68). The reference's top-level
+        ``attention_backend`` key is accepted and ignored."""
+        loaded = yaml.safe_load(Path(path).read_text(encoding="utf-8"))
+        loaded = {} if loaded is None else dict(loaded)
+        loaded.pop("attention_backend", None)
+        model_section = loaded.pop("model", None)
+        if not (isinstance(model_section, dict) and "model" in model_section):
             raise ValueError(f"{path}: expected a top-level 'model' section naming the model")
-        unknown = sorted(set(data) - set(_SECTIONS) - {"attention_backend"})
-        if unknown:
-            raise ValueError(f"{path}: unknown top-level sections {unknown}")
-        return cls(
-            model=ModelConfig(**model),
-            cache=CacheConfig(**(data.get("cache") or {})),
-            scheduler=SchedulerConfig(**(data.get("scheduler") or {})),
-        )
+        kinds = {"cache": CacheConfig, "scheduler": SchedulerConfig}
+        strangers = sorted(set(loaded) - set(kinds))
+        if strangers:
+            raise ValueError(f"{path}: unknown top-level sections {strangers}")
+        rest = {name: kind(**(loaded.get(name) or {})) for name, kind in kinds.items()}
+        return cls(model=ModelConfig(**model_section), **rest)
 
     @classmethod
     def defaults(cls, model: str, **overrides) -> "EngineConfig":
@@ -112,25 +115,21 @@ class EngineConfig:
         return cfg
 
     def set(self, key: str, value) -> None:
-        """Set ``key`` on every section that has such a field; unknown keys are an error.
-
-        ``max_model_len`` lives on both the model and the scheduler section and
-        is set on both, as in the reference (clockwork/config.py:76-86).
-        """
-        targets = [
-            sub
-            for sub in (self.model, self.cache, self.scheduler)
-            if key in {f.name for f in fields(sub)}
-        ]
-        if not targets:
+        """Set ``key`` in every section that has a field of that name; a key that no section has
+        is an error. ``max_model_len`` is a field of the model and of the scheduler section and
+        changes in both, as in the reference (clockwork/config.py:76-86)."""
+        hits = 0
+        for section in self.sections().values():
+            if any(f.name == key for f in fields(section)):
+                setattr(section, key, value)
+                hits += 1
+        if hits == 0:
             raise ValueError(f"unknown config override {key!r}")
-        for sub in targets:
-            setattr(sub, key, value)
 
     def apply_overrides(self, pairs: list[str]) -> None:
         """``KEY=VALUE`` strings, the value read as YAML (scripts/serve.py:13-30)."""
         for pair in pairs:
-            if "=" not in pair:
+            key, sep, raw = pair.partition("=")
+            if not sep:
                 raise ValueError(f"override {pair!r} is not KEY=VALUE")
-            key, raw = pair.split("=", 1)
             self.set(key, yaml.safe_load(raw))

@@ -1,16 +1,19 @@
 """Per-request state shared by the scheduler, the cache manager and the engine.
 
-Same fields and meanings as the reference (clockwork/engine/sequence.py:10-96);
+Same fields and meanings as the reference (clockwork/engine/sequence.py:10-82);
 block tables live in the cache manager, keyed by ``seq_id``, because a request
-may hold one table per layer group.
+may hold one table per layer group. ``SamplingParams`` (sampling/params.py) and
+``RequestOutput`` (engine/outputs.py) can be imported from here as in the reference.
 """
 
 from __future__ import annotations
 
 import time
-from dataclasses import dataclass, field
 from enum import Enum
 from typing import Optional
+
+from clockwork_amd.engine.outputs import RequestOutput  # noqa: F401  (the reference keeps it in this module)
+from clockwork_amd.sampling.params import SamplingParams
 
 
 class SequenceStatus(Enum):
@@ -22,31 +25,8 @@ class SequenceStatus(Enum):
     FINISHED_ABORTED = "finished_aborted"
 
 
-_FINISHED = frozenset(
-    {
-        SequenceStatus.FINISHED_STOPPED,
-        SequenceStatus.FINISHED_LENGTH,
-        SequenceStatus.FINISHED_ABORTED,
-    }
-)
-
-
-@dataclass
-class SamplingParams:
-    """clockwork/engine/sequence.py:28-41. ``temperature == 0`` means greedy."""
-
-    max_tokens: int = 64
-    temperature: float = 0.0
-    top_p: float = 1.0
-    top_k: int = -1
-    stop: list[str] = field(default_factory=list)
-    stop_token_ids: list[int] = field(default_factory=list)
-    ignore_eos: bool = False
-    seed: Optional[int] = None
-
-    @property
-    def greedy(self) -> bool:
-        return self.temperature == 0.0
+# the three ways a request ends (stop token or string, length, abort)
+_FINISHED = frozenset(status for status in SequenceStatus if status.name.startswith("FINISHED_"))
 
 
 class Sequence:
@@ -111,19 +91,3 @@ class Sequence:
     def __repr__(self) -> str:
         return (f"<Sequence {self.seq_id} {self.status.value}: {self.num_computed_tokens} of {len(self)} "
                 f"tokens cached, {len(self.output_token_ids)} generated>")
-
-
-@dataclass
-class RequestOutput:
-    """clockwork/engine/sequence.py:85-96."""
-
-    request_id: str
-    prompt_token_ids: list[int]
-    token_ids: list[int]
-    text: str
-    finished: bool
-    finish_reason: Optional[str]
-    num_cached_tokens: int
-    num_prompt_tokens: int
-    num_generated_tokens: int
-    delta_text: str = ""

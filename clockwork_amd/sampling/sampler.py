@@ -10,13 +10,16 @@ again after a preemption. The kernels are in csrc/sampling.hip.
 
 from __future__ import annotations
 
+from typing import TYPE_CHECKING
 from typing import Sequence as Seq
 
 import numpy as np
 import torch
 
 from clockwork_amd import ops
-from clockwork_amd.engine.sequence import Sequence
+
+if TYPE_CHECKING:
+    from clockwork_amd.engine.sequence import Sequence
 
 
 class Sampler:
