@@ -25,8 +25,8 @@ TINY_C = dict(
 # name -> (config, weight seed, cache block size)
 TINY_CONFIGS = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8), "C": (TINY_C, 5, 16)}
 
-# Sizes that none of the above pins: groups of 5, 7, 14 and 17 query heads (17: more than one
-# workgroup of the decode kernel takes), widths that are multiples of 2 only, a feed-forward of 7,
+# Sizes that none of the above pins: groups of 5, 7, 14, 17 and 66 query heads (17 and more: more than one
+# workgroup of the decode kernel takes), widths that are multiples of 2 only or odd, a feed-forward of 7,
 # pages of 4, 24 and 48 tokens, head sizes 32 to 256. name -> (config, weight seed, block size)
 ODD_CONFIGS = {
     "group14": (dict(model_type="qwen2", vocab_size=1001, hidden_size=66, head_dim=96, num_hidden_layers=2,
@@ -41,6 +41,13 @@ ODD_CONFIGS = {
     "group17": (dict(model_type="qwen2", vocab_size=2049, hidden_size=1032, head_dim=160, num_hidden_layers=1,
                      num_attention_heads=34, num_key_value_heads=2, intermediate_size=1000, rms_norm_eps=1e-6,
                      rope_theta=1000000.0, tie_word_embeddings=True), 14, 48),
+    # odd widths (rows that no 16-byte load fits) and a group of 66 query heads on one key head
+    "odd_widths": (dict(model_type="qwen2", vocab_size=33, hidden_size=65, head_dim=16, num_hidden_layers=2,
+                        num_attention_heads=3, num_key_value_heads=1, intermediate_size=9, rms_norm_eps=1e-6,
+                        rope_theta=10000.0, tie_word_embeddings=False), 15, 8),
+    "group66": (dict(model_type="qwen2", vocab_size=300, hidden_size=72, head_dim=32, num_hidden_layers=1,
+                     num_attention_heads=66, num_key_value_heads=1, intermediate_size=50, rms_norm_eps=1e-6,
+                     rope_theta=10000.0, tie_word_embeddings=False), 16, 16),
 }
 
 # Layers wide enough for the decode kernels that only take large shapes (the persistent
