@@ -1,7 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16] [--shape 1.5b]
-    python bench.py --workload mixed [--shape 7b] [--requests 64]
+    python bench.py --workload mixed|arrivals [--shape 7b] [--requests 64]
 
 Default workload: the layer sizes of Qwen2.5-1.5B with random weights (seed 2), bfloat16,
 8 requests that each hold a 2048-token prompt, context limit 4096, pages of 16 tokens. A
@@ -160,20 +160,26 @@ def run_mixed(args) -> dict:
     """A continuous batch through the whole engine: ``args.requests`` requests arrive at once,
     prompt lengths uniform in [128, 2048], half of them opening with the same 1024 tokens (the
     prefix cache serves those), prompts cut into portions under a budget of 2048 tokens a step
-    beside the decoding requests, 128 greedy tokens each."""
+    beside the decoding requests, 128 greedy tokens each.
+
+    ``--workload arrivals``: the requests come one by one instead, a new one every
+    ``--arrive-every`` steps, with short prompts (uniform in [32, 512], nothing shared): most
+    steps then hold one prompt beside the tokens of the requests that are decoding."""
     import torch
 
     from clockwork_amd.engine.llm_engine import LLMEngine
     from clockwork_amd.engine.sequence import SamplingParams
 
     n_req, out_len, shared = args.requests, 128, 1024
+    arrivals = args.workload == "arrivals"
+    shortest, longest = (32, 512) if arrivals else (128, PROMPT_LEN)
     cfg, runner = build_runner(args, prefix_cache=True, max_batch=n_req)
     vocab = runner.spec.vocab_size
     gen = torch.Generator().manual_seed(7)
     common = torch.randint(0, vocab, (shared,), generator=gen).tolist()
     prompts = []
     for i in range(n_req):
-        n = int(torch.randint(128, PROMPT_LEN + 1, (1,), generator=gen))
+        n = int(torch.randint(shortest, longest + 1, (1,), generator=gen))
         ids = torch.randint(0, vocab, (n,), generator=gen).tolist()
         if i % 2 == 1 and n > shared:
             ids[:shared] = common
@@ -187,16 +193,20 @@ def run_mixed(args) -> dict:
         _sync()
         before = engine.stats()
         t0 = time.perf_counter()
-        for i, ids in enumerate(prompts):
-            engine.add_request(f"{tag}-{i}", prompt_token_ids=ids, sampling_params=params)
-        first, done, steps = {}, 0, 0
-        while engine.has_unfinished_requests():
+        waiting = list(enumerate(prompts))
+        first, arrived, done, steps = {}, {}, 0, 0
+        while waiting or engine.has_unfinished_requests():
+            due = len(waiting) if not arrivals else int(steps % args.arrive_every == 0)
+            for i, ids in waiting[:due]:
+                engine.add_request(f"{tag}-{i}", prompt_token_ids=ids, sampling_params=params)
+                arrived[f"{tag}-{i}"] = time.perf_counter() - t0
+            del waiting[:due]
             outs = engine.step()
             steps += 1
             now = time.perf_counter() - t0
             for o in outs:
                 if o.num_generated_tokens >= 1 and o.request_id not in first:
-                    first[o.request_id] = now
+                    first[o.request_id] = now - arrived[o.request_id]
                 done += bool(o.finished)
         _sync()
         elapsed = time.perf_counter() - t0
@@ -205,11 +215,15 @@ def run_mixed(args) -> dict:
         return elapsed, steps, first, {k: after[k] - before[k] for k in ("total_cached_tokens", "num_preempted_total")}
 
     once("warm")  # graphs captured, library kernels chosen, prefix cache filled as in a running server
+    if arrivals:
+        once("warm2")  # a shape is captured when it comes the second time: steps of many shapes need two passes
     elapsed, steps, first, stats = once("run")
     n_prompt = sum(len(p) for p in prompts)
     ttft = sorted(first.values())
     return {
-        "metric": f"output tok/s, {SHAPES[args.shape][0]} shape, continuous batch of {n_req} requests",
+        "metric": f"output tok/s, {SHAPES[args.shape][0]} shape, "
+                  + (f"{n_req} requests arriving one every {args.arrive_every} steps" if arrivals
+                     else f"continuous batch of {n_req} requests"),
         "value": round(n_req * out_len / elapsed, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -232,7 +246,7 @@ def run_mixed(args) -> dict:
             "layers": args.layers,
             "layers_of_full_model": SHAPES[args.shape][1]["num_hidden_layers"],
             "requests": n_req,
-            "prompt_len": "uniform 128..2048, every second one shares its first 1024 tokens",
+            "prompt_len": "uniform 32..512" if arrivals else "uniform 128..2048, every second one shares its first 1024 tokens",
             "output_len": out_len,
             "token_budget": PROMPT_LEN,
             "seq_len": CONTEXT,
@@ -302,7 +316,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--no-tune", action="store_true", help="leave the matrix library's kernel choice at its default")
     ap.add_argument("--only-prefill", action="store_true", help="run the prefill alone: 2048 tokens, or --prompt-len tokens in portions of 2048")
-    ap.add_argument("--workload", default="decode", choices=("decode", "mixed"),
+    ap.add_argument("--arrive-every", type=int, default=4, help="--workload arrivals: steps between two requests")
+    ap.add_argument("--workload", default="decode", choices=("decode", "mixed", "arrivals"),
                     help="decode: the recorded benchmark; mixed: a continuous batch of --requests prompts of mixed lengths")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--peaks", action="store_true", help="measure a device copy and a large library product instead")
@@ -319,7 +334,7 @@ def main() -> int:
     if args.peaks:
         print(json.dumps(measure_peaks()))
         return 0
-    if args.workload == "mixed":
+    if args.workload in ("mixed", "arrivals"):
         print(json.dumps(run_mixed(args)))
         return 0
     cfg, runner = build_runner(args)

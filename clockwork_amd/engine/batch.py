@@ -399,3 +399,135 @@ class StaticPortionBatch:
         self.device_buf.copy_(self.host, non_blocking=True)
         self._sent = torch.cuda.Event()
         self._sent.record()
+
+
+class StaticMixedBatch:
+    """Single decoded tokens of up to ``decoders`` requests beside one request's portion of up to
+    ``portion`` tokens, with fixed shapes, for a captured HIP graph: the step that a short prompt
+    makes when it arrives among decoding requests, which the host's launches would otherwise bound.
+
+    Rows 0 .. decoders - 1 are the single tokens (request r in row r), the portion's tokens follow
+    from row ``decoders``; the portion is request number ``decoders``. Rows and requests that a step
+    does not fill are padding as in the two batches above: a single token 0 at position 0 of a
+    request without pages, and rows behind the portion's tokens that ``cu_q`` leaves out. Logits
+    are made for every single-token row and for the portion's last token; the caller picks what
+    was asked for. ``key_capacity``: the longest context among the decoding requests the graph is
+    planned for; ``typical_start``: where a portion of this class of steps begins.
+    """
+
+    def __init__(self, decoders: int, portion: int, key_capacity: int, typical_start: int, table_width: int,
+                 manager, device, prepare, num_compute_units: int, vocab_size: int) -> None:
+        self.decoders, self.portion = decoders, portion
+        self.vocab_size = vocab_size
+        self.table_width = table_width
+        self.block_size = manager.block_size
+        rows, requests = decoders + portion, decoders + 1
+        n_groups = len(manager.kv_groups)
+        offsets = {}
+        at = 0
+
+        def take(name, count):
+            nonlocal at
+            offsets[name] = (at, count)
+            at += -(-count // 4) * 4
+
+        take("token_ids", rows)
+        take("positions", rows)
+        for name in ("ctx_lens", "starts", "state_slots", "logit_rows"):
+            take(name, requests)
+        take("cu_q", requests + 1)
+        for g in range(n_groups):
+            take(f"slots{g}", rows)
+            take(f"table{g}", requests * table_width)
+        self._offsets = offsets
+        self.host = torch.zeros(at, dtype=torch.int32, pin_memory=True)
+        self.device_buf = torch.zeros(at, dtype=torch.int32, device=device)
+        self._np = self.host.numpy()
+
+        def view(name):
+            o, count = offsets[name]
+            return self.device_buf[o : o + count]
+
+        ctx = StepContext()
+        ctx.device = device
+        ctx.block_size = manager.block_size
+        ctx.num_tokens, ctx.num_requests, ctx.num_logit_rows = rows, requests, requests
+        ctx.token_ids, ctx.positions = view("token_ids"), view("positions")
+        ctx.ctx_lens, ctx.starts, ctx.state_slots = view("ctx_lens"), view("starts"), view("state_slots")
+        ctx.cu_q, ctx.logit_rows = view("cu_q"), view("logit_rows")
+        for g in range(n_groups):
+            ctx.slots.append(view(f"slots{g}"))
+            ctx.block_tables.append(view(f"table{g}").view(requests, table_width))
+        # what the parts' plans look at
+        ctx.h_q_lens = [1] * decoders + [portion]
+        ctx.h_ctx_lens = [key_capacity] * decoders + [typical_start + portion]
+        ctx.h_starts = [0] * decoders + [typical_start]
+        ctx.h_state_slots = [manager.idle_state_slot] * requests
+        ctx.seq_ids = [""] * requests
+        ctx.num_compute_units = num_compute_units
+        prepare(ctx)  # the parts' work items are the same every step: made once, outside the graph
+        self.ctx = ctx
+
+    def fill(self, singles: Sequence[StepEntry], portion: StepEntry, manager) -> None:
+        """This step's indices into the pinned buffer, then to the device. ``singles``: the
+        entries of one token each, in the order of their rows; ``portion``: the other entry."""
+        d, n = len(singles), len(portion.tokens)
+        D, width, bs = self.decoders, self.table_width, self.block_size
+        if d > D or not 0 < n <= self.portion:
+            raise ValueError(f"{d} single tokens and a portion of {n} for a batch of {D} and {self.portion}")
+        a = self._np
+        sent = getattr(self, "_sent", None)
+        if sent is not None:
+            sent.synchronize()  # the copy of the step before must have read the buffer
+
+        def region(name):
+            o, count = self._offsets[name]
+            return a[o : o + count]
+
+        ids = np.asarray(portion.tokens, dtype=np.int64)
+        if ids.shape != (n,) or ids.min() < 0 or ids.max() >= self.vocab_size:
+            raise ValueError(f"request {portion.seq_id}: a token id outside the vocabulary [0, {self.vocab_size})")
+        tok, pos = region("token_ids"), region("positions")
+        ctx_lens, starts, state = region("ctx_lens"), region("starts"), region("state_slots")
+        first = [e.start for e in singles]
+        tok[:] = 0
+        pos[:] = 0
+        tok[:d] = [e.tokens[0] for e in singles]
+        pos[:d] = first
+        tok[D : D + n] = ids
+        pos[D : D + n] = np.arange(portion.start, portion.start + n, dtype=np.int32)
+        ctx_lens[:d] = pos[:d] + 1
+        ctx_lens[d:D] = 1
+        ctx_lens[D] = portion.start + n
+        starts[:d] = first
+        starts[d:D] = 0
+        starts[D] = portion.start
+        state[:d] = [manager.state_slot(e.seq_id) for e in singles]
+        state[d:D] = manager.idle_state_slot
+        state[D] = manager.state_slot(portion.seq_id)
+        cu = region("cu_q")
+        cu[: D + 1] = np.arange(D + 1, dtype=np.int32)
+        cu[D + 1] = D + n
+        rows = region("logit_rows")
+        rows[:D] = np.arange(D, dtype=np.int32)
+        rows[D] = D + n - 1
+        for g in range(len(manager.kv_groups)):
+            slots = region(f"slots{g}")
+            table = region(f"table{g}").reshape(D + 1, width)
+            slots[:] = -1
+            table[:] = -1
+            for r, e in enumerate([*singles, portion]):
+                row = manager.block_table(e.seq_id, g)
+                if len(row) > width:
+                    raise ValueError(f"request {e.seq_id} holds {len(row)} pages, the graph was sized for {width}")
+                table[r if r < d else D, : len(row)] = row
+            for r, e in enumerate(singles):
+                page = manager.block_table(e.seq_id, g)[e.start // bs]
+                if page < 0:
+                    raise ValueError(f"request {e.seq_id}: position {e.start} lies in a page that was given back")
+                slots[r] = page * bs + e.start % bs
+            slots[D : D + n] = manager.slot_mapping(portion.seq_id, portion.start, portion.start + n, g)
+        self.ctx.seq_ids = [e.seq_id for e in singles] + [""] * (D - d) + [portion.seq_id]
+        self.device_buf.copy_(self.host, non_blocking=True)
+        self._sent = torch.cuda.Event()
+        self._sent.record()

@@ -23,6 +23,7 @@ from clockwork_amd.config.engine import EngineConfig
 from clockwork_amd.engine.graph_nodes import node_kinds, only_kernels
 from clockwork_amd.engine.batch import (
     StaticDecodeBatch,
+    StaticMixedBatch,
     StaticPortionBatch,
     StepEntry,
     build_context,
@@ -38,6 +39,9 @@ GRAPH_KEY_BUCKET = 512
 # a step that is one request's portion replays a graph captured for the token budget or for the
 # next of these sizes (a step of 65 to 500 tokens is otherwise bound by the host's launches)
 PORTION_GRAPH_SIZES = (128, 256, 384, 512)
+# a portion beside single decoded tokens is padded to the next of these (the small ones keep a step
+# of few tokens within the rows that the narrow products take)
+MIXED_PORTION_SIZES = (16, 32, 64, *PORTION_GRAPH_SIZES)
 # captured graphs kept at a time (each holds index buffers of its own): the least recently
 # replayed one goes when another shape is captured beyond this many
 GRAPH_LIMIT = 48
@@ -272,6 +276,70 @@ class ModelRunner:
         self.manager.release_behind_window(entry.seq_id, entry.start + n)
         return out if want else None
 
+    def _mixed_graph_step(self, entries: Sequence[StepEntry]):
+        """A step of single decoded tokens beside one request's portion of up to 512 tokens (a
+        short prompt that arrives among decoding requests, or a portion of a longer one) replays a
+        captured graph as well: padded to the next batch size and the next portion size, per
+        context bucket of the decoding requests and class of the portion. The first step of a
+        shape runs eagerly, the second is captured. Returns NotImplemented when the step has to
+        take the ordinary path."""
+        where = [i for i, e in enumerate(entries) if len(e.tokens) > 1]
+        if len(where) != 1:
+            return NotImplemented
+        portion = entries[where[0]]
+        singles = [e for e in entries if e is not portion]
+        n, d = len(portion.tokens), len(singles)
+        want = [int(w) for w in portion.want]
+        size = next((b for b in MIXED_PORTION_SIZES if b >= n), None)
+        limit = self._table_width * self.manager.block_size
+        if size is None or want not in ([], [n - 1]) or portion.start + n > limit:
+            return NotImplemented
+        longest = max(e.start + 1 for e in singles)
+        if longest > limit:
+            return NotImplemented
+        decoders = next(b for b in GRAPH_BATCH_SIZES if b >= d)
+        # the decoding requests' context in powers of two (it only sets how finely their keys are
+        # split): with two other sizes in the key, finer steps would make too many shapes
+        capacity = GRAPH_KEY_BUCKET
+        while capacity < longest:
+            capacity *= 2
+        shape = self.model.shape_class([1] * decoders + [size], [capacity] * decoders + [portion.start + size])
+        key = ("mixed", decoders, size, capacity, shape)
+        state = self._graphs.get(key)
+        if state is None:
+            self._graphs[key] = "seen"
+            return NotImplemented
+        if state == "eager":
+            return NotImplemented
+        for e in singles:
+            if not 0 <= int(e.tokens[0]) < self.spec.vocab_size:
+                raise ValueError(f"request {e.seq_id}: token id {e.tokens[0]} outside the vocabulary")
+            if any(w != 0 for w in e.want):
+                raise ValueError(f"request {e.seq_id}: wanted index outside its 1 token")
+        if state == "seen":
+            batch = StaticMixedBatch(decoders, size, capacity, portion.start, self._table_width, self.manager,
+                                     self.device, self.model.prepare, self.num_compute_units, self.spec.vocab_size)
+            batch.fill(singles, portion, self.manager)
+            torch.cuda.synchronize()
+            state = self._capture(key, batch)
+            if state is None:
+                return NotImplemented
+        self._graphs[key] = self._graphs.pop(key)  # most recently used last
+        batch, graph, out = state
+        batch.fill(singles, portion, self.manager)
+        graph.replay()
+        for e in entries:
+            self.manager.release_behind_window(e.seq_id, e.start + len(e.tokens))
+        # the graph's rows: the single tokens in their order, then the portion's last token
+        row_of = {id(e): r for r, e in enumerate(singles)}
+        row_of[id(portion)] = decoders
+        rows = [row_of[id(e)] for e in entries if len(e.want)]
+        if not rows:
+            return None
+        if rows == list(range(len(rows))):
+            return out[: len(rows)]
+        return out[torch.tensor(rows, device=self.device)]
+
     def _capture(self, key, batch):
         """Capture the model's step on ``batch`` (filled, its copy done) as the graph of ``key``.
         A graph that holds anything but kernel nodes is not kept (a library product may record a
@@ -290,6 +358,7 @@ class ModelRunner:
         graph.instantiate()
         if self._graph_pool is None:
             self._graph_pool = graph.pool()
+        self._graphs.pop(key, None)  # the newest entry: another one goes when there are too many
         state = self._graphs[key] = (batch, graph, out)
         self._drop_old_graphs()
         return state
@@ -375,6 +444,10 @@ class ModelRunner:
         if (self.use_graphs and len(entries) == 1
                 and len(entries[0].tokens) > ops.STREAM_MAX_ROWS):
             logits = self._portion_graph_step(entries[0])
+            if logits is not NotImplemented:
+                return logits
+        if self.use_graphs and 1 < len(entries) <= GRAPH_BATCH_SIZES[-1] + 1:
+            logits = self._mixed_graph_step(entries)
             if logits is not NotImplemented:
                 return logits
         ctx = build_context(entries, self.manager, self.device, self.spec.vocab_size)

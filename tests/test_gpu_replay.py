@@ -612,6 +612,69 @@ def test_short_prompts_replay_padded_graphs(model_dirs, dtype):
     _check(got_g, ref, dtype)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_single_tokens_beside_a_portion_replay_padded_graphs(model_dirs, name, dtype):
+    """Decoding requests beside one request's portion replay a graph captured for the next batch
+    size and the next portion size. Three, then five decoding requests (one joins after every
+    prompt, so the batch sizes 4 and 8 are used and left partly empty); prompts arrive one after the
+    other with lengths around the portion sizes, each in one step (its last token's logits wanted)
+    or in two (the first without logits), every decoding request's logits wanted in every step,
+    in an order of entries that puts the portion first, last or in the middle. NaN-poisoned pools.
+    Checked against a runner without graphs and against the plain implementation."""
+    from clockwork_amd.config.engine import EngineConfig
+    from clockwork_amd.engine.model_runner import ModelRunner
+
+    cfg, _, block_size = TINY_CONFIGS[name]
+    gen = torch.Generator().manual_seed(45)
+    vocab = cfg["vocab_size"]
+    toks = {f"d{i}": torch.randint(0, vocab, (n + 40,), generator=gen).tolist() for i, n in enumerate([33, 70, 9])}
+    at = {"d0": 33, "d1": 70, "d2": 9}
+    steps = [{"entries": [{"id": rid, "tokens": toks[rid][:n], "want": []}], "end": []} for rid, n in at.items()]
+    arrivals = [5, 5, 5, 16, 17, 30, 30, 64, 65, 100, 100, 128, 129, 200, 200, 2, 2, 2]
+    for i, n in enumerate(arrivals):
+        rid = f"p{i}"
+        toks[rid] = torch.randint(0, vocab, (n + 40,), generator=gen).tolist()
+        cuts = [n] if i % 3 else [n // 2, n - n // 2]
+        if min(cuts) < 2:
+            cuts = [n]
+        begin = 0
+        for c, size in enumerate(cuts):
+            singles = []
+            for d in sorted(at):
+                singles.append({"id": d, "tokens": toks[d][at[d] : at[d] + 1], "want": [0]})
+                at[d] += 1
+            portion = {"id": rid, "tokens": toks[rid][begin : begin + size], "want": [size - 1] if c == len(cuts) - 1 else []}
+            begin += size
+            where = (i + c) % (len(singles) + 1)
+            steps.append({"entries": singles[:where] + [portion] + singles[where:], "end": []})
+        if i in (3, 9):  # this prompt goes on decoding beside the others
+            at[rid] = n
+        else:
+            steps[-1]["end"] = [rid]
+    steps[-1]["end"] = steps[-1]["end"] + [d for d in at if d not in steps[-1]["end"]]
+
+    def runner(use_graphs):
+        ecfg = EngineConfig.defaults(
+            str(model_dirs[name]), dtype=dtype, block_size=block_size, num_blocks=160, enable_prefix_cache=False,
+            watermark=0.0, max_model_len=512,
+        )
+        return ModelRunner(ecfg, cache_fill=float("nan"), use_graphs=use_graphs)
+
+    with_graphs, eager = runner(True), runner(False)
+    got_g = replay.run_trace(with_graphs, [dict(s) for s in steps])
+    got_e = replay.run_trace(eager, [dict(s) for s in steps])
+    captured = sorted(k[1:3] for k, v in with_graphs._graphs.items() if isinstance(v, tuple) and k[0] == "mixed")
+    assert {(4, 16), (4, 32), (8, 128), (8, 256)} <= set(captured), f"mixed graphs captured: {captured}"
+    assert got_g.keys() == got_e.keys() and len(got_g) > 100
+    close = dict(rtol=2e-6, atol=2e-6) if dtype == "float32" else dict(rtol=2e-2, atol=2e-2)
+    for key in got_e:
+        torch.testing.assert_close(got_g[key], got_e[key], **close, msg=lambda m: f"padded graph differs from the eager step at {key}: {m}")
+    model = PlainQwen2(model_dirs[name])
+    ref = {k: model.logits(v) for k, v in toks.items()}
+    _check(got_g, ref, dtype)
+
+
 @pytest.mark.parametrize("tuned", [False, True])
 def test_wide_decode_batches_of_a_large_layer_replay_as_eager(tmp_path, tuned):
     """40 requests decoding together through one layer of the 7B shape: at this width some products
