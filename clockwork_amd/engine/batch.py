@@ -410,8 +410,8 @@ class StaticMixedBatch:
     from row ``decoders``; the portion is request number ``decoders``. Rows and requests that a step
     does not fill are padding as in the two batches above: a single token 0 at position 0 of a
     request without pages, and rows behind the portion's tokens that ``cu_q`` leaves out. Logits
-    are made for every single-token row and for the portion's last token; the caller picks what
-    was asked for. ``key_capacity``: the longest context among the decoding requests the graph is
+    are made for ``decoders + 1`` rows, which every step names anew (the wanted ones first, in the
+    caller's order). ``key_capacity``: the longest context among the decoding requests the graph is
     planned for; ``typical_start``: where a portion of this class of steps begins.
     """
 
@@ -468,9 +468,14 @@ class StaticMixedBatch:
         prepare(ctx)  # the parts' work items are the same every step: made once, outside the graph
         self.ctx = ctx
 
-    def fill(self, singles: Sequence[StepEntry], portion: StepEntry, manager) -> None:
+    def row_of_portion(self, num_tokens: int) -> int:
+        """The batch row of the last of the portion's ``num_tokens`` tokens."""
+        return self.decoders + num_tokens - 1
+
+    def fill(self, singles: Sequence[StepEntry], portion: StepEntry, manager, wanted_rows: Sequence[int]) -> None:
         """This step's indices into the pinned buffer, then to the device. ``singles``: the
-        entries of one token each, in the order of their rows; ``portion``: the other entry."""
+        entries of one token each, in the order of their rows; ``portion``: the other entry;
+        ``wanted_rows``: the batch rows whose logits the step makes first, in this order."""
         d, n = len(singles), len(portion.tokens)
         D, width, bs = self.decoders, self.table_width, self.block_size
         if d > D or not 0 < n <= self.portion:
@@ -508,9 +513,11 @@ class StaticMixedBatch:
         cu = region("cu_q")
         cu[: D + 1] = np.arange(D + 1, dtype=np.int32)
         cu[D + 1] = D + n
+        if len(wanted_rows) > D + 1 or any(not 0 <= r < D + n for r in wanted_rows):
+            raise ValueError("wanted rows outside the step's tokens")
         rows = region("logit_rows")
-        rows[:D] = np.arange(D, dtype=np.int32)
-        rows[D] = D + n - 1
+        rows[:] = 0
+        rows[: len(wanted_rows)] = wanted_rows
         for g in range(len(manager.kv_groups)):
             slots = region(f"slots{g}")
             table = region(f"table{g}").reshape(D + 1, width)

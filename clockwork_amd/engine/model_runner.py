@@ -316,29 +316,26 @@ class ModelRunner:
                 raise ValueError(f"request {e.seq_id}: token id {e.tokens[0]} outside the vocabulary")
             if any(w != 0 for w in e.want):
                 raise ValueError(f"request {e.seq_id}: wanted index outside its 1 token")
+        # the rows whose logits are wanted, in the order of the entries: single token r is row r of
+        # the batch, the portion's tokens follow the (padded) single tokens
+        row_of = {id(e): r for r, e in enumerate(singles)}
+        row_of[id(portion)] = decoders + n - 1
+        wanted_rows = [row_of[id(e)] for e in entries if len(e.want)]
         if state == "seen":
             batch = StaticMixedBatch(decoders, size, capacity, portion.start, self._table_width, self.manager,
                                      self.device, self.model.prepare, self.num_compute_units, self.spec.vocab_size)
-            batch.fill(singles, portion, self.manager)
+            batch.fill(singles, portion, self.manager, wanted_rows)
             torch.cuda.synchronize()
             state = self._capture(key, batch)
             if state is None:
                 return NotImplemented
         self._graphs[key] = self._graphs.pop(key)  # most recently used last
         batch, graph, out = state
-        batch.fill(singles, portion, self.manager)
+        batch.fill(singles, portion, self.manager, wanted_rows)
         graph.replay()
         for e in entries:
             self.manager.release_behind_window(e.seq_id, e.start + len(e.tokens))
-        # the graph's rows: the single tokens in their order, then the portion's last token
-        row_of = {id(e): r for r, e in enumerate(singles)}
-        row_of[id(portion)] = decoders
-        rows = [row_of[id(e)] for e in entries if len(e.want)]
-        if not rows:
-            return None
-        if rows == list(range(len(rows))):
-            return out[: len(rows)]
-        return out[torch.tensor(rows, device=self.device)]
+        return out[: len(wanted_rows)] if wanted_rows else None
 
     def _capture(self, key, batch):
         """Capture the model's step on ``batch`` (filled, its copy done) as the graph of ``key``.
