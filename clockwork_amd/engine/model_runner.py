@@ -38,10 +38,10 @@ GRAPH_BATCH_SIZES = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)
 GRAPH_KEY_BUCKET = 512
 # a step that is one request's portion replays a graph captured for the token budget or for the
 # next of these sizes (a step of 65 to 500 tokens is otherwise bound by the host's launches)
-PORTION_GRAPH_SIZES = (128, 256, 384, 512)
-# a portion beside single decoded tokens is padded to the next of these (the small ones keep a step
-# of few tokens within the rows that the narrow products take)
-MIXED_PORTION_SIZES = (16, 32, 64, *PORTION_GRAPH_SIZES)
+PORTION_GRAPH_SIZES = (16, 32, 64, 128, 256, 384, 512)
+# the rows that the narrow products take in one, two or four tiles of tokens: a step of single
+# tokens beside a short portion is padded to the next of these in all, if it fits one
+NARROW_STEP_ROWS = (16, 32, 64)
 # captured graphs kept at a time (each holds index buffers of its own): the least recently
 # replayed one goes when another shape is captured beyond this many
 GRAPH_LIMIT = 48
@@ -241,8 +241,9 @@ class ModelRunner:
 
     def _portion_graph_step(self, entry: StepEntry):
         """A step that is one portion of one request, of the token budget (what a long prompt's
-        prefill is made of) or of up to 512 tokens (a short prompt), replays a captured graph as
-        the decode steps do: the first step of a shape runs eagerly, the second is captured.
+        prefill is made of) or of up to 512 tokens (a short prompt, the end of a long one), replays
+        a captured graph as the decode steps do, padded to the next of a few sizes: the first step
+        of a shape runs eagerly, the second is captured.
         Returns NotImplemented when the step has to take the ordinary path."""
         n = len(entry.tokens)
         want = [int(w) for w in entry.want]
@@ -279,7 +280,8 @@ class ModelRunner:
     def _mixed_graph_step(self, entries: Sequence[StepEntry]):
         """A step of single decoded tokens beside one request's portion of up to 512 tokens (a
         short prompt that arrives among decoding requests, or a portion of a longer one) replays a
-        captured graph as well: padded to the next batch size and the next portion size, per
+        captured graph as well: padded to the next batch size and the next portion size (so that
+        a step of up to 64 rows in all keeps to the 16, 32 or 64 rows of the narrow products), per
         context bucket of the decoding requests and class of the portion. The first step of a
         shape runs eagerly, the second is captured. Returns NotImplemented when the step has to
         take the ordinary path."""
@@ -290,14 +292,15 @@ class ModelRunner:
         singles = [e for e in entries if e is not portion]
         n, d = len(portion.tokens), len(singles)
         want = [int(w) for w in portion.want]
-        size = next((b for b in MIXED_PORTION_SIZES if b >= n), None)
+        decoders = next(b for b in GRAPH_BATCH_SIZES if b >= d)
+        rows = next((t for t in NARROW_STEP_ROWS if decoders + n <= t), None)
+        size = rows - decoders if rows else next((b for b in PORTION_GRAPH_SIZES if b >= max(n, NARROW_STEP_ROWS[-1])), None)
         limit = self._table_width * self.manager.block_size
         if size is None or want not in ([], [n - 1]) or portion.start + n > limit:
             return NotImplemented
         longest = max(e.start + 1 for e in singles)
         if longest > limit:
             return NotImplemented
-        decoders = next(b for b in GRAPH_BATCH_SIZES if b >= d)
         # the decoding requests' context in powers of two (it only sets how finely their keys are
         # split): with two other sizes in the key, finer steps would make too many shapes
         capacity = GRAPH_KEY_BUCKET
@@ -438,8 +441,7 @@ class ModelRunner:
             logits = self._graph_step(entries)
             if logits is not NotImplemented:
                 return logits
-        if (self.use_graphs and len(entries) == 1
-                and len(entries[0].tokens) > ops.STREAM_MAX_ROWS):
+        if self.use_graphs and len(entries) == 1 and len(entries[0].tokens) > 1:
             logits = self._portion_graph_step(entries[0])
             if logits is not NotImplemented:
                 return logits
