@@ -1,8 +1,8 @@
 // Matrix products y = x * W^T (+ bias) for gfx950, W stored [N, K] row-major as checkpoints
 // hold it.
 //  * cw_gemm_f32: true float32 (VALU FMA, float32 operands and accumulation, no reduced-precision
-//    matrix mode). The K loop of one output element runs in the same order whatever M is, so a
-//    row's result does not depend on what else is in the batch.
+//    matrix mode). The order in which the products of one output element are summed depends on N
+//    and K alone, never on M, so a row's result does not depend on what else is in the batch.
 #include "common.h"
 
 #define GT_BM 64
@@ -10,37 +10,49 @@
 #define GT_BK 16
 
 // C[M, N] = A[M, K] * W[N, K]^T + bias[N]. 256 threads, each a 4x4 tile of a 64x64 block.
+// K is summed in ``splits`` parts of k_per_split values (a multiple of 16), and the parts in their
+// order: ((p_0 + p_1) + ...) + bias. gridDim.z == 1: a block does so by itself. gridDim.z ==
+// splits: block z makes part z alone and writes it to C + z * part_stride (no bias), and
+// gemm_f32_sum_kernel adds the parts up in the same order, so both ways give the same bits.
+// ONE_PART: a block makes one part (gridDim.z == splits, or there is only one part).
+template <bool ONE_PART>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ A, int64_t lda,
                                                        const float* __restrict__ W,
                                                        const float* __restrict__ bias,
                                                        float* __restrict__ C, int64_t ldc, int M,
-                                                       int N, int K) {
+                                                       int N, int K, int splits, int k_per_split,
+                                                       int64_t part_stride) {
   __shared__ float As[GT_BK][GT_BM + 4];
   __shared__ float Ws[GT_BK][GT_BN + 4];
   const int tid = threadIdx.x;
   const int tx = tid & 15, ty = tid >> 4;
   const int m0 = blockIdx.y * GT_BM, n0 = blockIdx.x * GT_BN;
+  const bool parallel = gridDim.z > 1;  // part blockIdx.z of several
+  const int z_first = ONE_PART ? blockIdx.z : 0, z_last = ONE_PART ? blockIdx.z : splits - 1;
+  float total[4][4];
+  // each thread loads 4 elements of A and 4 of W per K step: row = tid / 4, k = (tid % 4) * 4 .. +3
+  const int lr = tid >> 2, lk = (tid & 3) * 4;
+  const bool k_vec_ok = (K % 4 == 0) && (lda % 4 == 0);
+  for (int z = z_first; z <= z_last; ++z) {
+  const int k_begin = z * k_per_split;
+  const int k_end = min(K, k_begin + k_per_split);
   float acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
-
-  // each thread loads 4 elements of A and 4 of W per K step: row = tid / 4, k = (tid % 4) * 4 .. +3
-  const int lr = tid >> 2, lk = (tid & 3) * 4;
-  const bool k_vec_ok = (K % 4 == 0) && (lda % 4 == 0);
-  for (int k0 = 0; k0 < K; k0 += GT_BK) {
+  for (int k0 = k_begin; k0 < k_end; k0 += GT_BK) {
     {
       const int m = m0 + lr, k = k0 + lk;
       float v[4] = {0.f, 0.f, 0.f, 0.f};
       if (m < M) {
         const float* p = A + (int64_t)m * lda + k;
-        if (k_vec_ok && k + 3 < K) {
+        if (k_vec_ok && k + 3 < k_end) {
           const float4 q = *reinterpret_cast<const float4*>(p);
           v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
         } else {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) if (k + j < K) v[j] = p[j];
+          for (int j = 0; j < 4; ++j) if (k + j < k_end) v[j] = p[j];
         }
       }
 #pragma unroll
@@ -51,12 +63,12 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
       float v[4] = {0.f, 0.f, 0.f, 0.f};
       if (n < N) {
         const float* p = W + (int64_t)n * K + k;
-        if (K % 4 == 0 && k + 3 < K) {
+        if (K % 4 == 0 && k + 3 < k_end) {
           const float4 q = *reinterpret_cast<const float4*>(p);
           v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
         } else {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) if (k + j < K) v[j] = p[j];
+          for (int j = 0; j < 4; ++j) if (k + j < k_end) v[j] = p[j];
         }
       }
 #pragma unroll
@@ -88,25 +100,90 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
     __syncthreads();
   }
 #pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) total[i][j] = (ONE_PART || z == z_first) ? acc[i][j] : total[i][j] + acc[i][j];
+  }
+  float* out = parallel ? C + (int64_t)blockIdx.z * part_stride : C;
+#pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int m = m0 + ty * 4 + i;
     if (m >= M) continue;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
-      if (n < N) C[(int64_t)m * ldc + n] = acc[i][j] + (bias ? bias[n] : 0.0f);
+      if (n < N) out[(int64_t)m * ldc + n] = total[i][j] + (bias && !parallel ? bias[n] : 0.0f);
     }
   }
 }
 
+// C[m, n] = ((p_0 + p_1) + ... + p_{splits-1}) + bias[n] over the partial sums p_z[m, n] (rows of N
+// floats, part_stride floats between two splits): always in the order of the splits.
+__global__ __launch_bounds__(256) void gemm_f32_sum_kernel(const float* __restrict__ parts, int splits,
+                                                           int64_t part_stride, const float* __restrict__ bias,
+                                                           float* __restrict__ C, int64_t ldc, int rows, int N) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)rows * N) return;
+  const int m = (int)(idx / N), n = (int)(idx - (int64_t)m * N);
+  float total = parts[idx];
+  for (int z = 1; z < splits; ++z) total += parts[z * part_stride + idx];
+  C[(int64_t)m * ldc + n] = total + (bias ? bias[n] : 0.0f);
+}
+
+// Up to this many rows of x the parts of K are made by blocks of their own (beyond, there are
+// blocks enough without, and a block sums its parts itself).
+#define GT_SPLIT_ROWS 256
+
+// How the float32 product cuts K for an [N, K] weight matrix: a narrow output (24 blocks of 64
+// columns for a width of 1536) with few rows of x would leave most compute units without work and
+// stream the matrix through the few that have some, so K is cut until there are about 512 blocks
+// per 64 rows, with at least 256 values of K each. A function of N and K alone: the order of the
+// sums must not depend on how many rows the step has.
+static void gemm_f32_plan(int N, int K, int* splits, int* k_per_split) {
+  const int col_blocks = (N + GT_BN - 1) / GT_BN;
+  int s = (512 + col_blocks / 2) / col_blocks;
+  if (s > K / 256) s = K / 256;
+  if (s < 1) s = 1;
+  const int per = ((K + s - 1) / s + GT_BK - 1) / GT_BK * GT_BK;
+  *k_per_split = per;
+  *splits = (K + per - 1) / per;
+}
+
+// Floats of workspace cw_gemm_f32 needs for this product (0: none).
+CW_EXPORT int64_t cw_gemm_f32_workspace_floats(int M, int N, int K) {
+  int splits, per;
+  if (M <= 0 || M > GT_SPLIT_ROWS || N <= 0 || K <= 0) return 0;
+  gemm_f32_plan(N, K, &splits, &per);
+  return splits <= 1 ? 0 : (int64_t)splits * M * N;
+}
+
 CW_EXPORT int cw_gemm_f32(const float* A, int64_t lda, const float* W, const float* bias, float* C,
-                          int64_t ldc, int M, int N, int K, hipStream_t stream) {
+                          int64_t ldc, int M, int N, int K, float* workspace, int64_t workspace_floats,
+                          hipStream_t stream) {
   if (M < 0 || N <= 0 || K <= 0 || lda < K || ldc < N) return CW_ERR_ARG;
   if (M == 0) return CW_OK;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return CW_ERR_ARG;
-  dim3 grid((N + GT_BN - 1) / GT_BN, (M + GT_BM - 1) / GT_BM), block(256);
+  int splits, per;
+  gemm_f32_plan(N, K, &splits, &per);
+  const dim3 block(256);
+  dim3 grid((N + GT_BN - 1) / GT_BN, (M + GT_BM - 1) / GT_BM);
   if (grid.y > 65535) return CW_ERR_SIZE;
-  hipLaunchKernelGGL(gemm_f32_kernel, grid, block, 0, stream, A, lda, W, bias, C, ldc, M, N, K);
+  if (splits <= 1) {
+    hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, block, 0, stream, A, lda, W, bias, C, ldc, M, N, K, 1, per, (int64_t)0);
+    return cw_launch_status();
+  }
+  if (M > GT_SPLIT_ROWS) {
+    hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, block, 0, stream, A, lda, W, bias, C, ldc, M, N, K, splits, per,
+                       (int64_t)0);
+    return cw_launch_status();
+  }
+  const int64_t part_stride = (int64_t)M * N;
+  if (workspace == nullptr || workspace_floats < splits * part_stride) return CW_ERR_ARG;
+  grid.z = splits;
+  hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, block, 0, stream, A, lda, W, nullptr, workspace, (int64_t)N, M, N, K,
+                     splits, per, part_stride);
+  hipLaunchKernelGGL(gemm_f32_sum_kernel, dim3((unsigned)((part_stride + 255) / 256)), block, 0, stream, workspace,
+                     splits, part_stride, bias, C, ldc, M, N);
   return cw_launch_status();
 }
 

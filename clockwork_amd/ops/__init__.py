@@ -98,7 +98,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_bf16_to_f32": [P, P, L, P],
         },
         "gemm": {
-            "cw_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
+            "cw_gemm_f32": [P, L, P, P, P, L, I, I, I, P, L, P],
+            "cw_gemm_f32_workspace_floats": [I, I, I],
             "cw_gemm_bf16_skinny": [I, P, L, P, P, L, I, I, I, P],
             "cw_gemm_bf16_skinny_ksplits": [I, I, I],
             "cw_gemm_bf16_skinny_fast": [I, I, I, I],
@@ -388,7 +389,12 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
         if bias is not None:
             if not (bias.dtype == torch.float32 and bias.numel() == N):
                 raise KernelError("bias must be float32 [N]")
-        _check(_load("gemm").cw_gemm_f32(_ptr(x), K, _ptr(weight), _ptr(bias), _ptr(out), N, M, N, K, _stream()), "gemm_f32")
+        lib = _load("gemm")
+        # a narrow output with a long K is summed in parts over K (the same parts whatever M is)
+        need = lib.cw_gemm_f32_workspace_floats(M, N, K)
+        parts = torch.empty(need, dtype=torch.float32, device=x.device) if need else None
+        _check(lib.cw_gemm_f32(_ptr(x), K, _ptr(weight), _ptr(bias), _ptr(out), N, M, N, K, _ptr(parts), need, _stream()),
+               "gemm_f32")
         return out
     if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16):
         raise KernelError("a bfloat16 product needs bfloat16 operands")

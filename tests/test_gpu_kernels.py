@@ -287,7 +287,11 @@ def test_rope_is_relative_and_identity_at_zero():
     assert abs(float(qa @ kb) - float(q0 @ k0)) > 1e-3  # and it does depend on the distance
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 100, 176), (7, 64, 33), (64, 130, 64), (130, 17, 1000), (3, 1000, 192)])
+# the last four are summed in parts over K: 22 parts of 416 of a down product, 6 of 256 that a
+# block sums itself (more than 256 rows), parts whose last is short (K = 1000: 3 of 336), a K that
+# no part's length divides
+@pytest.mark.parametrize("M,N,K", [(1, 100, 176), (7, 64, 33), (64, 130, 64), (130, 17, 1000), (3, 1000, 192),
+                                   (8, 1536, 8960), (300, 1536, 1536), (1, 2048, 1000), (9, 70, 777)])
 def test_gemm_f32(M, N, K):
     from clockwork_amd import ops
 
@@ -309,6 +313,17 @@ def test_gemm_f32_rows_do_not_depend_on_batch():
     whole = ops.linear(x, w)
     for i in (0, 33, 69):
         assert torch.equal(ops.linear(x[i : i + 1].contiguous(), w)[0], whole[i])
+    # a product that is summed in parts over K, by blocks of their own for few rows and inside a
+    # block for many: the same bits for a row alone, among 300 and among 17
+    x = torch.randn(300, 1024, device=DEV)
+    w = torch.randn(90, 1024, device=DEV)
+    b = torch.randn(90, device=DEV)
+    assert ops._load("gemm").cw_gemm_f32_workspace_floats(17, 90, 1024) == 4 * 17 * 90
+    assert ops._load("gemm").cw_gemm_f32_workspace_floats(300, 90, 1024) == 0
+    whole = ops.linear(x, w, b)
+    for i in (0, 255, 256, 299):
+        assert torch.equal(ops.linear(x[i : i + 1].contiguous(), w, b)[0], whole[i])
+    assert torch.equal(ops.linear(x[250:267].contiguous(), w, b), whole[250:267])
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
