@@ -29,7 +29,7 @@ struct AttnParams {
   int table_stride;
   const int* ctx_lens;    // [requests] keys of the request after this step
   const int* cu_q;        // [requests + 1] offsets of each request's tokens in the batch
-  const int* items;       // [n_items, 4]: request, first token (relative), tokens, unused
+  const int* items;       // [n_items, 4]: request, first token (relative), tokens, part | parts << 8 (prefill kernel)
   int nh, nkv, block_size;
   int bs_shift;           // log2(block_size) when it is a power of two, else -1
   int gh;                 // query heads of a group handled by one workgroup
@@ -895,11 +895,23 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
   const int wg_last = pos0 + ntok - 1;
   const int wg_lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
   const int bs = p.block_size, sh = p.bs_shift;
+  // the stages of keys this workgroup walks: all that its rows see, or one of ``parts`` runs of
+  // them when the item's key range is shared among workgroups (the merge kernel puts the parts'
+  // results together); a part may be empty
+  int t_first = wg_lo / KT, t_last = wg_last / KT;
+  const int packed = p.items[4 * item + 3];
+  const int parts = p.part_o != nullptr ? max(1, (packed >> 8) & 0xff) : 1;  // no workspace: every part is the whole
+  const int part = packed & 0xff;
+  if (parts > 1) {
+    const int per = (t_last - t_first + parts) / parts;
+    t_first += part * per;
+    t_last = min(t_last, t_first + per - 1);
+  }
   // the pages of the keys this workgroup reads -> LDS, a window of Tile::TABLE entries at a time
   // (32k keys with pages of 16): no tile waits for a table entry from memory
   const int* table = p.block_tables + (int64_t)req * p.table_stride;
   const int page_last = cw_page_index<POW2>(wg_last, bs, sh);
-  int page0 = cw_page_index<POW2>(wg_lo, bs, sh);  // the page of tbl[0]
+  int page0 = cw_page_index<POW2>(min(max(t_first * KT, wg_lo), wg_last), bs, sh);  // the page of tbl[0]
   auto load_table = [&]() __attribute__((always_inline)) {
     const int n_pages = min(page_last - page0 + 1, Tile::TABLE);
     for (int i = threadIdx.x; i < n_pages; i += NT) tbl[i] = table[page0 + i];
@@ -949,7 +961,6 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
   // than they saved: measured)
   constexpr int TPK = NT / KT;                  // threads per key
   constexpr int NCK = (CPR + TPK - 1) / TPK;    // chunks per thread and matrix
-  const int t_first = wg_lo / KT, t_last = wg_last / KT;
   const int f_key = threadIdx.x / TPK, f_ch = threadIdx.x % TPK;
   const int64_t row_elems = (int64_t)p.nkv * HD;
   // Two row blocks: the workgroups are short of work per stage, so a stage's loads get two stages
@@ -1172,6 +1183,24 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
     }
   }
 
+  // ---- a part of the key range: unnormalised sums, maximum and sum of every row of the workgroup
+  // (unused rows too: zeros) for the merge kernel
+  if (parts > 1) {
+    const int64_t slot = ((int64_t)item * gridDim.y + blockIdx.y) * (RB * 32);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const float l = cw_quad_sum(l_run[b]);
+      const int64_t row = slot + wave * 32 + b * 16 + c;
+#pragma unroll
+      for (int db = 0; db < ND; ++db) *reinterpret_cast<f32x4_t*>(p.part_o + row * HD + db * 16 + 4 * s) = o[b][db];
+      if (s == 0) {
+        p.part_ml[row * 2] = m_run[b];
+        p.part_ml[row * 2 + 1] = l;
+      }
+    }
+    return;
+  }
+
   // ---- out[row][d]: lane (c, s) holds d = db * 16 + 4s .. + 3 of row (b, c)
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
@@ -1186,6 +1215,83 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
       packed.x = (uint32_t)cw_float_to_bf16_bits(o[b][db][0] * inv) | ((uint32_t)cw_float_to_bf16_bits(o[b][db][1] * inv) << 16);
       packed.y = (uint32_t)cw_float_to_bf16_bits(o[b][db][2] * inv) | ((uint32_t)cw_float_to_bf16_bits(o[b][db][3] * inv) << 16);
       *reinterpret_cast<uint2*>(orow + db * 16 + 4 * s) = packed;
+    }
+  }
+}
+
+// Puts together the parts of items whose key range was shared among workgroups. One workgroup per
+// (item, key/value head) as in the kernel above; the workgroups of an item's parts share its rows
+// (part z takes rows z * ceil(rows / parts) ...), each reading those rows of every part. With few
+// rows a workgroup its threads also share the parts: thread (row, 4 elements, slice) sums the parts
+// slice, slice + S, ..., and the slices meet in LDS in a fixed order.
+#define PREFILL_MAX_PARTS 255
+
+template <int HD, int RB>
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(AttnParams p) {
+  constexpr int ROWS = RB * 32;
+  constexpr int VEC = HD / 4;  // 16-byte pieces of a row
+  __shared__ float ms[ROWS + PREFILL_MAX_PARTS + 1], ls[ROWS + PREFILL_MAX_PARTS + 1];
+  __shared__ __align__(16) float red[256 * 4];
+  const int packed = p.items[4 * blockIdx.x + 3];
+  const int parts = (packed >> 8) & 0xff, part = packed & 0xff;
+  if (parts <= 1) return;
+  const int item = blockIdx.x - part;  // the item's part 0
+  const int kvh = blockIdx.y / p.n_chunks, chunk = blockIdx.y % p.n_chunks;
+  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1];
+  const int gh = p.gh, tpw = 32 / gh, group = p.nh / p.nkv;
+  const int q_begin = p.cu_q[req];
+  const int ntok = min(p.items[4 * item + 2], p.cu_q[req + 1] - q_begin - tok0);
+  const float sl2 = p.scale * 1.4426950408889634f;
+  const int rpb = (ROWS + parts - 1) / parts;  // rows of this workgroup
+  const int row0 = part * rpb;
+  if (row0 >= ROWS) return;
+  auto slot = [&](int z, int row) { return ((int64_t)(item + z) * gridDim.y + blockIdx.y) * ROWS + row; };
+  for (int i = threadIdx.x; i < rpb * parts; i += 256) {
+    const int r = i / parts, z = i - r * parts;
+    const bool in = row0 + r < ROWS;
+    ms[i] = in ? p.part_ml[slot(z, row0 + r) * 2] : -INFINITY;
+    ls[i] = in ? p.part_ml[slot(z, row0 + r) * 2 + 1] : 0.0f;
+  }
+  __syncthreads();
+  const int n_pairs = rpb * VEC;                      // (row, 4 elements) pairs of this workgroup
+  const int slices = n_pairs >= 256 ? 1 : 256 / n_pairs;
+  for (int u0 = 0; u0 < n_pairs * slices; u0 += 256) {  // one round when the parts are shared
+    const int u = u0 + threadIdx.x;
+    const bool has = u < n_pairs * slices;
+    const int pair = has ? u % n_pairs : 0, slice = has ? u / n_pairs : 0;
+    const int r = pair / VEC, d = (pair - r * VEC) * 4;
+    const int row = row0 + r;
+    const int wave = row >> 5, rr = row & 31;
+    const int tl = rr / gh, g = rr - tl * gh;
+    const int tokw = wave * tpw + tl, hig = chunk * gh + g;
+    const bool valid = has && row < ROWS && tl < tpw && tokw < ntok && hig < group;
+    float m = -INFINITY, l = 0.0f;
+    f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (valid) {
+      for (int z = 0; z < parts; ++z) m = fmaxf(m, ms[r * parts + z]);
+      for (int z = 0; z < parts; ++z) {
+        const float mz = ms[r * parts + z];
+        l = fmaf(ls[r * parts + z], mz == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f((mz - m) * sl2), l);
+      }
+      for (int z = slice; z < parts; z += slices) {
+        const float mz = ms[r * parts + z];
+        if (mz == -INFINITY) continue;
+        acc += *reinterpret_cast<const f32x4_t*>(p.part_o + slot(z, row) * HD + d) * __builtin_amdgcn_exp2f((mz - m) * sl2);
+      }
+    }
+    if (slices > 1) {
+      *reinterpret_cast<f32x4_t*>(&red[threadIdx.x * 4]) = acc;
+      __syncthreads();
+      if (slice == 0)
+        for (int sl = 1; sl < slices; ++sl) acc += *reinterpret_cast<const f32x4_t*>(&red[(sl * n_pairs + pair) * 4]);
+    }
+    if (valid && slice == 0) {
+      const float inv = 1.0f / l;
+      bf16_t* orow = (bf16_t*)p.out + (int64_t)(q_begin + tok0 + tokw) * p.out_stride + (int64_t)(kvh * group + hig) * HD;
+      uint2 two;
+      two.x = (uint32_t)cw_float_to_bf16_bits(acc[0] * inv) | ((uint32_t)cw_float_to_bf16_bits(acc[1] * inv) << 16);
+      two.y = (uint32_t)cw_float_to_bf16_bits(acc[2] * inv) | ((uint32_t)cw_float_to_bf16_bits(acc[3] * inv) << 16);
+      *reinterpret_cast<uint2*>(orow + d) = two;
     }
   }
 }
@@ -1217,9 +1323,20 @@ static int launch_prefill(const AttnParams& p, int n_items, int table_stride, hi
     raised = smem;
   }
   hipLaunchKernelGGL((attn_prefill_bf16_kernel<CW_HD, POW2, RB>), grid, block, smem, stream, p);
+  if (p.part_o != nullptr)
+    hipLaunchKernelGGL((attn_prefill_merge_kernel<CW_HD, RB>), grid, dim3(256), 0, stream, p);
   return cw_launch_status();
 }
 #endif
+
+// Floats of workspace cw_attention_prefill_bf16 needs when some items are parts of a key range.
+CW_EXPORT int64_t cw_attention_prefill_workspace_floats(int n_items, int nh, int nkv, int row_blocks) {
+  if (n_items <= 0 || nh <= 0 || nkv <= 0) return 0;
+  const int group = nh / nkv;
+  const int gh = group < 32 ? group : 32;
+  const int n_chunks = (group + gh - 1) / gh;
+  return (int64_t)n_items * nkv * n_chunks * row_blocks * 32 * (CW_HD + 2);
+}
 
 // 1 if the kernel for portions can run with this many row blocks a workgroup (4, and 2 for head
 // sizes up to 128).
@@ -1227,14 +1344,19 @@ CW_EXPORT int cw_attention_prefill_row_blocks_ok(int row_blocks) {
   return CW_HAS_PREFILL && (row_blocks == 4 || (row_blocks == 2 && CW_HD <= 128)) ? 1 : 0;
 }
 
-// Portions of prompts, bfloat16. items: (request, first token, tokens, 0) with
+// Portions of prompts, bfloat16. items: (request, first token, tokens, part | parts << 8) with
 // tokens <= row_blocks * (32 / gh), gh = min(group, 32) heads of a group per workgroup; tokens of
-// an item beyond that are not computed. row_blocks: 4, or 2 (see PrefillTile).
+// an item beyond that are not computed. row_blocks: 4, or 2 (see PrefillTile). An item with
+// parts > 1 stands ``parts`` times in the list, one after the other, as part 0, 1, ...: each takes
+// a share of the keys that its tokens see, and a second kernel puts the shares together. Any item
+// of that kind (``with_parts``) needs a float32 workspace of
+// cw_attention_prefill_workspace_floats(n_items, ...) elements; parts at most 255.
 CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride,
                                         const void* k_cache, const void* v_cache, const int* block_tables,
                                         int table_stride, const int* ctx_lens, const int* cu_q,
                                         const int* items, int n_items, int nh, int nkv, int block_size,
                                         int window, float scale, const void* zeros, int row_blocks,
+                                        int with_parts, float* workspace, int64_t workspace_floats,
                                         hipStream_t stream) {
 #if CW_HAS_PREFILL
   if (zeros == nullptr || ((uintptr_t)zeros & 15)) return CW_ERR_ARG;
@@ -1254,6 +1376,12 @@ CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* o
   p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = 1; p.window = window; p.scale = scale;
   p.part_o = nullptr; p.part_ml = nullptr; p.zeros = zeros;
   if ((int64_t)nkv * p.n_chunks > 65535) return CW_ERR_SIZE;
+  if (with_parts) {
+    const int64_t need = cw_attention_prefill_workspace_floats(n_items, nh, nkv, row_blocks);
+    if (workspace == nullptr || workspace_floats < need || ((uintptr_t)workspace & 15)) return CW_ERR_ARG;
+    p.part_o = workspace;
+    p.part_ml = workspace + need / (CW_HD + 2) * CW_HD;
+  }
 #if CW_HD <= 128
   if (row_blocks == 2)
     return p.bs_shift >= 0 ? launch_prefill<true, 2>(p, n_items, table_stride, stream)

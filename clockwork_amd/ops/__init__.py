@@ -123,7 +123,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_attention_workspace_floats": [I, I, I, I, I],
             "cw_attention": [I, I, P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P, L, P],
             "cw_attention_prefill_supported": [],
-            "cw_attention_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, P, I, P],
+            "cw_attention_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, P, I, I, P, L, P],
+            "cw_attention_prefill_workspace_floats": [I, I, I, I],
             "cw_attention_prefill_row_blocks_ok": [I],
             "cw_attention_decode_supported": [],
             "cw_attention_decode_gh": [I],
@@ -592,13 +593,23 @@ def prefill_attention_supported(hd: int, dtype: torch.dtype) -> bool:
 
 def attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
                       nh: int, nkv: int, hd: int, block_size: int, window: int, scale: float,
-                      n_tokens: int, n_requests: int, row_blocks: int = 4) -> None:
+                      n_tokens: int, n_requests: int, row_blocks: int = 4, workspace=None) -> None:
     """Portions of prompts through the bfloat16 matrix-core kernel; an item holds at most
     ``prefill_tokens_per_item(nh // nkv, row_blocks)`` tokens. ``row_blocks`` 2 instead of 4: smaller
-    workgroups for launches with few items (head sizes up to 128). Other arguments as for ``attention``."""
+    workgroups for launches with few items (head sizes up to 128). Other arguments as for ``attention``.
+    An item's fourth field is ``part | parts << 8``: with parts > 1 the item stands that many times
+    in the list, one after the other, and each takes a share of its keys; such a list needs a
+    float32 ``workspace`` of ``prefill_attention_workspace_floats`` elements (without one every item
+    computes all of its keys)."""
     if not (prefill_row_blocks_ok(hd, row_blocks)):
         raise KernelError(f"the kernel for head size {hd} does not take {row_blocks} row blocks")
-    _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items)
+    _gpu(out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, workspace)
+    ws_floats = 0
+    if workspace is not None:
+        need = prefill_attention_workspace_floats(hd, n_items, nh, nkv, row_blocks)
+        _need(workspace.dtype == torch.float32 and workspace.numel() >= need,
+              f"attention over parts of key ranges needs a float32 workspace of {need} elements")
+        ws_floats = workspace.numel()
     if not (q.is_cuda and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16):
         raise KernelError("the kernel is bfloat16")
     if not (out.dim() == 2 and out.shape[0] >= n_tokens and out.shape[1] == nh * hd):
@@ -617,9 +628,14 @@ def attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx
         _load("attention", hd).cw_attention_prefill_bf16(
             q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
             block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, nh, nkv, block_size,
-            window, float(scale), _zero_row(out.device), int(row_blocks), _stream()),
+            window, float(scale), _zero_row(out.device), int(row_blocks), int(workspace is not None), _ptr(workspace),
+            ws_floats, _stream()),
         "attention_prefill_bf16",
     )
+
+
+def prefill_attention_workspace_floats(hd: int, n_items: int, nh: int, nkv: int, row_blocks: int) -> int:
+    return int(_load("attention", hd).cw_attention_prefill_workspace_floats(n_items, nh, nkv, int(row_blocks)))
 
 
 def prefill_row_blocks_ok(hd: int, row_blocks: int) -> bool:

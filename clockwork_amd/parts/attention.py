@@ -35,6 +35,7 @@ class AttentionPlan:
     mfma_items: Optional[torch.Tensor] = None   # the same portions cut for the bfloat16 matrix-core kernel
     n_mfma: int = 0
     mfma_row_blocks: int = 4   # row blocks of that kernel's workgroups: 2 when 4 would leave compute units idle
+    mfma_parts: int = 1        # the most parts an item's key range is shared among (1: no item is cut)
     single_items: Optional[torch.Tensor] = None
     n_single: int = 0
     gh_single: int = 1
@@ -59,6 +60,41 @@ def portions_have_short_ranges(q_lens, ctx_lens) -> bool:
     tokens = sum(q for q in q_lens if q > 1)
     keys = sum(q * (c - q / 2.0) for q, c in zip(q_lens, ctx_lens) if q > 1)
     return tokens > 0 and keys / tokens < LONG_RANGE_KEYS
+
+
+# a part of an item's key range is at least this many keys (two stages of the kernel), and an item
+# is cut into at most this many parts
+MIN_PART_KEYS = 256
+MAX_PARTS = 64
+
+
+def _share_long_key_ranges(items: np.ndarray, ctx, workgroups_per_item: int):
+    """One workgroup of the kernel for portions keeps its compute unit busy by itself, so a launch
+    with fewer workgroups than half the compute units (a short portion behind a long cached
+    prefix: the end of a long prompt, a new turn of a long conversation) leaves most of the card
+    idle while a few units walk through thousands of keys. Such a launch's items stand in the
+    list once for each of several parts, one after the other, as ``part | parts << 8`` in the
+    fourth field; the kernel gives each part a run of the item's keys and a second kernel puts
+    them together. Launches that fill the card are left alone: there the parts cost more than
+    they bring (measured). Returns the flat item list and the most parts of an item (1: nothing
+    was cut)."""
+    workgroups = len(items) * workgroups_per_item
+    spare = ctx.num_compute_units // max(workgroups, 1)
+    if len(items) == 0 or spare < 2:
+        return items.reshape(-1), 1
+    ctx_lens = np.asarray(ctx.h_ctx_lens, dtype=np.int64)
+    q_lens = np.asarray(ctx.h_q_lens, dtype=np.int64)
+    req = items[:, 0]
+    keys = ctx_lens[req] - q_lens[req] + items[:, 1] + items[:, 2]  # keys that the item's last token sees
+    parts = np.minimum(spare, keys // MIN_PART_KEYS).clip(1, MAX_PARTS).astype(np.int64)
+    most = int(parts.max())
+    if most == 1:
+        return items.reshape(-1), 1
+    out = np.repeat(items, parts, axis=0)
+    first = np.cumsum(parts) - parts  # where each item's parts begin
+    part = np.arange(len(out)) - np.repeat(first, parts)
+    out[:, 3] = part | (np.repeat(parts, parts) << 8)
+    return out.astype(np.int32).reshape(-1), most
 
 
 def attention_plan(ctx, nh: int, nkv: int, narrow_ok: bool = False) -> AttentionPlan:
@@ -114,6 +150,7 @@ def _make_plan(ctx, nh: int, nkv: int, narrow_ok: bool) -> AttentionPlan:
     wide = np.concatenate(wide) if wide else np.zeros(0, dtype=np.int32)
     mfma = np.concatenate(mfma) if mfma else np.zeros(0, dtype=np.int32)
     plan = AttentionPlan(gh_wide=gh_wide, gh_single=gh_single, mfma_row_blocks=row_blocks)
+    mfma, plan.mfma_parts = _share_long_key_ranges(mfma.reshape(-1, 4), ctx, nkv * -(-group // 32))
     plan.n_wide, plan.n_single, plan.n_mfma = len(wide) // 4, len(single) // 4, len(mfma) // 4
     plan.chunks_single = -(-group // gh_single)
     if plan.n_single:
@@ -220,7 +257,12 @@ class PagedAttention(Part):
             scale=s.scale, n_tokens=T, n_requests=ctx.num_requests,
         )
         if plan.n_wide and mfma:
-            ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, row_blocks=plan.mfma_row_blocks, **common)
+            workspace = None
+            if plan.mfma_parts > 1:
+                need = ops.prefill_attention_workspace_floats(hd, plan.n_mfma, nh, nkv, plan.mfma_row_blocks)
+                workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+            ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, row_blocks=plan.mfma_row_blocks,
+                                  workspace=workspace, **common)
         elif plan.n_wide:
             ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide,
                           n_splits=1, **common)

@@ -568,7 +568,7 @@ def _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens, poison=100.0)
 
 
 def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs, window=0, splits=None, scale=None,
-                   decode_kernel=False, prefill_kernel=False, fixed_ranges=False):
+                   decode_kernel=False, prefill_kernel=False, fixed_ranges=False, key_parts=0):
     from clockwork_amd import ops
     from clockwork_amd.engine.batch import StepContext
     from clockwork_amd.parts.attention import attention_plan
@@ -601,7 +601,17 @@ def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs,
                   cu_q=cu, nh=nh, nkv=nkv, hd=hd, block_size=bs, window=window, scale=scale, n_tokens=T, n_requests=R)
     if plan.n_wide and prefill_kernel:
         assert ops.prefill_attention_supported(hd, dtype)
-        ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, row_blocks=plan.mfma_row_blocks, **common)
+        items, n_items, ws = plan.mfma_items, plan.n_mfma, None
+        if key_parts:  # every item's key range shared among this many workgroups (some parts may be empty)
+            rec = items.cpu().numpy().reshape(-1, 4)[:n_items]
+            rec = rec[(rec[:, 3] & 255) == 0]  # each item once, whatever the plan made of it
+            rec = rec.repeat(key_parts, axis=0)
+            rec[:, 3] = (torch.arange(len(rec)).numpy() % key_parts) | (key_parts << 8)
+            items, n_items = torch.tensor(rec.reshape(-1), dtype=torch.int32, device=DEV), len(rec)
+        if key_parts or plan.mfma_parts > 1:
+            ws = torch.full((ops.prefill_attention_workspace_floats(hd, n_items, nh, nkv, plan.mfma_row_blocks),),
+                            float("nan"), dtype=torch.float32, device=DEV)
+        ops.attention_prefill(items=items, n_items=n_items, row_blocks=plan.mfma_row_blocks, workspace=ws, **common)
     elif plan.n_wide:
         ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide, n_splits=1, **common)
     if plan.n_single and decode_kernel:
@@ -781,6 +791,76 @@ def test_prefill_attention_kernel(nh, nkv, hd, bs, window, row_blocks):
                                      window=window or None)
         torch.testing.assert_close(out[at : at + q_len].float().cpu(), want, **tol(dtype))
         at += q_len
+
+
+@pytest.mark.parametrize("nh,nkv,hd,bs", [(4, 2, 32, 4), (12, 2, 128, 16), (2, 1, 256, 16), (40, 1, 64, 8), (7, 7, 96, 16)])
+@pytest.mark.parametrize("window", [0, 40])
+@pytest.mark.parametrize("row_blocks", [4, 2])
+@pytest.mark.parametrize("key_parts", [2, 5])
+def test_prefill_attention_kernel_with_shared_key_ranges(nh, nkv, hd, bs, window, row_blocks, key_parts):
+    """Every item's keys in 2 or 5 parts, each a workgroup of its own, put together by the merge
+    kernel: contexts of one stage (all parts but the first empty) up to many stages, a portion
+    behind a cached prefix, single-token requests in between, NaN in unowned pages and in the
+    workspace."""
+    dtype = torch.bfloat16
+    if row_blocks == 2 and hd > 128:
+        pytest.skip("head sizes beyond 128 have the kernel with four row blocks only")
+    ctx_lens = [21, 700, 2, 1, 333, 1100]
+    q_lens = [6, 150, 2, 1, 333, 64]
+    num_blocks = sum(-(-c // bs) for c in ctx_lens) + 3
+    perm = torch.randperm(num_blocks).tolist()
+    tables, at = [], 0
+    for c in ctx_lens:
+        n = -(-c // bs)
+        tables.append(perm[at : at + n])
+        at += n
+    kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens, poison=float("nan"))
+    tables_dev = [list(t) for t in tables]
+    if window:
+        for r, (c, q) in enumerate(zip(ctx_lens, q_lens)):
+            for b in range(max(0, (c - q) - window + 1) // bs):
+                tables_dev[r][b] = -1
+    qs = [torch.randn(q, nh, hd, device=DEV).to(dtype) for q in q_lens]
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables_dev, ctx_lens, q_lens, kc, vc, qs, window=window,
+                         prefill_kernel=row_blocks, decode_kernel=ops_decode_ok(hd), key_parts=key_parts)
+    assert not torch.isnan(out.float()).any()
+    at = 0
+    for r, q_len in enumerate(q_lens):
+        want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5,
+                                     window=window or None)
+        torch.testing.assert_close(out[at : at + q_len].float().cpu(), want, **tol(dtype))
+        at += q_len
+
+
+def test_the_plan_shares_long_key_ranges_among_workgroups():
+    """A short portion behind a long cached prefix makes few workgroups with long walks: its items
+    are cut into as many parts as there are idle compute units for. A launch that fills the card
+    (a whole prompt of 2048 tokens) and items with few keys are left alone."""
+    import numpy as np
+
+    from clockwork_amd.engine.batch import StepContext
+    from clockwork_amd.parts.attention import MAX_PARTS, MIN_PART_KEYS, attention_plan
+
+    def plan_of(q_lens, ctx_lens):
+        ctx = StepContext()
+        ctx.device = torch.device(DEV)
+        ctx.h_q_lens, ctx.h_ctx_lens = list(q_lens), list(ctx_lens)
+        assert ctx.num_compute_units == 256
+        plan = attention_plan(ctx, 12, 2, narrow_ok=True)
+        return plan, plan.mfma_items.cpu().numpy().reshape(-1, 4)[: plan.n_mfma]
+
+    plan, items = plan_of([2048], [2048])
+    assert plan.mfma_parts == 1 and (items[:, 3] == 0).all()
+    plan, items = plan_of([200], [8392])  # 10 items of 20 tokens on 2 key/value heads: 20 workgroups, 12 parts each
+    assert plan.mfma_row_blocks == 4 and plan.mfma_parts == 12 and plan.n_mfma == 120
+    parts, part = (items[:, 3] >> 8) & 255, items[:, 3] & 255
+    assert (parts == 12).all() and items[part == 0][:, 2].sum() == 200  # every token in one item before the items were repeated
+    for i in np.flatnonzero(part == 0):  # the parts of an item follow one another
+        assert (items[i : i + 12, :3] == items[i, :3]).all() and list(part[i : i + 12]) == list(range(12))
+    plan, items = plan_of([16], [30016])  # 4 workgroups: as many parts as the kernel's list allows
+    assert plan.mfma_parts == MAX_PARTS == 64 and 30000 // MAX_PARTS >= MIN_PART_KEYS
+    plan, items = plan_of([100, 1, 1], [100, 500, 700])  # few workgroups, but of few keys
+    assert plan.mfma_parts == 1 and (items[:, 3] == 0).all()
 
 
 @pytest.mark.parametrize("window", [0, 700])

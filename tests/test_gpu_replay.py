@@ -450,6 +450,47 @@ def test_first_tokens_and_long_decoding(model_dirs, dtype):
     _check(got, ref, dtype)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B_peaked", "C"])
+def test_short_portions_behind_a_long_prefix(model_dirs, name, dtype):
+    """Portions of 2 to 170 tokens behind 700 to 1100 cached ones make few attention workgroups with
+    long key ranges: in bfloat16 the plan shares every item's keys among several workgroups and a
+    second kernel puts their parts together. Every token's logits are compared, with attention that
+    looks at single far keys (B_peaked); a second request decodes beside some of the portions,
+    which come twice in the same shape so that they also run as captured graphs."""
+    from clockwork_amd.engine.batch import StepContext
+    from clockwork_amd.parts.attention import attention_plan
+
+    cfg, _, block_size = TINY_CONFIGS[name.split("_")[0]]
+    gen = torch.Generator().manual_seed(46)
+    toks = {"x": torch.randint(0, cfg["vocab_size"], (1100,), generator=gen).tolist(),
+            "d": torch.randint(0, cfg["vocab_size"], (60,), generator=gen).tolist()}
+    steps = [{"entries": [{"id": "x", "tokens": toks["x"][:700], "want": [699]}], "end": []},
+             {"entries": [{"id": "d", "tokens": toks["d"][:40], "want": [39]}], "end": []}]
+    at, d_at = 700, 40
+    for i, n in enumerate([3, 17, 17, 64, 100, 40, 40, 2, 117]):
+        entries = [{"id": "x", "tokens": toks["x"][at : at + n], "want": list(range(n))}]
+        if i % 2:
+            entries.insert(0, {"id": "d", "tokens": toks["d"][d_at : d_at + 1], "want": [0]})
+            d_at += 1
+        steps.append({"entries": entries, "end": []})
+        at += n
+    assert at == 1100
+    steps[-1]["end"] = ["x", "d"]
+    # the plan of such a step cuts its items (heads as in the model, 256 compute units)
+    probe = StepContext()
+    probe.device = torch.device("cuda")
+    probe.h_q_lens, probe.h_ctx_lens = [64], [800]
+    assert attention_plan(probe, cfg["num_attention_heads"], cfg["num_key_value_heads"], narrow_ok=True).mfma_parts >= 2
+    runner = replay.make_runner(model_dirs[name], dtype, block_size, -(-1100 // block_size) + -(-60 // block_size) + 2,
+                                max_model_len=1200)
+    got = replay.run_trace(runner, steps)
+    model = PlainQwen2(model_dirs[name])
+    ref = {k: model.logits(v) for k, v in toks.items()}
+    assert len(got) == 2 + 400 + 4
+    _check(got, ref, dtype)
+
+
 @pytest.mark.parametrize("dtype,graph_limit", [("float32", None), ("bfloat16", None), ("bfloat16", 1)])
 def test_graph_replays_equal_eager_steps(model_dirs, dtype, graph_limit, monkeypatch):
     """Decode steps replay a captured HIP graph. Every replay is checked against the same step run
