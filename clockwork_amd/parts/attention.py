@@ -69,8 +69,8 @@ MAX_PARTS = 64
 
 
 def _share_long_key_ranges(items: np.ndarray, ctx, workgroups_per_item: int):
-    """One workgroup of the kernel for portions keeps its compute unit busy by itself, so a launch
-    with fewer workgroups than half the compute units (a short portion behind a long cached
+    """A compute unit holds one workgroup of the kernel for portions at a time (its tiles fill the
+    unit's LDS), so a launch with fewer workgroups than half the compute units (a short portion behind a long cached
     prefix: the end of a long prompt, a new turn of a long conversation) leaves most of the card
     idle while a few units walk through thousands of keys. Such a launch's items stand in the
     list once for each of several parts, one after the other, as ``part | parts << 8`` in the
