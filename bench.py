@@ -33,7 +33,17 @@ QWEN25_7B = dict(QWEN25_1P5B, vocab_size=152064, hidden_size=3584, num_attention
                  intermediate_size=18944, tie_word_embeddings=False)
 QWEN25_32B = dict(QWEN25_1P5B, vocab_size=152064, hidden_size=5120, num_hidden_layers=64, num_attention_heads=40,
                   num_key_value_heads=8, intermediate_size=27648, tie_word_embeddings=False)
-SHAPES = {"1.5b": ("Qwen2.5-1.5B", QWEN25_1P5B), "7b": ("Qwen2.5-7B", QWEN25_7B), "32b": ("Qwen2.5-32B", QWEN25_32B)}
+QWEN25_0P5B = dict(QWEN25_1P5B, hidden_size=896, num_hidden_layers=24, num_attention_heads=14, num_key_value_heads=2,
+                   intermediate_size=4864)
+QWEN25_3B = dict(QWEN25_1P5B, hidden_size=2048, num_hidden_layers=36, num_attention_heads=16, num_key_value_heads=2,
+                 intermediate_size=11008)
+QWEN25_14B = dict(QWEN25_1P5B, vocab_size=152064, hidden_size=5120, num_hidden_layers=48, num_attention_heads=40,
+                  num_key_value_heads=8, intermediate_size=13824, tie_word_embeddings=False)
+QWEN25_72B = dict(QWEN25_1P5B, vocab_size=152064, hidden_size=8192, num_hidden_layers=80, num_attention_heads=64,
+                  num_key_value_heads=8, intermediate_size=29568, tie_word_embeddings=False)
+SHAPES = {"0.5b": ("Qwen2.5-0.5B", QWEN25_0P5B), "1.5b": ("Qwen2.5-1.5B", QWEN25_1P5B), "3b": ("Qwen2.5-3B", QWEN25_3B),
+          "7b": ("Qwen2.5-7B", QWEN25_7B), "14b": ("Qwen2.5-14B", QWEN25_14B), "32b": ("Qwen2.5-32B", QWEN25_32B),
+          "72b": ("Qwen2.5-72B", QWEN25_72B)}
 PROMPT_LEN = 2048   # the prefill measurement, and the decode requests' prompts unless --prompt-len says otherwise
 CONTEXT = 4096
 BLOCK = 16
