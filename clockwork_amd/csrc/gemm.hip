@@ -427,11 +427,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
   } else {
     // Token tile by token tile, a row's k-steps one after the other: a lane's 16 bytes of step u
     // and of step u + 1 are halves of one 128-byte line, and asked for back to back the second
-    // finds the line in the compute unit's own cache (step by step over all token tiles, every
     // finds the line in the compute unit's own cache. The loads are unconditional, from clamped
     // addresses; what lies past M or K is zeroed afterwards. (Every workgroup pulls all of x from
-    // L2: with 64 rows that is 44 MB beside the 55 MB of a gate/up matrix, and the two share what
-    // L2 delivers, about 5.7 TB/s: 13 us with 8 rows, 19 us with 64.)
+    // L2: with 64 rows that is 44 MB beside the 55 MB of a gate/up matrix, and the kernel takes
+    // both in at about 5.7 TB/s: 13 us with 8 rows, 19 us with 64.)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const bf16_t* xrow = X + (int64_t)min(mt * 16 + r, M - 1) * ldx;
