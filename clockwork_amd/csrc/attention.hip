@@ -314,8 +314,10 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   const int item = blockIdx.x;
   const int kvh = blockIdx.y / p.n_chunks;
   const int chunk = blockIdx.y % p.n_chunks;
-  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1], ntok = p.items[4 * item + 2];
+  const int req = p.items[4 * item], tok0 = p.items[4 * item + 1];
   const int q_begin = p.cu_q[req];
+  // as in the kernel above: an item may reach past the request's tokens, and those rows are nobody's
+  const int ntok = min(p.items[4 * item + 2], p.cu_q[req + 1] - q_begin - tok0);
   const int group = p.nh / p.nkv;
   const int gh = p.gh;
   const int64_t base = ((int64_t)item * gridDim.y + blockIdx.y) * p.n_splits;

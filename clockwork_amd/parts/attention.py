@@ -32,6 +32,7 @@ class AttentionPlan:
     wide_items: Optional[torch.Tensor] = None
     n_wide: int = 0
     gh_wide: int = 1
+    wide_splits: int = 1       # parts every wide item's key range is cut into (few items with many keys)
     mfma_items: Optional[torch.Tensor] = None   # the same portions cut for the bfloat16 matrix-core kernel
     n_mfma: int = 0
     mfma_row_blocks: int = 4   # row blocks of that kernel's workgroups: 2 when 4 would leave compute units idle
@@ -152,6 +153,12 @@ def _make_plan(ctx, nh: int, nkv: int, narrow_ok: bool) -> AttentionPlan:
     plan = AttentionPlan(gh_wide=gh_wide, gh_single=gh_single, mfma_row_blocks=row_blocks)
     mfma, plan.mfma_parts = _share_long_key_ranges(mfma.reshape(-1, 4), ctx, nkv * -(-group // 32))
     plan.n_wide, plan.n_single, plan.n_mfma = len(wide) // 4, len(single) // 4, len(mfma) // 4
+    if plan.n_wide:
+        # the 64-row kernel cuts every item's keys the same number of ways: as many as there are idle
+        # compute units for, while the longest portion's keys give each part MIN_PART_KEYS
+        spare = ctx.num_compute_units // (plan.n_wide * nkv * -(-group // gh_wide))
+        most_keys = max(c for q, c in zip(ctx.h_q_lens, ctx.h_ctx_lens) if q > 1)
+        plan.wide_splits = int(max(1, min(spare, most_keys // MIN_PART_KEYS, MAX_PARTS)))
     plan.chunks_single = -(-group // gh_single)
     if plan.n_single:
         groups_running = plan.n_single * nkv * plan.chunks_single
@@ -264,8 +271,12 @@ class PagedAttention(Part):
             ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, row_blocks=plan.mfma_row_blocks,
                                   workspace=workspace, **common)
         elif plan.n_wide:
+            workspace = None
+            if plan.wide_splits > 1:
+                need = ops.attention_workspace_floats(hd, 64, plan.n_wide, nkv, -(-(nh // nkv) // plan.gh_wide), plan.wide_splits)
+                workspace = torch.empty(need, dtype=torch.float32, device=x.device)
             ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide,
-                          n_splits=1, **common)
+                          n_splits=plan.wide_splits, workspace=workspace, **common)
         if plan.n_single and ops.decode_attention_supported(hd, x.dtype):
             workspace = None
             if plan.decode_splits > 1:

@@ -613,7 +613,13 @@ def _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs,
                             float("nan"), dtype=torch.float32, device=DEV)
         ops.attention_prefill(items=items, n_items=n_items, row_blocks=plan.mfma_row_blocks, workspace=ws, **common)
     elif plan.n_wide:
-        ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide, n_splits=1, **common)
+        n_splits, ws = key_parts or plan.wide_splits, None
+        if n_splits > 1:
+            chunks = -(-(nh // nkv) // plan.gh_wide)
+            ws = torch.full((ops.attention_workspace_floats(hd, 64, plan.n_wide, nkv, chunks, n_splits),), float("nan"),
+                            dtype=torch.float32, device=DEV)
+        ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide, n_splits=n_splits,
+                      workspace=ws, **common)
     if plan.n_single and decode_kernel:
         assert ops.decode_attention_supported(hd, dtype)
         n_splits = splits if splits is not None else plan.decode_splits
@@ -670,9 +676,11 @@ def test_attention_single_tokens(dtype, nh, nkv, hd, bs, ctx_lens, splits):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,hd,bs", [(4, 2, 16, 4), (6, 1, 32, 8), (3, 3, 48, 16), (12, 2, 128, 16), (2, 1, 256, 16)])
-def test_attention_portions_and_mixed_batches(dtype, nh, nkv, hd, bs):
+@pytest.mark.parametrize("key_parts", [0, 3])
+def test_attention_portions_and_mixed_batches(dtype, nh, nkv, hd, bs, key_parts):
     """Portions (cached prefix + new tokens, end-aligned mask: clockwork/kernels/attention.py:45-65,
-    tests/test_attention_kernels.py:49-62) next to single tokens, scrambled pages, poisoned free slots."""
+    tests/test_attention_kernels.py:49-62) next to single tokens, scrambled pages, poisoned free slots.
+    key_parts: every portion item's keys cut three ways and merged (parts of short ranges are empty)."""
     ctx_lens = [21, 150, 2, 77, 1, 64]
     q_lens = [6, 150, 2, 1, 1, 33]
     num_blocks = sum(-(-c // bs) for c in ctx_lens) + 3
@@ -684,7 +692,7 @@ def test_attention_portions_and_mixed_batches(dtype, nh, nkv, hd, bs):
         at += n
     kc, vc, ks, vs = _paged_setup(dtype, nkv, hd, bs, num_blocks, tables, ctx_lens)
     qs = [torch.randn(q, nh, hd, device=DEV).to(dtype) for q in q_lens]
-    out = _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs)
+    out = _run_attention(dtype, nh, nkv, hd, bs, tables, ctx_lens, q_lens, kc, vc, qs, key_parts=key_parts)
     at = 0
     for r, q_len in enumerate(q_lens):
         want = plain.attention_dense(qs[r].float().cpu(), ks[r].float().cpu(), vs[r].float().cpu(), hd ** -0.5)
