@@ -75,7 +75,8 @@ def build_runner(args, prefix_cache: bool = False, max_batch: int = 0):
     mcfg = arch.parse_config(config)
     spec = arch.build_spec(mcfg)
     source = RandomSource(arch.weight_plan(mcfg, spec), model_param_specs(spec), seed=2, device="cuda")
-    max_batch = max(args.batch, 64, max_batch)
+    # the cache holds the largest batch the run decodes: 64 for the recorded points
+    max_batch = max(args.batch, 1 if getattr(args, "no_points", False) else 64, max_batch)
     context = context_of(args)
     cfg = EngineConfig.defaults(
         f"random:{SHAPES[args.shape][0].lower()}", dtype=args.dtype, max_model_len=context, block_size=BLOCK,
