@@ -1,7 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16] [--shape 1.5b]
-    python bench.py --workload mixed|arrivals [--shape 7b] [--requests 64]
+    python bench.py --workload mixed|arrivals|agent [--shape 7b] [--requests 64]
 
 Default workload: the layer sizes of Qwen2.5-1.5B with random weights (seed 2), bfloat16,
 8 requests that each hold a 2048-token prompt, context limit 4096, pages of 16 tokens. A
@@ -268,6 +268,124 @@ def run_mixed(args) -> dict:
     }
 
 
+def run_agent(args) -> dict:
+    """Sessions of several turns over a shared opening, the shape of traffic that the reference's
+    agent traces model (docs/results.md: a system prompt of 1024 tokens that every session opens
+    with, 4 to 8 turns a session): turn t's prompt is the opening, the session's earlier turns
+    (their inputs and the generated answers) and 64 to 256 new tokens; 32 to 96 greedy tokens are
+    generated a turn. ``--concurrency`` sessions run at a time, each sending its next turn when the
+    last one is finished; ``--requests`` sessions in all. With the prefix cache a turn computes its
+    new tokens only; ``--no-prefix-cache`` runs the same traffic without it."""
+    import torch
+
+    from clockwork_amd.engine.llm_engine import LLMEngine
+    from clockwork_amd.engine.sequence import SamplingParams
+
+    n_sessions, opening = args.requests, 1024
+    cfg, runner = build_runner(args, prefix_cache=not args.no_prefix_cache, max_batch=max(args.concurrency, 8))
+    vocab = runner.spec.vocab_size
+    gen = torch.Generator().manual_seed(11)
+    common = torch.randint(0, vocab, (opening,), generator=gen).tolist()
+    sessions = []
+    for _ in range(n_sessions):
+        turns = int(torch.randint(4, 9, (1,), generator=gen))
+        sessions.append([torch.randint(0, vocab, (int(torch.randint(64, 257, (1,), generator=gen)),), generator=gen).tolist()
+                         for _ in range(turns)])
+    # answers of 32 to 96 tokens, so that the sessions do not fall into step with one another
+    answer = [[int(torch.randint(32, 97, (1,), generator=gen)) for _ in turns] for turns in sessions]
+    engine = LLMEngine(cfg, runner=runner)
+
+    def once(tag):
+        engine.prefix_cache.reset()
+        _sync()
+        before = engine.stats()
+        t0 = time.perf_counter()
+        history = {}   # session -> tokens so far
+        turn_of = {}   # session -> index of the turn that is running
+        sent, first = {}, []
+        queue = list(range(n_sessions))
+        prompt_tokens = outputs = steps = 0
+
+        def send(i):
+            nonlocal prompt_tokens
+            t = turn_of[i]
+            history[i] = history[i] + sessions[i][t]
+            rid = f"{tag}-{i}-{t}"
+            engine.add_request(rid, prompt_token_ids=history[i],
+                               sampling_params=SamplingParams(max_tokens=answer[i][t], temperature=0.0, ignore_eos=True))
+            sent[rid] = time.perf_counter()
+            prompt_tokens += len(history[i])
+
+        running = 0
+        while queue or running:
+            while queue and running < args.concurrency:
+                i = queue.pop(0)
+                history[i], turn_of[i] = list(common), 0
+                send(i)
+                running += 1
+            outs = engine.step()
+            steps += 1
+            now = time.perf_counter()
+            for o in outs:
+                if o.num_generated_tokens == 1:
+                    first.append(now - sent[o.request_id])
+                if o.finished:
+                    outputs += o.num_generated_tokens
+                    i = int(o.request_id.split("-")[1])
+                    history[i] = history[i] + list(o.token_ids)
+                    turn_of[i] += 1
+                    if turn_of[i] < len(sessions[i]):
+                        send(i)
+                    else:
+                        running -= 1
+        _sync()
+        elapsed = time.perf_counter() - t0
+        after = engine.stats()
+        cached = after["total_cached_tokens"] - before["total_cached_tokens"]
+        return elapsed, steps, first, prompt_tokens, outputs, cached
+
+    once("warm")   # graphs captured, the library's kernels chosen
+    once("warm2")  # a shape is captured when it comes the second time
+    elapsed, steps, first, prompt_tokens, outputs, cached = once("run")
+    first.sort()
+    return {
+        "metric": f"output tok/s, {SHAPES[args.shape][0]} shape, {n_sessions} sessions of 4 to 8 turns, {args.concurrency} at a time",
+        "value": round(outputs / elapsed, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": 0,
+        "ms_per_step": round(1e3 * elapsed / steps, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: uniform random token ids, random weights (seed 2)",
+        "seconds": round(elapsed, 4),
+        "turns": len(first),
+        "prompt_tokens": prompt_tokens,
+        "prompt_tokens_from_prefix_cache": cached,
+        "hit_rate": round(cached / max(prompt_tokens, 1), 3),
+        "first_token_ms": {"p50": round(1e3 * first[len(first) // 2], 2), "p99": round(1e3 * first[min(len(first) - 1, int(0.99 * len(first)))], 2)},
+        "config": {
+            "model": f"{SHAPES[args.shape][0]} shape (random weights)",
+            "layers": args.layers,
+            "layers_of_full_model": SHAPES[args.shape][1]["num_hidden_layers"],
+            "sessions": n_sessions,
+            "concurrency": args.concurrency,
+            "opening": opening,
+            "turn_input": "uniform 64..256",
+            "output_len": "uniform 32..96",
+            "prefix_cache": not args.no_prefix_cache,
+            "token_budget": PROMPT_LEN,
+            "seq_len": CONTEXT,
+            "block_size": BLOCK,
+            "sampling": "greedy",
+            "parallelism": "single GPU",
+        },
+    }
+
+
 def measure_peaks() -> dict:
     """What this card reaches on the two plainest workloads, beside the published peaks the
     fractions are priced against: a device-to-device copy of 2 GiB (bytes read + written) and the
@@ -328,8 +446,11 @@ def main() -> int:
     ap.add_argument("--no-tune", action="store_true", help="leave the matrix library's kernel choice at its default")
     ap.add_argument("--only-prefill", action="store_true", help="run the prefill alone: 2048 tokens, or --prompt-len tokens in portions of 2048")
     ap.add_argument("--arrive-every", type=int, default=4, help="--workload arrivals: steps between two requests")
-    ap.add_argument("--workload", default="decode", choices=("decode", "mixed", "arrivals"),
-                    help="decode: the recorded benchmark; mixed: a continuous batch of --requests prompts of mixed lengths")
+    ap.add_argument("--workload", default="decode", choices=("decode", "mixed", "arrivals", "agent"),
+                    help="decode: the recorded benchmark; mixed: a continuous batch of --requests prompts of mixed lengths; "
+                         "arrivals: short prompts coming one by one; agent: sessions of several turns over a shared opening")
+    ap.add_argument("--concurrency", type=int, default=8, help="--workload agent: sessions that run at a time")
+    ap.add_argument("--no-prefix-cache", action="store_true", help="--workload agent: the same traffic without the prefix cache")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--peaks", action="store_true", help="measure a device copy and a large library product instead")
     ap.add_argument("--temperature", type=float, default=0.0, help="sample instead of the greedy decoding of the recorded benchmark")
@@ -344,6 +465,9 @@ def main() -> int:
 
     if args.peaks:
         print(json.dumps(measure_peaks()))
+        return 0
+    if args.workload == "agent":
+        print(json.dumps(run_agent(args)))
         return 0
     if args.workload in ("mixed", "arrivals"):
         print(json.dumps(run_mixed(args)))
