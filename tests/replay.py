@@ -277,3 +277,64 @@ def compare(got: dict, plain_logits: dict, rtol: float, atol: float) -> float:
             )
         worst = max(worst, float(err.max()))
     return worst
+
+
+def random_trace(seed: int, vocab: int):
+    """A random trace of three to six requests, at most four live at a time: portions of 2 to 200
+    tokens and single tokens in any mix, requests left out of steps, wants at random places, and
+    requests that begin as a fork of the request before them or with a share of its pages (cut at
+    any token). A request that another will derive from stays live until that one has begun.
+    Returns (steps, {id: the request's whole token sequence})."""
+    import random
+
+    rng = random.Random(seed)
+    seqs, derive = {}, {}
+    for i in range(rng.randint(3, 6)):
+        rid, prev = f"r{i}", f"r{i - 1}"
+        if i and rng.random() < 0.5 and len(seqs[prev]) > 1:
+            cut = rng.randint(1, len(seqs[prev]) - 1)
+            derive[rid] = (rng.choice(["fork", "share"]), prev, cut)
+            seqs[rid] = seqs[prev][:cut] + [rng.randrange(vocab) for _ in range(rng.randint(2, 200))]
+        else:
+            seqs[rid] = [rng.randrange(vocab) for _ in range(rng.choice([1, 3, 20, 70, 150, 400]))]
+    order = list(seqs)
+    pos, live, steps, admitted = {}, [], [], 0
+    while admitted < len(order) or live:
+        step = {"entries": [], "end": [], "fork": [], "share": []}
+        fresh = set()
+        while admitted < len(order) and len(live) < 4:
+            rid = order[admitted]
+            if rid in derive:
+                kind, src, cut = derive[rid]
+                if pos[src] < cut or src in fresh:
+                    break  # the request before has not come that far yet, or begins in this very step
+                if kind == "fork" and pos[src] == cut:
+                    step["fork"].append({"id": rid, "from": src})
+                else:
+                    step["share"].append({"id": rid, "from": src, "tokens": cut})
+                pos[rid] = cut
+            else:
+                pos[rid] = 0
+            live.append(rid)
+            fresh.add(rid)
+            admitted += 1
+        busy = [r for r in live if pos[r] < len(seqs[r])]
+        for rid in list(live):
+            left = len(seqs[rid]) - pos[rid]
+            index = order.index(rid)
+            heir = order[index + 1] if index + 1 < len(order) and index + 1 >= admitted else None
+            heir = heir if heir in derive and derive[heir][1] == rid else None
+            if left and not (len(busy) > 1 and rng.random() < 0.15):
+                n = 1 if rng.random() < 0.5 else rng.choice([2, 3, 7, 16, 33, 64, 100, 200])
+                if heir and derive[heir][0] == "fork" and pos[rid] < derive[heir][2]:
+                    n = min(n, derive[heir][2] - pos[rid])  # stop where the fork will be taken
+                n = max(1, min(n, left))
+                want = sorted(rng.sample(range(n), rng.randint(0, min(n, 3))))
+                step["entries"].append({"id": rid, "tokens": seqs[rid][pos[rid] : pos[rid] + n], "want": want})
+                pos[rid] += n
+            if pos[rid] == len(seqs[rid]) and heir is None:
+                step["end"].append(rid)
+                live.remove(rid)
+        if step["entries"] or step["end"] or step["fork"] or step["share"]:
+            steps.append(step)
+    return steps, seqs

@@ -451,6 +451,29 @@ def test_first_tokens_and_long_decoding(model_dirs, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A_peaked", "B_peaked", "C"])
+def test_random_traces_match_plain(model_dirs, name, dtype):
+    """Twenty random traces a model (replay.random_trace: portions and single tokens in any mix,
+    requests left out of steps, forks and shares cut at any token, logits wanted at random
+    places), on page pools that hold the four longest requests and little more, so that pages are
+    used again and again. Every wanted row is compared with the plain implementation."""
+    cfg, _, block_size = TINY_CONFIGS[name.split("_")[0]]
+    model = PlainQwen2(model_dirs[name])
+    rows = 0
+    for seed in range(20):
+        steps, seqs = replay.random_trace(1000 * len(name) + seed, cfg["vocab_size"])
+        longest = sorted((-(-len(t) // block_size) for t in seqs.values()), reverse=True)[:4]
+        runner = replay.make_runner(model_dirs[name], dtype, block_size, sum(longest) + len(seqs) + 2, max_model_len=1024)
+        got = replay.run_trace(runner, steps)
+        ref = {rid: model.logits(toks) for rid, toks in seqs.items()}
+        _check(got, ref, dtype)
+        assert not runner.manager.live_requests()
+        assert runner.manager.min_free_blocks() == runner.manager.num_blocks
+        rows += len(got)
+    assert rows > 500
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["B_peaked", "C"])
 def test_short_portions_behind_a_long_prefix(model_dirs, name, dtype):
     """Portions of 2 to 170 tokens behind 700 to 1100 cached ones make few attention workgroups with

@@ -97,3 +97,34 @@ def test_a_fork_copies_fixed_size_state_and_a_share_is_refused_for_such_a_model(
     with pytest.raises(ValueError, match="cannot share prefixes"):
         replayer.run_step({"share": [{"id": "c", "from": "a", "tokens": 2}]})
     assert not runner.manager.has("c")
+
+
+def test_random_traces_are_what_they_say():
+    """The traces that the GPU tests draw at random: every entry continues its request where the
+    last one stopped, at most four requests are live, a fork or a share names a live request that
+    holds the tokens it takes, and every request is run to its end and given back."""
+    from tests import replay
+
+    kinds = {"share": 0, "fork": 0, "mixed": 0}
+    for seed in range(200):
+        steps, seqs = replay.random_trace(seed, 512)
+        lengths = {}
+        for step in steps:
+            for share in step["share"]:
+                assert 0 < share["tokens"] <= lengths[share["from"]]
+                lengths[share["id"]] = share["tokens"]
+                kinds["share"] += 1
+            for fork in step["fork"]:
+                lengths[fork["id"]] = lengths[fork["from"]]
+                kinds["fork"] += 1
+            for e in step["entries"]:
+                at = lengths.get(e["id"], 0)
+                assert e["tokens"] and e["tokens"] == seqs[e["id"]][at : at + len(e["tokens"])]
+                assert all(0 <= w < len(e["tokens"]) for w in e["want"])
+                lengths[e["id"]] = at + len(e["tokens"])
+            assert len(lengths) <= 4
+            kinds["mixed"] += len(step["entries"]) > 1 and any(len(e["tokens"]) > 1 for e in step["entries"])
+            for rid in step["end"]:
+                assert lengths.pop(rid) == len(seqs[rid])
+        assert not lengths
+    assert min(kinds.values()) > 50
