@@ -237,6 +237,20 @@ class CacheManager:
                 return False
         return True
 
+    def can_extend_all(self, spans) -> bool:
+        """Can every one of these requests write its positions at once? ``spans``:
+        ``(seq_id, computed, upto)`` each. (``can_extend`` answers for one request alone: three
+        requests at a page's edge with two pages free can each, but not all.)"""
+        need = [0] * len(self.pools)
+        for seq_id, computed, upto in spans:
+            rec = self._requests[seq_id]
+            if self._fits_as_is(rec, computed, upto):
+                continue
+            for g in range(len(self.pools)):
+                new, cow = self._growth(rec, g, computed, upto)
+                need[g] += new + (1 if cow else 0)
+        return all(n <= pool.num_free for n, pool in zip(need, self.pools))
+
     def extend(self, seq_id: str, computed: int, upto: int) -> list[tuple[int, int, int]]:
         """Back positions [computed, upto). Returns ``(group, src_page, dst_page)`` copies the
         caller must perform on the device before the step runs."""

@@ -257,9 +257,9 @@ class Scheduler:
             if (len(seq.output_token_ids) + 1 >= seq.sampling_params.max_tokens
                     or len(seq) + 1 >= limit):
                 return None  # its last token is being made right now
-        for p in prev.portions:
-            if not self.manager.can_extend(p.seq.seq_id, p.start + 1, p.start + 2):
-                return None
+        # all of them together: pages that are there for each alone may not be there for all
+        if not self.manager.can_extend_all([(p.seq.seq_id, p.start + 1, p.start + 2) for p in prev.portions]):
+            return None
         out = SchedulerOutput(version=self.version)
         for p in prev.portions:
             out.copies += self.manager.extend(p.seq.seq_id, p.start + 1, p.start + 2)

@@ -387,7 +387,8 @@ def test_sampled_tokens_do_not_depend_on_steps_queued_ahead(model_dirs):
     assert len({tuple(v) for v in ahead.values()}) == 3
 
 
-@pytest.mark.parametrize("seed", [0, 1])
+# seeds 12 and 15 run out of pages for three requests at once while a step is decided ahead
+@pytest.mark.parametrize("seed", [0, 1, 12, 15])
 def test_long_random_session_equals_every_request_alone(model_dirs, seed):
     """Arrivals at random times, stop tokens, aborts, so few pages that requests are preempted,
     shared prefixes, steps queued ahead: every request that finishes gives the tokens and the

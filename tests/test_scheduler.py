@@ -446,3 +446,27 @@ def test_schedule_ahead_never_preempts_or_evicts():
     assert sched.stats.num_preempted_total == before and len(sched.running) == 2
     out = sched.schedule()                      # the ordinary schedule preempts the later request
     assert ids(out.preempted) == ["b"]
+
+
+def test_schedule_ahead_counts_the_pages_of_all_requests_together():
+    # 7 pages of 4: three requests of 4 tokens hold a page each and decode their fifth token into a
+    # second one (6 held); at position 8 each needs a third page and one is free: each alone could
+    # go on, all three cannot, and looking ahead must leave that to the ordinary schedule
+    # untouched (it once took pages for the first requests and then failed on the last)
+    sched, manager, _ = make_env(num_blocks=7, budget=16, chunked=True)
+    seqs = [make_seq(name, range(4), float(i)) for i, name in enumerate("abc")]
+    for seq in seqs:
+        sched.add_seq(seq)
+    apply(sched, sched.schedule())              # the prompts
+    for _ in range(4):                          # positions 4 to 7
+        out = sched.schedule()
+        assert len(out.portions) == 3
+        apply(sched, out)
+    assert manager.min_free_blocks() == 1
+    assert all(manager.can_extend(s.seq_id, 8, 9) for s in seqs)
+    assert not manager.can_extend_all([(s.seq_id, 8, 9) for s in seqs])
+    held = {s.seq_id: list(manager.block_table(s.seq_id, 0)) for s in seqs}
+    assert sched.schedule_ahead(out) is None
+    assert manager.min_free_blocks() == 1 and held == {s.seq_id: list(manager.block_table(s.seq_id, 0)) for s in seqs}
+    out = sched.schedule()                      # the ordinary schedule makes room by preempting
+    assert ids(out.preempted) and len(out.portions) + len(out.preempted) >= 2
