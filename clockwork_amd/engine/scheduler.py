@@ -15,7 +15,8 @@ New here: a prompt no longer has to fit the token budget whole. A request
 contributes ``min(remaining, budget left, max_prefill_chunk)`` tokens per step, so
 running requests are either *prefilling* (more than one token still to run) or
 *decoding* (exactly one). With ``enable_chunked_prefill`` off the reference's
-behaviour returns: a prompt is admitted only whole.
+behaviour returns: a prompt is admitted only whole (a request that was preempted and has
+outgrown the budget by what it generated is the exception: it runs again in portions).
 
 When pages run out: before a request is refused admission and before a running
 request is preempted, idle blocks of the prefix cache are evicted, oldest first.
@@ -159,6 +160,14 @@ class Scheduler:
                 return False
         return True
 
+    def _whole_only(self, seq: Sequence, remaining: int) -> bool:
+        """Without chunked prefill a prompt runs whole or not at all (the reference's rule). A
+        request that is run again after a preemption has grown by what it generated and may no
+        longer fit the token budget: that one runs in portions, or it could never go on."""
+        if self.cfg.enable_chunked_prefill:
+            return False
+        return not (seq.output_token_ids and remaining > self.cfg.max_num_batched_tokens)
+
     def _serve_running(self, out: SchedulerOutput) -> None:
         """Every running request, in order of arrival, gets its next tokens: one if it decodes
         (always served), else a portion of what it still has to run, as the budget allows."""
@@ -169,7 +178,7 @@ class Scheduler:
             seq = unserved.popleft()
             remaining = seq.num_uncomputed_tokens()
             n = 1 if remaining == 1 else self._chunk(remaining, budget - out.num_batched_tokens)
-            if remaining > 1 and not self.cfg.enable_chunked_prefill and n < remaining:
+            if remaining > 1 and n < remaining and self._whole_only(seq, remaining):
                 n = 0  # a prompt runs whole or not at all
             if n <= 0:
                 kept.append(seq)  # stays running, contributes nothing this step
@@ -197,7 +206,7 @@ class Scheduler:
         remaining = len(seq) - cached
         budget_left = self.cfg.max_num_batched_tokens - out.num_batched_tokens
         n = self._chunk(remaining, budget_left)
-        if not self.cfg.enable_chunked_prefill and n < remaining:
+        if n < remaining and self._whole_only(seq, remaining):
             n = 0
         fits = n > 0
         if fits:

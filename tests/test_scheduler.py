@@ -470,3 +470,32 @@ def test_schedule_ahead_counts_the_pages_of_all_requests_together():
     assert manager.min_free_blocks() == 1 and held == {s.seq_id: list(manager.block_table(s.seq_id, 0)) for s in seqs}
     out = sched.schedule()                      # the ordinary schedule makes room by preempting
     assert ids(out.preempted) and len(out.portions) + len(out.preempted) >= 2
+
+
+def test_a_preempted_request_that_outgrew_the_budget_runs_again_in_portions():
+    # chunked prefill off, a budget of 8 tokens, 5 pages of 4. Two prompts of 7 tokens run whole,
+    # one after the other. Both generate; at position 8 each needs a third page and there is one:
+    # b, the later arrival, is preempted with 7 + 2 = 9 tokens, more than a step may hold. Once a
+    # is finished b must come back, in a portion of 8 tokens and then the rest, not wait forever.
+    sched, manager, _ = make_env(num_blocks=5, budget=8, chunked=False)
+    a, b = make_seq("a", range(7), 0.0, max_tokens=6), make_seq("b", range(7), 1.0, max_tokens=6)
+    sched.add_seq(a)
+    sched.add_seq(b)
+    preempted = False
+    for _ in range(12):
+        out = engine_step(sched)
+        preempted = preempted or ids(out.preempted) == ["b"]
+        if a.is_finished():
+            break
+    assert preempted and a.is_finished() and b.status is SequenceStatus.PREEMPTED and len(b) == 9
+    out = engine_step(sched)
+    assert [(p.seq.seq_id, p.start, p.num_tokens, p.samples) for p in out.portions] == [("b", 0, 8, False)]
+    out = engine_step(sched)
+    assert [(p.seq.seq_id, p.start, p.num_tokens, p.samples) for p in out.portions] == [("b", 8, 1, True)]
+    while not b.is_finished():
+        engine_step(sched)
+    assert len(b.output_token_ids) == 6 and manager.min_free_blocks() == 5
+    # a prompt that is longer than the budget still never runs without chunked prefill
+    sched2, _, _ = make_env(num_blocks=16, budget=8, chunked=False)
+    sched2.add_seq(make_seq("long", range(9), 0.0))
+    assert not sched2.schedule().portions
