@@ -279,12 +279,12 @@ def compare(got: dict, plain_logits: dict, rtol: float, atol: float) -> float:
     return worst
 
 
-def random_trace(seed: int, vocab: int):
+def random_trace(seed: int, vocab: int, kinds=("fork", "share")):
     """A random trace of three to six requests, at most four live at a time: portions of 2 to 200
     tokens and single tokens in any mix, requests left out of steps, wants at random places, and
     requests that begin as a fork of the request before them or with a share of its pages (cut at
-    any token). A request that another will derive from stays live until that one has begun.
-    Returns (steps, {id: the request's whole token sequence})."""
+    any token; ``kinds`` says which of the two a trace may hold). A request that another will derive
+    from stays live until that one has begun. Returns (steps, {id: the request's whole token sequence})."""
     import random
 
     rng = random.Random(seed)
@@ -292,8 +292,11 @@ def random_trace(seed: int, vocab: int):
     for i in range(rng.randint(3, 6)):
         rid, prev = f"r{i}", f"r{i - 1}"
         if i and rng.random() < 0.5 and len(seqs[prev]) > 1:
-            cut = rng.randint(1, len(seqs[prev]) - 1)
-            derive[rid] = (rng.choice(["fork", "share"]), prev, cut)
+            kind = rng.choice(list(kinds))
+            # a fork is taken where the request before stands: not before that one's own beginning
+            first = derive[prev][2] if kind == "fork" and prev in derive else 1
+            cut = rng.randint(max(1, first), len(seqs[prev]) - 1)
+            derive[rid] = (kind, prev, cut)
             seqs[rid] = seqs[prev][:cut] + [rng.randrange(vocab) for _ in range(rng.randint(2, 200))]
         else:
             seqs[rid] = [rng.randrange(vocab) for _ in range(rng.choice([1, 3, 20, 70, 150, 400]))]
@@ -308,7 +311,8 @@ def random_trace(seed: int, vocab: int):
                 kind, src, cut = derive[rid]
                 if pos[src] < cut or src in fresh:
                     break  # the request before has not come that far yet, or begins in this very step
-                if kind == "fork" and pos[src] == cut:
+                if kind == "fork":
+                    assert pos[src] == cut, "the request before ran past the place of the fork"
                     step["fork"].append({"id": rid, "from": src})
                 else:
                     step["share"].append({"id": rid, "from": src, "tokens": cut})
@@ -324,7 +328,8 @@ def random_trace(seed: int, vocab: int):
             index = order.index(rid)
             heir = order[index + 1] if index + 1 < len(order) and index + 1 >= admitted else None
             heir = heir if heir in derive and derive[heir][1] == rid else None
-            if left and not (len(busy) > 1 and rng.random() < 0.15):
+            waits = heir is not None and derive[heir][0] == "fork" and pos[rid] == derive[heir][2]  # for the fork to be taken
+            if left and not waits and not (len(busy) > 1 and rng.random() < 0.15):
                 n = 1 if rng.random() < 0.5 else rng.choice([2, 3, 7, 16, 33, 64, 100, 200])
                 if heir and derive[heir][0] == "fork" and pos[rid] < derive[heir][2]:
                     n = min(n, derive[heir][2] - pos[rid])  # stop where the fork will be taken

@@ -378,6 +378,22 @@ def test_a_toy_architecture_registers_builds_and_steps(toy_dir, dtype, mode):
     assert [p.num_free for p in runner.manager.pools] == [64, 64]
 
 
+def test_random_traces_of_the_toy_architecture(toy_dir):
+    """Fifteen random traces (replay.random_trace with forks only: this model's cache cannot share
+    prefixes) in float32: state copied at a fork, pages behind the window given back while the
+    request runs, a borrowed cache, on pools that hold little more than four requests."""
+    for seed in range(15):
+        steps, seqs = replay.random_trace(seed, 300, kinds=("fork",))
+        block_size = (4, 8, 16)[seed % 3]
+        longest = sorted((-(-len(t) // block_size) for t in seqs.values()), reverse=True)[:4]
+        runner = replay.make_runner(toy_dir, "float32", block_size, sum(longest) + len(seqs) + 2, max_model_len=1024)
+        got = replay.run_trace(runner, steps)
+        ref = {rid: _toy_plain_logits(toy_dir, toks) for rid, toks in seqs.items()}
+        replay.compare(got, ref, rtol=1e-5, atol=1e-5)
+        assert not runner.manager.live_requests()
+        assert all(p.num_free == runner.manager.num_blocks for p in runner.manager.pools)
+
+
 # ---------------------------------------------------------------------------------- a second toy
 @dataclass(frozen=True)
 class ScaledEmbeddingSpec:
