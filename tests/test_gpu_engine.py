@@ -460,3 +460,69 @@ def test_long_random_session_equals_every_request_alone(model_dirs, seed):
         assert finals[rid][0] == want, rid
         checked += 1
     assert checked == 12
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_engine_configurations_and_sessions(model_dirs, seed):
+    """Engine options drawn at random (page size, pages, token budget, requests at a time, prefix
+    cache, chunked prefill, looking ahead, watermark) and a session drawn at random (prompts of 1
+    to 180 tokens that share openings of 0 to 64, greedy or seeded temperature / top-k / top-p
+    sampling, stop tokens, 1 to 90 tokens, arrivals spread over the steps, a request aborted now
+    and then), in float32: every request that finishes gives the tokens and the reason it gives
+    alone, an aborted one gives nothing more, and every page comes back."""
+    import random
+
+    from clockwork_amd.engine.llm_engine import LLMEngine
+
+    rng = random.Random(seed)
+    name = rng.choice(["A", "B", "C"])
+    vocab = TINY_CONFIGS[name][0]["vocab_size"]
+    block_size, budget = rng.choice([4, 8, 16]), rng.choice([16, 48, 96, 256])
+    options = dict(dtype="float32", block_size=block_size, watermark=rng.choice([0.0, 0.02]), max_model_len=300,
+                   max_num_seqs=rng.choice([2, 4, 12]), max_num_batched_tokens=budget,
+                   enable_prefix_cache=rng.random() < 0.6, enable_chunked_prefill=rng.random() < 0.7,
+                   lookahead=rng.random() < 0.7, seed=seed)
+    if not options["enable_chunked_prefill"]:
+        options["max_num_batched_tokens"] = max(budget, 200)  # every prompt fits a step whole
+    opening = [rng.randrange(vocab) for _ in range(64)]
+    requests = []
+    for i in range(rng.randint(4, 30)):
+        prompt = (opening[: rng.choice([0, 0, 8, 33, 64])] + [rng.randrange(vocab) for _ in range(rng.choice([1, 2, 9, 30, 70, 150]))])[:180]
+        how = dict(temperature=0.0)
+        if rng.random() < 0.5:
+            how = dict(temperature=rng.choice([0.5, 1.0, 1.5]), top_k=rng.choice([-1, 1, 5, 50]), top_p=rng.choice([1.0, 0.9, 0.5]),
+                       seed=rng.randrange(1000))
+        stops = [rng.randrange(vocab) for _ in range(rng.choice([0, 0, 20]))]
+        requests.append((f"q{i}", prompt, dict(max_tokens=rng.choice([1, 2, 10, 40, 90]), stop_token_ids=stops, ignore_eos=True, **how)))
+    longest = max(len(prompt) + how["max_tokens"] for _, prompt, how in requests)
+    num_blocks = max(-(-longest // block_size) + 2, rng.choice([20, 40, 100]))  # the longest request fits alone
+    eng = LLMEngine(EngineConfig.defaults(str(model_dirs[name]), num_blocks=num_blocks, **options))
+    finals, pending, live, aborted = {}, list(requests), set(), set()
+    for _ in range(20000):
+        if not pending and not eng.has_unfinished_requests():
+            break
+        for _ in range(rng.choice([0, 1, 1, 3])):
+            if pending:
+                rid, prompt, how = pending.pop(0)
+                eng.add_request(rid, prompt_token_ids=prompt, sampling_params=SamplingParams(**how))
+                live.add(rid)
+        if live and rng.random() < 0.05:
+            victim = rng.choice(sorted(live))
+            eng.abort_request(victim)
+            aborted.add(victim)
+            live.discard(victim)
+        if eng.has_unfinished_requests():
+            for out in eng.step():
+                assert out.request_id not in aborted
+                if out.finished:
+                    finals[out.request_id] = (out.token_ids, out.finish_reason)
+                    live.discard(out.request_id)
+    assert not pending and not eng.has_unfinished_requests() and len(finals) + len(aborted) == len(requests)
+    eng.prefix_cache.reset()
+    assert eng.manager.min_free_blocks() == eng.manager.num_blocks
+    alone = LLMEngine(EngineConfig.defaults(str(model_dirs[name]), num_blocks=-(-longest // block_size) + 4,
+                                            **dict(options, max_num_seqs=2, enable_prefix_cache=False, lookahead=False)))
+    for rid, prompt, how in requests:
+        if rid not in aborted:
+            out = alone.generate([prompt], SamplingParams(**how))[0]
+            assert (out.token_ids, out.finish_reason) == finals[rid], rid
