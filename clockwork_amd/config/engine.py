@@ -62,8 +62,8 @@ class CacheConfig:
 class SchedulerConfig:
     """Batching limits (clockwork/config.py:42-47) plus chunked prefill.
 
-    ``max_prefill_chunk`` caps the tokens one request contributes to a step;
-    0 means "as many as the token budget allows". With
+    ``max_prefill_chunk`` caps the tokens one request contributes to a step
+    (only with chunked prefill on); 0 means "as many as the token budget allows". With
     ``enable_chunked_prefill`` off a prompt is admitted only whole, as in the
     reference (clockwork/scheduler/scheduler.py:120-146).
     """

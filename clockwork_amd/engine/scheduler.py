@@ -141,7 +141,9 @@ class Scheduler:
     # ------------------------------------------------------------------ one step
     def _chunk(self, remaining: int, budget_left: int) -> int:
         n = min(remaining, budget_left)
-        if self.cfg.max_prefill_chunk > 0:
+        # the cap on a portion belongs to chunked prefill: without it a prompt runs whole, so a
+        # cap would only keep every prompt longer than itself from ever running
+        if self.cfg.max_prefill_chunk > 0 and self.cfg.enable_chunked_prefill:
             n = min(n, self.cfg.max_prefill_chunk)
         return n
 

@@ -499,3 +499,76 @@ def test_a_preempted_request_that_outgrew_the_budget_runs_again_in_portions():
     sched2, _, _ = make_env(num_blocks=16, budget=8, chunked=False)
     sched2.add_seq(make_seq("long", range(9), 0.0))
     assert not sched2.schedule().portions
+
+
+# 1424 and 1950: a step decided ahead for requests that each alone, but not all together, find a page
+@pytest.mark.parametrize("seed", [*range(300), 1424, 1950])
+def test_random_sessions_end_with_every_page_back(seed):
+    """Scheduler options and sessions drawn at random, run as the engine runs them (a step decided
+    ahead is used when nothing changed meanwhile; when nothing can run, the idle prefix blocks are
+    evicted once): requests arrive over time, stop at random tokens or at their length, are aborted
+    now and then. No step raises, every request ends, the page pools pass their audit after every
+    step and are whole at the end, and a request never holds fewer pages than its cached tokens need."""
+    import random
+
+    rng = random.Random(seed)
+    chunked = rng.random() < 0.7
+    budget = rng.choice([8, 16, 48, 96])
+    max_prompt = 60
+    if not chunked:
+        budget = max(budget, max_prompt)
+    num_blocks = rng.choice([24, 32, 64, 200])  # pages of 4: the longest request (60 + 40 tokens) fits alone
+    sched, manager, cache = make_env(num_blocks=max(num_blocks, (max_prompt + 40) // BS + 2), max_num_seqs=rng.choice([2, 4, 12]),
+                                     budget=budget, watermark=rng.choice([0.0, 0.05]), prefix=rng.random() < 0.6,
+                                     chunked=chunked, chunk=rng.choice([0, 0, 7]))
+    opening = [rng.randrange(50) for _ in range(32)]
+    pending = []
+    for i in range(rng.randint(3, 40)):
+        prompt = (opening[: rng.choice([0, 0, 4, 17, 32])] + [rng.randrange(50) for _ in range(rng.choice([1, 2, 9, 30]))])[:max_prompt]
+        pending.append(make_seq(f"q{i}", prompt, float(i), max_tokens=rng.choice([1, 2, 10, 40])))
+    seqs = list(pending)
+
+    def run(out):
+        """The stand-in for the step: tokens drawn at random, one in ten of them a stop token."""
+        for p in out.portions:
+            p.seq.num_computed_tokens = p.start + p.num_tokens
+            if p.samples:
+                p.seq.append_token(rng.randrange(50))
+                if rng.random() < 0.1:
+                    p.seq.status = SequenceStatus.FINISHED_STOPPED
+                elif len(p.seq.output_token_ids) >= p.seq.sampling_params.max_tokens:
+                    p.seq.status = SequenceStatus.FINISHED_LENGTH
+        sched.free_finished()
+
+    ahead = None
+    for _ in range(5000):
+        if not pending and not sched.has_unfinished():
+            break
+        for _ in range(rng.choice([0, 0, 1, 2])):
+            if pending:
+                sched.add_seq(pending.pop(0))
+        live = sched.running + sched.waiting
+        if live and rng.random() < 0.04:
+            sched.abort(rng.choice(live).seq_id)
+        if not sched.has_unfinished():
+            continue
+        if ahead is not None and ahead.version == sched.version:
+            out = ahead
+            sched.commit_ahead(out)
+        else:
+            out = sched.schedule()
+            if not out.portions and not out.preempted and cache is not None and cache.evict(manager.num_blocks) > 0:
+                out = sched.schedule()
+            assert out.portions or out.preempted, "nothing runs although requests wait and the prefix cache is empty"
+        for p in out.portions:
+            held = len(manager.block_table(p.seq.seq_id, 0)) * BS
+            assert held >= p.start + p.num_tokens, f"{p.seq.seq_id} runs tokens that no page backs"
+        ahead = sched.schedule_ahead(out) if out.portions and rng.random() < 0.8 else None
+        run(out)
+        manager.audit()
+    assert not pending and not sched.has_unfinished(), "the session does not end"
+    assert all(s.is_finished() for s in seqs)
+    if cache is not None:
+        cache.reset()
+    manager.audit()
+    assert manager.min_free_blocks() == manager.num_blocks
