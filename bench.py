@@ -281,7 +281,8 @@ def run_agent(args) -> dict:
     from clockwork_amd.engine.llm_engine import LLMEngine
     from clockwork_amd.engine.sequence import SamplingParams
 
-    n_sessions, opening = args.requests, 1024
+    n_sessions, opening = args.requests, args.opening
+    args.prompt_len = max(args.prompt_len, opening)  # the context is sized for twice this
     cfg, runner = build_runner(args, prefix_cache=not args.no_prefix_cache, max_batch=max(args.concurrency, 8))
     vocab = runner.spec.vocab_size
     gen = torch.Generator().manual_seed(11)
@@ -378,7 +379,7 @@ def run_agent(args) -> dict:
             "output_len": "uniform 32..96",
             "prefix_cache": not args.no_prefix_cache,
             "token_budget": PROMPT_LEN,
-            "seq_len": CONTEXT,
+            "seq_len": context_of(args),
             "block_size": BLOCK,
             "sampling": "greedy",
             "parallelism": "single GPU",
@@ -450,6 +451,7 @@ def main() -> int:
                     help="decode: the recorded benchmark; mixed: a continuous batch of --requests prompts of mixed lengths; "
                          "arrivals: short prompts coming one by one; agent: sessions of several turns over a shared opening")
     ap.add_argument("--concurrency", type=int, default=8, help="--workload agent: sessions that run at a time")
+    ap.add_argument("--opening", type=int, default=1024, help="--workload agent: tokens that every session opens with")
     ap.add_argument("--no-prefix-cache", action="store_true", help="--workload agent: the same traffic without the prefix cache")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--peaks", action="store_true", help="measure a device copy and a large library product instead")
