@@ -331,9 +331,16 @@ class CacheManager:
         for pool, page in zip(self.pools, handle):
             pool.drop(page)
 
+    def share_handles(self, handles: Sequence[tuple[int, ...]]) -> None:
+        """``share_handle`` for many handles at once."""
+        for g, pool in enumerate(self.pools):
+            pool.share_many(handle[g] for handle in handles)
+
     def handles(self, seq_id: str, num_blocks: int) -> list[tuple[int, ...]]:
         rec = self._requests[seq_id]
-        return [tuple(t[b] for t in rec.tables) for b in range(num_blocks)]
+        if any(len(t) < num_blocks for t in rec.tables):
+            raise IndexError(f"sequence {seq_id} holds fewer than {num_blocks} blocks")
+        return list(zip(*(t[:num_blocks] for t in rec.tables)))
 
     # ------------------------------------------------------------------ addressing
     def slot_mapping(self, seq_id: str, start: int, end: int, group: int = 0) -> list[int]:

@@ -56,13 +56,17 @@ class PrefixMatch:
 
 
 class PrefixCache:
-    def __init__(self, block_size: int, share: Callable, drop: Callable, enabled: bool = True) -> None:
+    def __init__(self, block_size: int, share: Callable, drop: Callable, enabled: bool = True,
+                 share_many: Optional[Callable] = None) -> None:
+        """``share(handle)`` / ``drop(handle)`` take and give back a hold on a block's pages;
+        ``share_many(handles)``, when given, takes the holds of a whole match at once."""
         if block_size <= 0:
             raise ValueError(f"block_size must be positive, got {block_size}")
         self.block_size = block_size
         self.enabled = enabled
         self._share = share
         self._drop = drop
+        self._share_many = share_many
         self.stats = PrefixCacheStats()
         self._root = _Node(None, (), None)
         self._tick = 0
@@ -111,8 +115,11 @@ class PrefixCache:
             node = child
         if not handles:
             return PrefixMatch()
-        for handle in handles:
-            self._share(handle)
+        if self._share_many is not None:
+            self._share_many(handles)
+        else:
+            for handle in handles:
+                self._share(handle)
         node.locks += 1
         matched = len(handles) * self.block_size
         self.stats.hit_tokens += matched

@@ -12,6 +12,7 @@ from __future__ import annotations
 import itertools
 from typing import Optional
 
+import numpy as np
 import torch
 
 from clockwork_amd.cache.prefix import PrefixCache
@@ -79,6 +80,7 @@ class LLMEngine:
             share=self.manager.share_handle,
             drop=self.manager.drop_handle,
             enabled=cfg.cache.enable_prefix_cache and self.manager.supports_prefix_sharing,
+            share_many=self.manager.share_handles,
         )
         self.scheduler = Scheduler(cfg.scheduler, self.manager, self.prefix_cache)
         self.sampler = Sampler(self.runner.device, cfg.model.seed)
@@ -131,13 +133,18 @@ class LLMEngine:
             if self.tokenizer is None:
                 raise ValueError("a text prompt needs a tokenizer; pass prompt_token_ids instead")
             prompt_token_ids = self.tokenizer.encode(prompt)
-        prompt_token_ids = [int(t) for t in prompt_token_ids]
-        if not prompt_token_ids:
+        # a long prompt is checked as an array, not token by token
+        ids = np.asarray(prompt_token_ids)
+        if ids.ndim != 1:
+            raise ValueError("prompt_token_ids must be a flat sequence of token ids")
+        if ids.size == 0:
             raise ValueError("prompt must contain at least one token")
+        ids = ids.astype(np.int64)
         vocab = self.runner.spec.vocab_size
-        bad = [t for t in prompt_token_ids if not 0 <= t < vocab]
-        if bad:
-            raise ValueError(f"token ids {bad[:5]} lie outside the vocabulary [0, {vocab})")
+        outside = (ids < 0) | (ids >= vocab)
+        if outside.any():
+            raise ValueError(f"token ids {ids[outside][:5].tolist()} lie outside the vocabulary [0, {vocab})")
+        prompt_token_ids = ids.tolist()
         if len(prompt_token_ids) >= self.cfg.model.max_model_len:
             raise ValueError(
                 f"prompt of {len(prompt_token_ids)} tokens leaves no room to generate "

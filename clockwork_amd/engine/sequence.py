@@ -46,7 +46,9 @@ class Sequence:
     def __init__(self, seq_id: str, prompt_token_ids: list[int], sampling_params: Optional[SamplingParams] = None,
                  arrival_time: Optional[float] = None) -> None:
         self.seq_id = seq_id
-        self.prompt_token_ids = [int(t) for t in prompt_token_ids]
+        # plain ints (a list of them is taken as it is: an engine's prompt may be tens of thousands long)
+        plain = type(prompt_token_ids) is list and set(map(type, prompt_token_ids)) <= {int}
+        self.prompt_token_ids = list(prompt_token_ids) if plain else [int(t) for t in prompt_token_ids]
         self.output_token_ids: list[int] = []
         self.sampling_params = sampling_params or SamplingParams()
         self.arrival_time = arrival_time if arrival_time is not None else time.monotonic()

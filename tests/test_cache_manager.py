@@ -99,6 +99,51 @@ def test_pool_fuzz_against_a_dict_model():
 
 
 # ------------------------------------------------------------------ groups
+@pytest.mark.parametrize("seed", range(6))
+def test_many_holds_at_once_equal_one_hold_after_the_other(seed):
+    """The array form of a request's holds leaves the counts and the order of the free stack
+    that a loop of single holds leaves, also when a page is named twice or is not in use."""
+    rng = random.Random(seed)
+    num_pages = rng.choice([12, 40, 97])
+    fast, slow = PagePool(num_pages, 4), PagePool(num_pages, 4)
+    for pool in (fast, slow):
+        pool.take_many(num_pages - 3)
+    for _ in range(60):
+        in_use = [p for p in range(num_pages) if slow.refcount(p) > 0]
+        step = rng.choice([1, -1])
+        pages = rng.sample(in_use, rng.randint(0, len(in_use))) if in_use else []
+        if pages and rng.random() < 0.15:
+            pages.append(rng.choice(pages))  # the same page twice
+        failed = []
+        for pool, call in ((fast, lambda: fast.hold_many(pages, step)),
+                           (slow, lambda: [slow.hold(page, step) for page in pages])):
+            try:
+                call()
+                failed.append(None)
+            except ValueError as err:
+                failed.append(str(err))
+        assert failed[0] == failed[1]
+        if failed[0] is not None:  # a loop stops half way, the array form before it starts
+            fast, slow = PagePool(num_pages, 4), PagePool(num_pages, 4)
+            for pool in (fast, slow):
+                pool.take_many(num_pages - 3)
+            continue
+        assert fast._holders.tolist() == slow._holders.tolist()
+        assert fast._idle[: fast.num_free].tolist() == slow._idle[: slow.num_free].tolist()
+        fast.audit()
+        if slow.num_free > 4 and rng.random() < 0.5:
+            n = rng.randint(1, slow.num_free)
+            assert fast.take_many(n) == slow.take_many(n)
+    with pytest.raises(ValueError, match="no holder"):
+        free_page = PagePool(16, 4)
+        held = free_page.take_many(10)
+        free_page.drop(held[3])
+        free_page.hold_many(held, -1)
+    assert free_page.refcount(held[0]) == 1  # refused before anything changed
+    with pytest.raises(ValueError, match="outside"):
+        free_page.hold_many([0, 1, 2, 4, 5, 6, 7, 8, 99], 1)
+
+
 def test_layers_with_the_same_need_share_a_group():
     needs = [KVPagesSpec(2, 16), KVPagesSpec(2, 16, window=8), KVPagesSpec(2, 16), None, StateSpec((4,)), KVPagesSpec(2, 16, window=8)]
     groups = plan_groups(needs)
