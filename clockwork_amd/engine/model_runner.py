@@ -86,7 +86,7 @@ class ModelRunner:
         self.model_config = self.arch.parse_config(self.config_dict)
         self.spec = self.arch.build_spec(self.model_config)
         self.model = DecoderModel(self.spec)
-        ops.preload(self.model.kernel_libraries(), tiled_products=cfg.model.hip_products)
+        ops.preload(self.model.kernel_libraries(), tiled_products=cfg.model.hip_products or self.dtype == torch.bfloat16)
         plan = self.arch.weight_plan(self.model_config, self.spec)
         params = load_parameters(
             cfg.model.model, plan, self.model.param_specs(), self.dtype, self.device, source=weight_source

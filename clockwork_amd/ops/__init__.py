@@ -65,8 +65,9 @@ def _load(name: str, head_dim: int | None = None) -> ctypes.CDLL:
 def preload(libraries=(), tiled_products: bool = False, sampling: bool = False) -> None:
     """Build (side by side, if several are missing) and load what a model runs: the common
     kernels, the products and the ``libraries`` its parts name, as (name, head size or None)
-    pairs, e.g. ("attention", 128); the tiled product and the sampling kernels only for a caller
-    that uses them."""
+    pairs, e.g. ("attention", 128); the tiled products (a bfloat16 model's gate/up product of a
+    long portion, and every large product with ``hip_products``) and the sampling kernels only for
+    a caller that uses them."""
     jobs = [("core", None), ("gemm", None)]
     if tiled_products:
         jobs.append(("gemm_tile", None))
@@ -109,6 +110,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
         },
         "gemm_tile": {
             "cw_gemm_bf16_tiled": [I, P, L, P, P, I, P, L, I, I, I, P],
+            "cw_gemm_bf16_wide_tiles": [I, I, I, I, L],
+            "cw_gemm_bf16_wide": [I, P, L, P, P, I, P, L, I, I, I, I, P],
         },
         "sampling": {
             "cw_argmax_chunks": [I],
@@ -445,10 +448,12 @@ STREAM_MAX_ROWS = 64
 FUSED_QKV_MAX_WEIGHTS = 8 << 20
 
 
-def linear_tiled(x: torch.Tensor, weight: torch.Tensor, bias=None, swiglu: bool = False) -> torch.Tensor:
+def linear_tiled(x: torch.Tensor, weight: torch.Tensor, bias=None, swiglu: bool = False, wide=None) -> torch.Tensor:
     """y = x @ weight.T (+ bias), or with ``swiglu`` silu(x @ gate.T) * (x @ up.T) for weight =
-    [gate; up], through the LDS-tiled matrix-core kernel for many bfloat16 rows (csrc/gemm_tile.hip).
-    The rows of x may have a stride (a slice of a wider buffer)."""
+    [gate; up], through the LDS-tiled matrix-core kernels for many bfloat16 rows (csrc/gemm_tile.hip):
+    the one with 256 x 192 tiles where it takes the shape and has tiles enough to fill the GPU, the
+    one with 128 x 128 tiles otherwise (``wide``: True or False to say which). The rows of x may
+    have a stride (a slice of a wider buffer)."""
     _gpu(weight, bias)
     if not (x.is_cuda and x.dim() == 2):
         raise KernelError("x must be a 2-d tensor on the GPU")
@@ -464,13 +469,49 @@ def linear_tiled(x: torch.Tensor, weight: torch.Tensor, bias=None, swiglu: bool 
         if not (bias.numel() == N and bias.dtype in (torch.bfloat16, torch.float32)):
             raise KernelError("bias must be [N] bfloat16 or float32")
     out = torch.empty((M, N // 2 if swiglu else N), dtype=torch.bfloat16, device=x.device)
-    _check(
-        _load("gemm_tile").cw_gemm_bf16_tiled(
-            2 if swiglu else 0, _ptr(x), x.stride(0), _ptr(weight), _ptr(bias),
-            int(bias is not None and bias.dtype == torch.float32), _ptr(out), out.shape[1], M, N, K, _stream()),
-        "gemm_bf16_tiled",
-    )
+    lib = _load("gemm_tile")
+    mode = 2 if swiglu else 0
+    bias_f32 = int(bias is not None and bias.dtype == torch.float32)
+    if wide is None:
+        wide = lib.cw_gemm_bf16_wide_tiles(mode, M, N, K, x.stride(0)) >= WIDE_MIN_TILES
+    if wide:
+        _check(lib.cw_gemm_bf16_wide(mode, _ptr(x), x.stride(0), _ptr(weight), _ptr(bias), bias_f32, _ptr(out), out.shape[1],
+                                     M, N, K, _compute_units(x.device), _stream()), "gemm_bf16_wide")
+    else:
+        _check(lib.cw_gemm_bf16_tiled(mode, _ptr(x), x.stride(0), _ptr(weight), _ptr(bias), bias_f32, _ptr(out), out.shape[1],
+                                      M, N, K, _stream()), "gemm_bf16_tiled")
     return out
+
+
+# the wide-tile kernel runs one workgroup per compute unit: with fewer tiles than this the
+# 128 x 128 kernel, whose tiles are a quarter of the size, fills the GPU better
+WIDE_MIN_TILES = 64
+# The engine takes the wide-tile kernel for the gate/up product by itself (no ``hip_products``)
+# where it beats the library product followed by the gate kernel. Measured on an MI355X over the
+# Qwen2.5 layer shapes from 0.5B to 72B with 256 to 4096 rows: with 180 tiles or more (seven tenths
+# of the compute units busy in the last round) and 1024 rows or more it is 5 to 25 % faster; with
+# fewer rows the product is bound by reading W once, which the library does better for the large
+# shapes (and 512 rows win only for the small ones).
+WIDE_SWIGLU_MIN_TILES = 180
+WIDE_SWIGLU_MIN_ROWS = 1024
+WIDE_SWIGLU_SMALL_WEIGHTS = 64 << 20    # elements of [gate; up] up to which 512 rows are enough
+
+_cu_counts: dict = {}
+
+
+def _compute_units(device) -> int:
+    n = _cu_counts.get(device)
+    if n is None:
+        n = _cu_counts[device] = int(torch.cuda.get_device_properties(device).multi_processor_count)
+    return n
+
+
+def wide_swiglu_pays(M: int, two_i: int, K: int, ldx: int) -> bool:
+    """Is the gate/up product of M rows faster through the wide-tile kernel (with the gate in its
+    epilogue) than through the library and the gate kernel?"""
+    if M < WIDE_SWIGLU_MIN_ROWS and not (M >= WIDE_SWIGLU_MIN_ROWS // 2 and two_i * K <= WIDE_SWIGLU_SMALL_WEIGHTS):
+        return False
+    return _load("gemm_tile").cw_gemm_bf16_wide_tiles(2, M, two_i, K, ldx) >= WIDE_SWIGLU_MIN_TILES
 
 
 @contextlib.contextmanager
@@ -571,8 +612,11 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
         _check(_load("gemm").cw_gemm_bf16_skinny(2, _ptr(x), K, _ptr(gate_up_weight), _ptr(out), two_i // 2, M, two_i, K, _stream()),
                "gemm_bf16_skinny(swiglu)")
         return out
-    if HIP_PRODUCTS and x.dtype == torch.bfloat16 and K % 8 == 0 and x.is_contiguous():
-        return linear_tiled(x, gate_up_weight, swiglu=True)
+    if x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and K % 8 == 0 and x.is_contiguous():
+        if HIP_PRODUCTS:
+            return linear_tiled(x, gate_up_weight, swiglu=True)
+        if wide_swiglu_pays(M, two_i, K, K):
+            return linear_tiled(x, gate_up_weight, swiglu=True, wide=True)
     return silu_mul(linear(x, gate_up_weight), out)
 
 

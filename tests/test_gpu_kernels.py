@@ -491,6 +491,85 @@ def test_tiled_product(M, N, K):
     assert torch.equal(alone[0], ops.linear_tiled(x, w)[M - 1])
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 1000, 256), (777, 2 * 489, 320), (1000, 2 * 488, 448), (257, 200, 1024),
+                                   (2048, 2 * 1000, 1536), (513, 4000, 704)])
+def test_wide_tile_product(M, N, K):
+    """The product with 256 x 192 tiles, whose operands go from memory straight into LDS: plain
+    with a bias of either type, and gated; sizes that are no multiples of the tile, outputs whose
+    rows are no multiples of 16 bytes, rows of x with a stride, more tiles than one round of
+    workgroups and fewer; a row does not depend on the other rows of the batch."""
+    from clockwork_amd import ops
+
+    padded = torch.randn(M, K + 24, device=DEV).to(torch.bfloat16)
+    x = padded[:, :K]  # row stride K + 24
+    w = (torch.randn(N, K, device=DEV) / K ** 0.5).to(torch.bfloat16)
+    want = x.float() @ w.float().t()
+    got = ops.linear_tiled(x, w, wide=True)
+    torch.testing.assert_close(got.float(), want, rtol=1e-2, atol=1e-2)
+    for bias_dtype in (torch.bfloat16, torch.float32):
+        b = torch.randn(N, device=DEV).to(bias_dtype)
+        torch.testing.assert_close(ops.linear_tiled(x, w, b, wide=True).float(), want + b.float(), rtol=1e-2, atol=2e-2)
+    I = N // 2
+    gated = ops.linear_tiled(x, w, swiglu=True, wide=True)
+    assert tuple(gated.shape) == (M, I)
+    torch.testing.assert_close(gated.float(), torch.nn.functional.silu(want[:, :I]) * want[:, I:], rtol=2e-2, atol=2e-2)
+    alone = ops.linear_tiled(x[M - 1 :], w, wide=True)
+    assert torch.equal(alone[0], got[M - 1])
+    # the same bits as the kernel with the small tiles would not be promised; the same product is
+    torch.testing.assert_close(got.float(), ops.linear_tiled(x, w, wide=False).float(), rtol=1e-2, atol=1e-2)
+
+
+def test_wide_tile_product_finds_one_large_entry():
+    """A product is a sum over all of K and over the right rows: one large element of x and of W
+    shows in exactly one output, whatever stage, fragment and lane hold it."""
+    from clockwork_amd import ops
+
+    M, N, K = 520, 2 * 300, 1024
+    g = torch.Generator(device="cpu").manual_seed(3)
+    for _ in range(6):
+        m, n, k = (int(torch.randint(0, hi, (1,), generator=g)) for hi in (M, N, K))
+        x = torch.zeros(M, K, device=DEV, dtype=torch.bfloat16)
+        w = torch.zeros(N, K, device=DEV, dtype=torch.bfloat16)
+        x[m, k], w[n, k] = 3.0, 5.0
+        y = ops.linear_tiled(x, w, wide=True).float()
+        assert y[m, n].item() == 15.0 and torch.count_nonzero(y).item() == 1, (m, n, k)
+
+
+def test_wide_tile_product_refuses_what_it_does_not_take():
+    from clockwork_amd import ops
+    from clockwork_amd.ops import KernelError
+
+    x = torch.randn(300, 200, device=DEV).to(torch.bfloat16)   # K no multiple of 64
+    w = torch.randn(128, 200, device=DEV).to(torch.bfloat16)
+    with pytest.raises(KernelError):
+        ops.linear_tiled(x, w, wide=True)
+    assert not ops.wide_swiglu_pays(2048, 2 * 8960, 1500, 1500)
+    # the gate/up product of the 1.5B and 7B shapes: long portions take the kernel, short ones do not
+    assert ops.wide_swiglu_pays(2048, 2 * 8960, 1536, 1536) and ops.wide_swiglu_pays(512, 2 * 8960, 1536, 1536)
+    assert not ops.wide_swiglu_pays(256, 2 * 8960, 1536, 1536)
+    assert ops.wide_swiglu_pays(1024, 2 * 18944, 3584, 3584) and not ops.wide_swiglu_pays(512, 2 * 18944, 3584, 3584)
+
+
+def test_gate_up_of_a_long_portion_goes_through_the_wide_tile_kernel():
+    from clockwork_amd import ops
+
+    x = torch.randn(1024, 1536, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(2 * 8960, 1536, device=DEV) / 40).to(torch.bfloat16)
+    calls = []
+    real = ops.linear_tiled
+    ops.linear_tiled = lambda *a, **k: (calls.append(k), real(*a, **k))[1]
+    try:
+        got = ops.linear_swiglu(x, w)
+        few = ops.linear_swiglu(x[:100], w)
+    finally:
+        ops.linear_tiled = real
+    assert len(calls) == 1 and calls[0].get("wide") is True
+    y = x.float() @ w.float().t()
+    want = torch.nn.functional.silu(y[:, :8960]) * y[:, 8960:]
+    torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(few.float(), want[:100], rtol=2e-2, atol=2e-2)
+
+
 def test_hip_products_switch_routes_large_products_to_the_tiled_kernel():
     from clockwork_amd import ops
 
