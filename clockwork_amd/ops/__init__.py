@@ -491,7 +491,10 @@ WIDE_MIN_TILES = 64
 # Qwen2.5 layer shapes from 0.5B to 72B with 256 to 4096 rows: with 180 tiles or more (seven tenths
 # of the compute units busy in the last round) and 1024 rows or more it is 5 to 25 % faster; with
 # fewer rows the product is bound by reading W once, which the library does better for the large
-# shapes (and 512 rows win only for the small ones).
+# shapes (and 512 rows win only for the small ones). Against the library's TUNED choice it wins for
+# the 0.5B, 1.5B, 3B, 14B and 32B shapes (the 1.5B shape's whole prefill step: 8.9 -> 7.9 ms) and
+# loses 3 % of the step for the 7B and 72B shapes, so a start-up that tunes (``library_tuning``)
+# times both ways on the model's own weights and keeps the faster (``_swiglu_choices``).
 WIDE_SWIGLU_MIN_TILES = 180
 WIDE_SWIGLU_MIN_ROWS = 1024
 WIDE_SWIGLU_SMALL_WEIGHTS = 64 << 20    # elements of [gate; up] up to which 512 rows are enough
@@ -525,12 +528,40 @@ def library_tuning():
 
     if not os.environ.get("PYTORCH_TUNABLEOP_FILENAME"):
         tunable.set_filename(os.path.join(tempfile.gettempdir(), f"clockwork_amd_products_{os.getuid()}.csv"), True)
+    global _tuning
     tunable.enable(True)
     tunable.tuning_enable(True)
+    _tuning = True
     try:
         yield
     finally:
+        _tuning = False
         tunable.tuning_enable(False)
+
+
+_tuning = False
+# (rows of [gate; up], K) -> was the wide-tile kernel the faster way when both were timed?
+_swiglu_choices: dict = {}
+
+
+def _timed_us(fn, repeats: int = 5) -> float:
+    fn()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin.record()
+    for _ in range(repeats):
+        fn()
+    end.record()
+    end.synchronize()
+    return begin.elapsed_time(end) * 1e3 / repeats
+
+
+def _measure_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor, out: torch.Tensor) -> bool:
+    """Time the two ways of a long portion's gate/up product on these operands (the library has
+    just chosen its kernel for the shape): is this package's kernel at least as fast as the
+    library's product followed by the gate kernel?"""
+    library = _timed_us(lambda: silu_mul(linear(x, gate_up_weight), out))
+    own = _timed_us(lambda: linear_tiled(x, gate_up_weight, swiglu=True, wide=True))
+    return own <= library
 
 
 def qkv_rope_fused_supported(x: torch.Tensor, weight: torch.Tensor, rotary_dim: int, hd: int) -> bool:
@@ -616,7 +647,13 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
         if HIP_PRODUCTS:
             return linear_tiled(x, gate_up_weight, swiglu=True)
         if wide_swiglu_pays(M, two_i, K, K):
-            return linear_tiled(x, gate_up_weight, swiglu=True, wide=True)
+            # with enough rows the shape of the weights decides, and a start-up that tunes the
+            # library's products has measured it for this model's
+            measured = M >= WIDE_SWIGLU_MIN_ROWS
+            if measured and _tuning and (two_i, K) not in _swiglu_choices:
+                _swiglu_choices[(two_i, K)] = _measure_swiglu(x, gate_up_weight, out)
+            if not measured or _swiglu_choices.get((two_i, K), True):
+                return linear_tiled(x, gate_up_weight, swiglu=True, wide=True)
     return silu_mul(linear(x, gate_up_weight), out)
 
 

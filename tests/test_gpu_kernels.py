@@ -570,6 +570,42 @@ def test_gate_up_of_a_long_portion_goes_through_the_wide_tile_kernel():
     torch.testing.assert_close(few.float(), want[:100], rtol=2e-2, atol=2e-2)
 
 
+def test_a_tuning_start_up_measures_which_gate_up_product_is_faster():
+    """While the library tunes, the first long portion of a weight shape times both ways and the
+    choice is kept: later products of that shape follow it."""
+    from clockwork_amd import ops
+
+    x = torch.randn(1024, 1536, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(2 * 8960, 1536, device=DEV) / 40).to(torch.bfloat16)
+    key = (2 * 8960, 1536)
+    kept = ops._swiglu_choices.pop(key, None)
+    calls = []
+    real = ops.linear_tiled
+    ops.linear_tiled = lambda *a, **k: (calls.append(k), real(*a, **k))[1]
+    try:
+        ops._tuning = True   # what library_tuning() sets, without touching the library's own tuner
+        first = ops.linear_swiglu(x, w)
+        ops._tuning = False
+        assert key in ops._swiglu_choices
+        for choice in (False, True):
+            ops._swiglu_choices[key] = choice
+            calls.clear()
+            again = ops.linear_swiglu(x, w)
+            assert bool(calls) == choice
+            torch.testing.assert_close(again.float(), first.float(), rtol=2e-2, atol=2e-2)
+        # fewer rows than the measurement speaks for: the rule, not the choice
+        ops._swiglu_choices[key] = False
+        calls.clear()
+        ops.linear_swiglu(x[:512], w)
+        assert calls
+    finally:
+        ops._tuning = False
+        ops.linear_tiled = real
+        ops._swiglu_choices.pop(key, None)
+        if kept is not None:
+            ops._swiglu_choices[key] = kept
+
+
 def test_hip_products_switch_routes_large_products_to_the_tiled_kernel():
     from clockwork_amd import ops
 
