@@ -419,8 +419,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
             return out
     if HIP_PRODUCTS and K % 8 == 0 and x.is_contiguous():
         y = linear_tiled(x, weight, bias)
+    elif _wide_product_chosen(x, weight, bias):
+        y = linear_tiled(x, weight, bias, wide=True)
     else:
-        y = torch.mm(x, weight.t()) if bias is None else torch.addmm(bias, x, weight.t())
+        y = _library_product(x, weight, bias)
     if out_dtype == torch.float32:
         out = torch.empty((M, N), dtype=torch.float32, device=x.device)
         _check(_load("core").cw_bf16_to_f32(_ptr(y), _ptr(out), M * N, _stream()), "bf16_to_f32")
@@ -542,17 +544,54 @@ def library_tuning():
 _tuning = False
 # (rows of [gate; up], K) -> was the wide-tile kernel the faster way when both were timed?
 _swiglu_choices: dict = {}
+# (N, K, with bias) -> the same for a plain product; shapes that were never timed take the library
+_product_choices: dict = {}
+# a plain product is timed against the library's only with this many rows and tiles (half the
+# compute units busy): below that the library has always been the faster one
+WIDE_PRODUCT_MIN_ROWS = 1024
+WIDE_PRODUCT_MIN_TILES = 128
+
+
+def _library_product(x, weight, bias):
+    return torch.mm(x, weight.t()) if bias is None else torch.addmm(bias, x, weight.t())
+
+
+def _wide_product_chosen(x: torch.Tensor, weight: torch.Tensor, bias) -> bool:
+    """Does a plain product of many bfloat16 rows go through the wide-tile kernel? Only where a
+    tuning start-up has timed it against the library's tuned kernel on these very shapes and
+    found it faster (measured: the 7B shape's down product, 279 against 351 us)."""
+    M, K = x.shape
+    if M < WIDE_PRODUCT_MIN_ROWS or not _product_choices and not _tuning:
+        return False
+    key = (weight.shape[0], K, bias is not None)
+    choice = _product_choices.get(key)
+    if choice is None and _tuning and x.is_contiguous():
+        if _load("gemm_tile").cw_gemm_bf16_wide_tiles(0, M, key[0], K, K) >= WIDE_PRODUCT_MIN_TILES:
+            library = _timed_us(lambda: _library_product(x, weight, bias))
+            own = _timed_us(lambda: linear_tiled(x, weight, bias, wide=True))
+            choice = own <= library
+        else:
+            choice = False
+        _product_choices[key] = choice
+    return bool(choice) and x.is_contiguous()
 
 
 def _timed_us(fn, repeats: int = 5) -> float:
+    """The median time of ``fn`` with its operands out of the caches, as a layer finds its weights
+    in a model larger than the last-level cache: 512 MB are written between the runs. (Timed
+    back to back, a product whose weights fit that cache looks faster than it is in a step.)"""
     fn()
-    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    begin.record()
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
+    times = []
     for _ in range(repeats):
+        flush.zero_()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
         fn()
-    end.record()
-    end.synchronize()
-    return begin.elapsed_time(end) * 1e3 / repeats
+        end.record()
+        end.synchronize()
+        times.append(begin.elapsed_time(end) * 1e3)
+    return sorted(times)[len(times) // 2]
 
 
 def _measure_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor, out: torch.Tensor) -> bool:

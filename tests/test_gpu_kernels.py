@@ -606,6 +606,46 @@ def test_a_tuning_start_up_measures_which_gate_up_product_is_faster():
             ops._swiglu_choices[key] = kept
 
 
+def test_a_tuning_start_up_times_plain_products_too():
+    """A plain product of many rows is timed against the library's while the library tunes, if it
+    has tiles enough; the choice then holds for the shape, and untimed shapes take the library."""
+    from clockwork_amd import ops
+
+    x = torch.randn(2048, 1024, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(3584, 1024, device=DEV) / 32).to(torch.bfloat16)     # 8 x 19 tiles
+    small = (torch.randn(512, 1024, device=DEV) / 32).to(torch.bfloat16)  # 8 x 3 tiles
+    b = torch.randn(3584, device=DEV).to(torch.bfloat16)
+    kept = dict(ops._product_choices)
+    ops._product_choices.clear()
+    calls = []
+    real = ops.linear_tiled
+    ops.linear_tiled = lambda *a, **k: (calls.append(k), real(*a, **k))[1]
+    try:
+        want = ops.linear(x, w, b)
+        assert not calls and not ops._product_choices       # nothing is timed outside a tuning start-up
+        ops._tuning = True
+        ops.linear(x, w, b)
+        ops.linear(x, small)
+        ops._tuning = False
+        assert (3584, 1024, True) in ops._product_choices and ops._product_choices[(512, 1024, False)] is False
+        for choice in (True, False):
+            ops._product_choices[(3584, 1024, True)] = choice
+            calls.clear()
+            got = ops.linear(x, w, b)
+            assert bool(calls) == choice
+            torch.testing.assert_close(got.float(), want.float(), rtol=2e-2, atol=2e-2)
+        calls.clear()
+        ops._product_choices[(3584, 1024, True)] = True
+        ops.linear(x[:512], w, b)          # too few rows for the measurement to speak for
+        ops.linear(x, w)                   # another shape (no bias): never timed
+        assert not calls
+    finally:
+        ops._tuning = False
+        ops.linear_tiled = real
+        ops._product_choices.clear()
+        ops._product_choices.update(kept)
+
+
 def test_hip_products_switch_routes_large_products_to_the_tiled_kernel():
     from clockwork_amd import ops
 
