@@ -368,6 +368,51 @@ def test_the_whole_benchmark_model(benchmark_model, mode, dtype):
         assert all(g < 1e-1 * scale for g in gaps) and len(gaps) < 30
 
 
+def test_a_long_portion_takes_the_wide_tile_product(tmp_path):
+    """A prompt of 1,300 tokens through a layer with the benchmark model's widths, bfloat16: run
+    whole, its gate/up product goes through the package's own wide-tile kernel (1,300 rows: 6 row
+    tiles, the last one a third full); run in portions of 300 through the library and the gate
+    kernel; a second prompt rides beside the long one's last portion. Both against the plain
+    implementation, and the two ways against each other."""
+    from clockwork_amd import ops
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests.configs import LAYER_1P5B
+
+    config = dict(LAYER_1P5B, vocab_size=1203, tie_word_embeddings=False)
+    model_dir = write_random_model(tmp_path / "model", config, 5)
+    gen = torch.Generator().manual_seed(17)
+    long = torch.randint(0, 1203, (1300,), generator=gen).tolist()
+    short = torch.randint(0, 1203, (1100,), generator=gen).tolist()
+    plain = PlainQwen2(model_dir)
+    want = {"long": plain.logits(long), "short": plain.logits(short)}
+    want["other"] = want["long"][:200]   # the long prompt's first 200 tokens as a request of their own
+    wanted = [0, 1, 255, 256, 257, 700, 1023, 1024, 1279, 1280, 1298, 1299]
+    calls = []
+    real = ops.linear_tiled
+    ops.linear_tiled = lambda *a, **k: (calls.append((a[0].shape[0], k.get("wide"))), real(*a, **k))[1]
+    try:
+        runner = replay.make_runner(model_dir, "bfloat16", 16, 170, max_model_len=2048)
+        whole = replay.run_trace(runner, [
+            {"entries": [{"id": "long", "tokens": long, "want": wanted}], "end": ["long"]},
+            # 1,100 + 200 rows in one step: two requests share the product's row tiles
+            {"entries": [{"id": "short", "tokens": short, "want": [w for w in wanted if w < 1100]},
+                         {"id": "other", "tokens": long[:200], "want": [0, 199]}], "end": ["short", "other"]},
+        ])
+        assert calls == [(1300, True), (1300, True)]
+        calls.clear()
+        steps = [{"entries": [{"id": "long", "tokens": long[at : at + 300], "want": [w - at for w in wanted if at <= w < at + 300]}],
+                  "end": []} for at in range(0, 1300, 300)]
+        steps[-1]["end"] = ["long"]
+        cut = replay.run_trace(runner, steps)
+        assert not calls
+    finally:
+        ops.linear_tiled = real
+    assert len(whole) == len(wanted) + sum(w < 1100 for w in wanted) + 2 and len(cut) == len(wanted)
+    replay.compare_to_scale(whole, want)
+    replay.compare_to_scale(cut, want)
+    replay.compare_to_scale(cut, {"long": {p: whole[("long", p)] for p in wanted}})
+
+
 @pytest.mark.parametrize("which", ["LAYER_7B", "LAYER_32B"])
 def test_layers_of_the_larger_models(tmp_path, which):
     """One layer of the 7B and of the 32B shape, bfloat16: a prompt in two portions, then tokens
