@@ -408,6 +408,18 @@ def test_a_long_portion_takes_the_wide_tile_product(tmp_path):
     finally:
         ops.linear_tiled = real
     assert len(whole) == len(wanted) + sum(w < 1100 for w in wanted) + 2 and len(cut) == len(wanted)
+    # 450 tokens as a step of their own replay the graph for 512 rows, which holds the wide-tile
+    # kernel: the first run is eager, the second is captured, the third replays
+    for turn in range(3):
+        calls.clear()
+        ops.linear_tiled = lambda *a, **k: (calls.append((a[0].shape[0], k.get("wide"))), real(*a, **k))[1]
+        try:
+            again = replay.run_trace(runner, [{"entries": [{"id": "g", "tokens": long[:450], "want": [449]}], "end": ["g"]}])
+        finally:
+            ops.linear_tiled = real
+        # eager with its own 450 rows (the library's product), captured with 512, then replayed
+        assert (set(calls) == {(512, True)}) if turn == 1 else not calls, (turn, calls)
+        replay.compare_to_scale(again, {"g": want["long"]})
     replay.compare_to_scale(whole, want)
     replay.compare_to_scale(cut, want)
     replay.compare_to_scale(cut, {"long": {p: whole[("long", p)] for p in wanted}})
