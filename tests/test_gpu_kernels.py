@@ -178,7 +178,8 @@ def test_rmsnorm_zero_row_and_scale_invariance():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nh,nkv,hd,rotary,theta", [(4, 2, 16, 16, 1e4), (6, 1, 32, 32, 1e6), (3, 3, 48, 48, 5e4), (5, 1, 64, 32, 1e4)])
+@pytest.mark.parametrize("nh,nkv,hd,rotary,theta", [(4, 2, 16, 16, 1e4), (6, 1, 32, 32, 1e6), (3, 3, 48, 48, 5e4), (5, 1, 64, 32, 1e4),
+                                                    (12, 2, 128, 128, 1e6)])
 def test_rope_kv_write(dtype, nh, nkv, hd, rotary, theta):
     from clockwork_amd import ops
 
@@ -215,6 +216,38 @@ def test_rope_kv_write(dtype, nh, nkv, hd, rotary, theta):
     for s in range(rows):
         if s not in written:
             assert torch.all(kc[s] == 100.0) and torch.all(vc[s] == 100.0)
+
+
+@pytest.mark.parametrize("bias_dtype", [None, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("nh,nkv,hd", [(12, 2, 128), (5, 1, 48), (2, 2, 256)])
+def test_rope_kv_write_in_16_byte_pieces_equals_the_kernel_for_any_row(nh, nkv, hd, bias_dtype):
+    """bfloat16 rows whose heads are rotated whole go through a kernel that moves 16 bytes at a
+    time; rows that do not lie on a 16-byte boundary go through the one that moves single
+    elements. The same rows through both: the same bits, in q and in the cache."""
+    from clockwork_amd import ops
+
+    T, rows = 37, 64
+    width = (nh + 2 * nkv) * hd
+    gen = torch.Generator(device="cpu").manual_seed(nh * hd)
+    values = torch.randn(T, width, generator=gen).to(torch.bfloat16)
+    bias = None if bias_dtype is None else (0.5 * torch.randn(width, generator=gen)).to(bias_dtype).to(DEV)
+    positions = torch.randint(0, 30000, (T,), generator=gen).to(torch.int32).to(DEV)
+    slots = torch.randperm(rows, generator=gen)[:T].to(torch.int32)
+    slots[5] = -1
+    slots = slots.to(DEV)
+    inv_freq = plain.inv_frequencies(hd, 1e6).to(DEV)
+    results = []
+    for shift in (0, 4):   # 4 elements: 8 bytes off the boundary
+        store = torch.zeros(T * width + 8, dtype=torch.bfloat16, device=DEV)
+        work = store[shift : shift + T * width].view(T, width)
+        work.copy_(values)
+        assert (work.data_ptr() % 16 == 0) == (shift == 0)
+        kc = torch.full((rows, nkv, hd), 100.0, device=DEV, dtype=torch.bfloat16)
+        vc = torch.full((rows, nkv, hd), 100.0, device=DEV, dtype=torch.bfloat16)
+        ops.rope_kv_write(work, bias, positions, slots, inv_freq, hd, nh, nkv, hd, kc, vc)
+        results.append((work[:, : nh * hd].clone(), kc, vc))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
