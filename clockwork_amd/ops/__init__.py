@@ -598,7 +598,7 @@ def _measure_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor, out: torch.Te
     """Time the two ways of a long portion's gate/up product on these operands (the library has
     just chosen its kernel for the shape): is this package's kernel at least as fast as the
     library's product followed by the gate kernel?"""
-    library = _timed_us(lambda: silu_mul(linear(x, gate_up_weight), out))
+    library = _timed_us(lambda: silu_mul(_library_product(x, gate_up_weight, None), out))
     own = _timed_us(lambda: linear_tiled(x, gate_up_weight, swiglu=True, wide=True))
     return own <= library
 
