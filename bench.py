@@ -63,18 +63,11 @@ def context_of(args) -> int:
 def build_runner(args, prefix_cache: bool = False, max_batch: int = 0):
     from clockwork_amd.config.engine import EngineConfig
     from clockwork_amd.engine.model_runner import GRAPH_BATCH_SIZES, ModelRunner
-    from clockwork_amd.parts.model import model_param_specs
-    from clockwork_amd.registry import resolve_architecture
-    from clockwork_amd.weights.random_init import RandomSource
 
     config = dict(SHAPES[args.shape][1])
     if args.layers is not None:
         config["num_hidden_layers"] = args.layers
     args.layers = config["num_hidden_layers"]
-    arch = resolve_architecture(config)
-    mcfg = arch.parse_config(config)
-    spec = arch.build_spec(mcfg)
-    source = RandomSource(arch.weight_plan(mcfg, spec), model_param_specs(spec), seed=2, device="cuda")
     # the cache holds the largest batch the run decodes: 64 for the recorded points
     max_batch = max(args.batch, 1 if getattr(args, "no_points", False) else 64, max_batch)
     context = context_of(args)
@@ -82,8 +75,10 @@ def build_runner(args, prefix_cache: bool = False, max_batch: int = 0):
         f"random:{SHAPES[args.shape][0].lower()}", dtype=args.dtype, max_model_len=context, block_size=BLOCK,
         num_blocks=max_batch * context // BLOCK, enable_prefix_cache=prefix_cache, watermark=0.0,
         max_num_seqs=max_batch, max_num_batched_tokens=max(PROMPT_LEN, max_batch),
+        # the engine's random-weights mode: every tensor drawn from the seed by the GPU's generator
+        weights="random_device", weight_seed=2,
     )
-    runner = ModelRunner(cfg, weight_source=source, config_dict=config)
+    runner = ModelRunner(cfg, config_dict=config)
     if not args.no_tune:
         # the engine's start-up option ``tune_products``: the library's fastest kernel per product shape
         runner.tune_products([PROMPT_LEN, *GRAPH_BATCH_SIZES])

@@ -27,7 +27,7 @@ from typing import Optional, Sequence
 import numpy as np
 
 from clockwork_amd.cache.allocator import OutOfPages, PagePool
-from clockwork_amd.config.spec import KVPagesSpec, ModelSpec, StateSpec
+from clockwork_amd.config.spec import KVPagesSpec, ModelSpec, PagedRowsSpec, StateSpec
 
 NO_PAGE = -1
 
@@ -37,12 +37,13 @@ class GroupLayout:
     """One layer group: which run entries it serves and what one of them stores."""
 
     index: int
-    need: object            # KVPagesSpec or StateSpec
+    need: object            # KVPagesSpec / PagedRowsSpec (pages) or StateSpec (a slot)
     entries: tuple[int, ...]  # indices into ModelSpec.run that own a cache in this group
 
     @property
     def is_kv(self) -> bool:
-        return isinstance(self.need, KVPagesSpec)
+        """Does the group keep rows per token in pages (keys and values, or planes of a mixer's own)?"""
+        return isinstance(self.need, (KVPagesSpec, PagedRowsSpec))
 
     @property
     def window(self) -> Optional[int]:
@@ -59,8 +60,8 @@ def plan_groups(needs: Sequence[Optional[object]]) -> list[GroupLayout]:
     for i, need in enumerate(needs):
         if need is None:
             continue
-        if not isinstance(need, (KVPagesSpec, StateSpec)):
-            raise TypeError(f"run entry {i}: a cache need must be KVPagesSpec or StateSpec, got {need!r}")
+        if not isinstance(need, (KVPagesSpec, PagedRowsSpec, StateSpec)):
+            raise TypeError(f"run entry {i}: a cache need must be KVPagesSpec, PagedRowsSpec or StateSpec, got {need!r}")
         key = need.group_key()
         if key not in members:
             order.append(key)

@@ -8,6 +8,8 @@ starting a server it generates for the prompts given and prints one JSON line pe
     python -m clockwork_amd.cli --config engine.yaml --set dtype=bfloat16 \
         --prompt-ids 5,17,3 --prompt-ids 9,9,9 --max-tokens 16 --temperature 0.8 --seed 1
 
+    python -m clockwork_amd.cli --model config.json --random-weights 2 --prompt-ids 5,17,3 --max-tokens 8
+
     python -m clockwork_amd.cli make-random --config-json config.json --seed 0 --out DIR
 """
 
@@ -21,11 +23,15 @@ from clockwork_amd.config.engine import EngineConfig
 from clockwork_amd.engine.sequence import SamplingParams
 
 
-def _generate(argv) -> int:
+def parse_generate(argv):
+    """(arguments, engine configuration, prompts) of a generation command line; touches no GPU."""
     p = argparse.ArgumentParser(prog="clockwork-generate", description=__doc__,
                                 formatter_class=argparse.RawDescriptionHelpFormatter)
     p.add_argument("--config", help="engine YAML (sections model / cache / scheduler)")
     p.add_argument("--model", help="model folder; stands in for --config with defaults")
+    p.add_argument("--random-weights", type=int, default=None, metavar="SEED",
+                   help="serve random weights drawn from SEED instead of a checkpoint (the values that "
+                        "make-random writes); --model may then name a bare config.json")
     p.add_argument("--set", dest="overrides", action="append", default=[], metavar="KEY=VALUE",
                    help="override any model, cache or scheduler field, e.g. --set num_blocks=1024")
     p.add_argument("--prompt-ids", action="append", default=[], metavar="I,J,K", help="a prompt as token ids")
@@ -46,6 +52,9 @@ def _generate(argv) -> int:
         p.error("give exactly one of --config and --model")
     cfg = EngineConfig.from_yaml(args.config) if args.config else EngineConfig.defaults(args.model)
     try:
+        if args.random_weights is not None:
+            cfg.set("weights", "random")
+            cfg.set("weight_seed", args.random_weights)
         cfg.apply_overrides(args.overrides)
     except ValueError as e:
         raise SystemExit(str(e))
@@ -57,7 +66,11 @@ def _generate(argv) -> int:
     prompts += args.prompt
     if not prompts:
         p.error("no prompts: use --prompt-ids, --prompt-file or --prompt")
+    return args, cfg, prompts
 
+
+def _generate(argv) -> int:
+    args, cfg, prompts = parse_generate(argv)
     tokenizer = None
     if args.tokenizer:
         from transformers import AutoTokenizer  # tokenizer files only; no model code is involved

@@ -13,6 +13,9 @@ from pathlib import Path
 import yaml
 
 
+WEIGHT_MODES = ("checkpoint", "random", "random_device")
+
+
 @dataclass
 class ModelConfig:
     """Which model folder to serve and how (clockwork/config.py:17-31)."""
@@ -27,8 +30,18 @@ class ModelConfig:
     # portion and of the wide decode batches and keep the fastest (bfloat16 only)
     tune_products: bool = False
     # run the large bfloat16 products on this package's own tiled kernel instead of the matrix
-    # library (slower; for runs that must not depend on the library). Process-wide.
+    # library (slower; for runs that must not depend on the library)
     hip_products: bool = False
+    # where the weights come from: "checkpoint" (the safetensors files of the folder ``model``),
+    # "random" (drawn from ``weight_seed`` on the host, the very values that ``make-random`` writes
+    # into a folder; ``model`` may then name a bare config.json) or "random_device" (drawn by the
+    # GPU's generator: other values, made in seconds for the largest shapes)
+    weights: str = "checkpoint"
+    weight_seed: int = 0
+
+    def __post_init__(self):
+        if self.weights not in WEIGHT_MODES:
+            raise ValueError(f"weights {self.weights!r}: expected one of {WEIGHT_MODES}")
 
     def torch_dtype(self):
         """The torch dtype of ``dtype``; the reference's float16 is named so that a user of it
@@ -121,7 +134,15 @@ class EngineConfig:
         hits = 0
         for section in self.sections().values():
             if any(f.name == key for f in fields(section)):
+                previous = getattr(section, key)
                 setattr(section, key, value)
+                check = getattr(section, "__post_init__", None)
+                if check is not None:
+                    try:
+                        check()
+                    except ValueError:
+                        setattr(section, key, previous)
+                        raise
                 hits += 1
         if hits == 0:
             raise ValueError(f"unknown config override {key!r}")

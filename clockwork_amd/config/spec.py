@@ -49,20 +49,59 @@ class KVPagesSpec:
     def group_key(self) -> tuple:
         return ("kv", self.num_kv_heads, self.head_dim, self.window)
 
+    @property
+    def planes(self) -> tuple:
+        """What a page holds per token, as (name, row shape) pairs: a key row and a value row."""
+        row = (self.num_kv_heads, self.head_dim)
+        return (("k", row), ("v", row))
+
+
+@dataclass(frozen=True)
+class PagedRowsSpec:
+    """A mixer that keeps rows of its own making for earlier tokens in pages: ``planes`` names
+    each kind of row and gives its shape, e.g. ``(("latent", (24,)),)`` for one 24-wide vector a
+    token and no values, or keys and values of different widths. Pages, block tables, windows
+    and sharing work as for :class:`KVPagesSpec` (which is the case of two equal planes named
+    ``k`` and ``v``); the mixer finds its planes in ``EntryCache.planes`` by name, each a flat
+    [num_blocks * block_size, *row shape] view, and addresses them through the step's block
+    tables and slots of its group.
+    """
+
+    planes: tuple
+    window: Optional[int] = None
+
+    def __post_init__(self):
+        names = [name for name, _ in self.planes]
+        if not self.planes or len(set(names)) != len(names):
+            raise ValueError(f"a paged cache needs planes with names of their own, got {self.planes!r}")
+        for name, shape in self.planes:
+            if not shape or any(int(d) < 1 for d in shape):
+                raise ValueError(f"plane {name!r} has no valid row shape: {shape!r}")
+
+    def group_key(self) -> tuple:
+        return ("rows", tuple((name, tuple(shape)) for name, shape in self.planes), self.window)
+
 
 @dataclass(frozen=True)
 class StateSpec:
     """A mixer that keeps a fixed-size state per request (a recurrence, a convolution tail).
 
-    One slot of ``shape``/``dtype`` per live request and per run entry; zeroed
-    when a request's first token arrives.
+    One slot of ``shape``/``dtype`` per live request and per run entry; when a request's first
+    token arrives its slot is set to the fresh state: ``init`` says which, ``("zeros",)`` or
+    ``("fill", value)`` (a part with another beginning, learned say, writes it into the pool's
+    template row at ``bind`` time: ``CachePools.set_fresh_state``).
     """
 
     shape: tuple[int, ...]
     dtype: str = "float32"
+    init: tuple = ("zeros",)
+
+    def __post_init__(self):
+        if self.init[0] not in ("zeros", "fill") or (self.init[0] == "fill" and len(self.init) != 2):
+            raise ValueError(f"a fresh state is ('zeros',) or ('fill', value), got {self.init!r}")
 
     def group_key(self) -> tuple:
-        return ("state", self.shape, self.dtype)
+        return ("state", self.shape, self.dtype, self.init)
 
 
 @dataclass(frozen=True)
@@ -148,12 +187,17 @@ class ModelSpec:
 class WeightTarget:
     """How one parameter of the model is filled from checkpoint tensors.
 
-    ``sources`` are tensor names in the checkpoint with their expected shapes;
-    several sources are concatenated along dim 0 (fused projections).
-    ``optional`` sources may be absent (a tied output head).
+    ``sources`` are tensor names in the checkpoint with their expected shapes (as the file holds
+    them); several sources are concatenated along dim 0 (fused projections).
+    ``optional`` sources may be absent (a tied output head). ``transform`` reshapes every source
+    after it is read and before it is put in its place: one step or a tuple of steps, each a tuple
+    of a name from ``clockwork_amd.weights.transforms`` and its arguments, e.g. ``("transpose",)``
+    for a matrix the checkpoint stores the other way round, ``("split_rows", 1, 3)`` for the second
+    third of a tensor that holds three projections, or both in a row.
     """
 
     param: str
     sources: tuple[str, ...]
     source_shapes: tuple[tuple[int, ...], ...]
     optional: bool = False
+    transform: Optional[tuple] = None

@@ -84,18 +84,18 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_bf16_kernel(TileArgs a) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int64_t m = min((int64_t)tm * GT_BM + row0 + 32 * i, (int64_t)M - 1);  // a row past the end repeats the last one
-    xp[i] = a.X + m * a.ldx + chunk * 8;
+    xp[i] = a.X + m * a.ldx;
     bool ok;
     int64_t n = gt_w_row<MODE>(tn, row0 + 32 * i, N, &ok);
     if (!ok) n = 0;  // never stored
-    wp[i] = a.W + n * K + chunk * 8;
+    wp[i] = a.W + n * K;
   }
   u32x4_t gx[4], gw[4];
   const int k_tiles = (K + GT_BK - 1) / GT_BK;
   auto fetch = [&](int kt) __attribute__((always_inline)) {
     const int k = kt * GT_BK + chunk * 8;
     const bool ok = k + 8 <= K;        // K is a multiple of 8: a chunk is inside or outside
-    const int at = ok ? kt * GT_BK : 0;
+    const int at = ok ? k : 0;         // a chunk outside reads the row's first one (inside the tensor) and is zeroed
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       gx[i] = *reinterpret_cast<const u32x4_t*>(xp[i] + at);
@@ -433,6 +433,10 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
     if (set == 0) {
       if (with_fetch) W_WAIT_LOADS(8);  // all but the 8 loads just issued: stages t + 2 and t + 3 are in
       else W_WAIT_LOADS(0);
+    } else {
+      // the next iteration asks for stage t + 6, which lands in the slot of stage t + 1: this wave's
+      // fragment reads of that stage (issued above) have to be back before any wave may do so
+      __builtin_amdgcn_s_waitcnt(0xC07F);
     }
     // every wave's loads of stage t + 2 are in LDS, and every wave has read stage t + 1
     W_BARRIER();

@@ -79,6 +79,7 @@ class StepContext:
         self.plans: dict = {}     # what parts have planned for this step, under keys of their own
         self._pinned: list = []   # host buffers of the plans' uploads, alive as long as the step
         self.num_compute_units = 256
+        self.products = None      # the engine's ops.ProductPolicy (None: the defaults)
 
     def upload(self, arrays) -> list:
         """int32 arrays to the device in one copy; returns a device view of each. For a part
@@ -265,8 +266,8 @@ class StaticDecodeBatch:
                     table[r, have:] = -1
                 elif state_r[1] < have:
                     table[r, state_r[1] : have] = row[state_r[1] :]
-                if g == len(manager.kv_groups) - 1:
-                    state_r[0], state_r[1] = epoch, have
+                if g == 0:
+                    state_r[0], state_r[1] = epoch, have  # what group 0's row holds now: only it is written in pieces
                 page = row[e.start // bs]
                 if page < 0:
                     raise ValueError(f"request {e.seq_id}: position {e.start} lies in a page that was given back")
@@ -274,7 +275,7 @@ class StaticDecodeBatch:
             for r in range(n, size):
                 if rows[r][0] is not None or g > 0:
                     table[r, :] = -1
-                    if g == len(manager.kv_groups) - 1:
+                    if g == 0:
                         rows[r][0], rows[r][1] = None, 0
         self.ctx.seq_ids = [e.seq_id for e in entries] + [""] * (size - n)
         if upload:

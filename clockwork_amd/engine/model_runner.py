@@ -31,6 +31,7 @@ from clockwork_amd.engine.batch import (
 from clockwork_amd.parts.model import DecoderModel
 from clockwork_amd.registry import resolve_architecture
 from clockwork_amd.weights.loader import load_parameters, read_config_json
+from clockwork_amd.weights.random_init import RandomSource
 
 
 # padded batch sizes a decode graph is captured for, and the step in which the planned context grows
@@ -80,7 +81,9 @@ class ModelRunner:
             raise ValueError(f"device {cfg.model.device!r}: this engine runs on the GPU only")
         self.device = require_gpu()
         self.dtype = cfg.model.torch_dtype()
-        ops.use_hip_products(cfg.model.hip_products)  # process-wide: the runner made last decides
+        # how this engine runs its large bfloat16 products (its own: another engine in the process
+        # has another); the parts find it in every step's context
+        self.products = ops.ProductPolicy(hip_products=cfg.model.hip_products)
         self.config_dict = config_dict if config_dict is not None else read_config_json(cfg.model.model)
         self.arch = resolve_architecture(self.config_dict)
         self.model_config = self.arch.parse_config(self.config_dict)
@@ -88,6 +91,11 @@ class ModelRunner:
         self.model = DecoderModel(self.spec)
         ops.preload(self.model.kernel_libraries(), tiled_products=cfg.model.hip_products or self.dtype == torch.bfloat16)
         plan = self.arch.weight_plan(self.model_config, self.spec)
+        if weight_source is None and cfg.model.weights != "checkpoint":
+            # a model without a checkpoint (clockwork/engine/loader.py:82-103 builds its tiny
+            # models from a seed): the tensors a checkpoint would hold, drawn from the seed
+            drawn_on = self.device if cfg.model.weights == "random_device" else "cpu"
+            weight_source = RandomSource(plan, self.model.param_specs(), cfg.model.weight_seed, device=drawn_on)
         params = load_parameters(
             cfg.model.model, plan, self.model.param_specs(), self.dtype, self.device, source=weight_source
         )
@@ -187,7 +195,7 @@ class ModelRunner:
                 continue
             self.reserve(seq_id, 0, n, total_len=n)
             try:
-                with ops.library_tuning():
+                with ops.library_tuning(self.products):
                     self.step([StepEntry(seq_id, 0, [0] * n, [n - 1])])
                 torch.cuda.synchronize()
                 done.append(n)
@@ -424,6 +432,7 @@ class ModelRunner:
         """The model's step on a laid-out batch: requests that begin in it start from an empty
         fixed-size state (cleared on the device, by the step's own first positions, so that a
         captured step does it too), then the parts run."""
+        ctx.products = self.products
         if self.pools.state:
             self.pools.zero_fresh_state(ctx.state_slots, ctx.starts, ctx.num_requests)
         return self.model.forward(ctx, self.caches)

@@ -1,6 +1,6 @@
 """Trace replay: feed given token ids through the model step by step and write logits.
 
-    trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+    trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--page TOKENS]
 
 Reads one JSON object a line from standard input,
 ``{"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}``,
@@ -83,6 +83,19 @@ class TraceReplayer:
         return entries, logits
 
 
+def replay_config(model: str, dtype: str, max_tokens: int, page: int = PAGE):
+    """The engine configuration of a replay: a pool of just the pages that ``max_tokens`` tokens
+    need (each live request's count rounded up to pages), so that pages are used again; one
+    request may hold them all; nothing is kept for later requests."""
+    from clockwork_amd.config.engine import EngineConfig
+
+    pages = max(1, -(-max_tokens // page))
+    return EngineConfig.defaults(
+        model, dtype=dtype, block_size=page, num_blocks=pages, max_model_len=page * pages,
+        enable_prefix_cache=False, watermark=0.0,
+    )
+
+
 def main(argv: Optional[list] = None) -> int:
     parser = argparse.ArgumentParser(prog="trace_run", description=__doc__,
                                      formatter_class=argparse.RawDescriptionHelpFormatter)
@@ -91,24 +104,17 @@ def main(argv: Optional[list] = None) -> int:
     parser.add_argument("--out", required=True, help="folder the logits files go to")
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at a time (each rounded up to 64)")
+    parser.add_argument("--page", type=int, default=PAGE, metavar="TOKENS",
+                        help=f"tokens a page of the cache holds (default {PAGE})")
     args = parser.parse_args(argv)
+    if args.page < 1:
+        parser.error("--page must be at least 1")
 
-    from clockwork_amd.config.engine import EngineConfig
     from clockwork_amd.engine.model_runner import ModelRunner
 
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
-    cfg = EngineConfig.defaults(
-        args.model,
-        dtype=args.dtype,
-        block_size=PAGE,
-        num_blocks=max(1, -(-args.max_tokens // PAGE)),
-        # one request may hold every token of the pool
-        max_model_len=max(PAGE, PAGE * -(-args.max_tokens // PAGE)),
-        enable_prefix_cache=False,
-        watermark=0.0,
-    )
-    replayer = TraceReplayer(ModelRunner(cfg))
+    replayer = TraceReplayer(ModelRunner(replay_config(args.model, args.dtype, args.max_tokens, args.page)))
     for line in sys.stdin:
         line = line.strip()
         if not line:

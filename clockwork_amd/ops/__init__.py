@@ -375,12 +375,15 @@ def zero_state_rows(pool: torch.Tensor, slots: torch.Tensor, starts: torch.Tenso
                                             _ptr(starts), int(n), _stream()), "zero_state_rows")
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, partial_ok: bool = False):
+def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, partial_ok: bool = False,
+           policy: "ProductPolicy | None" = None):
     """y = x @ weight.T (+ bias). float32: the true-float32 HIP product. bfloat16: few rows go
     through the weight-streaming kernel, many through the library product (as the reference's
-    engine uses one); float32 accumulation either way. With ``partial_ok`` the result may come
-    back as :class:`PartialSums` (a narrow output with a long K, few rows): only for a result
-    that goes straight into ``add_rmsnorm``."""
+    engine uses one) or, where ``policy`` (the calling engine's :class:`ProductPolicy`) says so,
+    through this package's tiled kernels; float32 accumulation either way. With ``partial_ok``
+    the result may come back as :class:`PartialSums` (a narrow output with a long K, few rows):
+    only for a result that goes straight into ``add_rmsnorm``."""
+    policy = policy if policy is not None else DEFAULT_POLICY
     _gpu(x, weight, bias)
     M, K = x.shape
     N = weight.shape[0]
@@ -417,9 +420,9 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
             _check(lib.cw_gemm_bf16_skinny(1 if want_f32 else 0, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, _stream()),
                    "gemm_bf16_skinny")
             return out
-    if HIP_PRODUCTS and K % 8 == 0 and x.is_contiguous():
+    if policy.hip_products and K % 8 == 0 and x.is_contiguous():
         y = linear_tiled(x, weight, bias)
-    elif _wide_product_chosen(x, weight, bias):
+    elif _wide_product_chosen(x, weight, bias, policy):
         y = linear_tiled(x, weight, bias, wide=True)
     else:
         y = _library_product(x, weight, bias)
@@ -430,15 +433,29 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
     return y
 
 
-# True: products of many bfloat16 rows go through this package's own LDS-tiled kernel instead of
-# the library (about half as fast on an MI355X; for a run that must not depend on the library).
-# Set through ``use_hip_products`` / the model section's ``hip_products``.
-HIP_PRODUCTS = False
+class ProductPolicy:
+    """How one engine runs its products of many bfloat16 rows. Every runner has one of its own and
+    hands it to the parts through the step context, so two engines in a process (other options,
+    other weights) never see each other's choices.
+
+    ``hip_products``: such products go through this package's own LDS-tiled kernels instead of the
+    library (about half as fast on an MI355X; for a run that must not depend on the library).
+    ``swiglu_choices`` / ``product_choices``: for a weight shape that a tuning start-up has timed
+    both ways, whether the wide-tile kernel was the faster one ((rows of [gate; up], K) and
+    (N, K, with bias)); shapes never timed follow the fixed rules. ``tuning``: such a start-up is
+    under way (``library_tuning``)."""
+
+    __slots__ = ("hip_products", "swiglu_choices", "product_choices", "tuning")
+
+    def __init__(self, hip_products: bool = False) -> None:
+        self.hip_products = bool(hip_products)
+        self.swiglu_choices: dict = {}
+        self.product_choices: dict = {}
+        self.tuning = False
 
 
-def use_hip_products(on: bool) -> None:
-    global HIP_PRODUCTS
-    HIP_PRODUCTS = bool(on)
+# what a call without an engine behind it runs by: the library for large products, nothing timed
+DEFAULT_POLICY = ProductPolicy()
 
 
 # up to this many rows every product goes through the weight-streaming kernels
@@ -496,7 +513,7 @@ WIDE_MIN_TILES = 64
 # shapes (and 512 rows win only for the small ones). Against the library's TUNED choice it wins for
 # the 0.5B, 1.5B, 3B, 14B and 32B shapes (the 1.5B shape's whole prefill step: 8.9 -> 7.9 ms) and
 # loses 3 % of the step for the 7B and 72B shapes, so a start-up that tunes (``library_tuning``)
-# times both ways on the model's own weights and keeps the faster (``_swiglu_choices``).
+# times both ways on the model's own weights and keeps the faster (``ProductPolicy.swiglu_choices``).
 WIDE_SWIGLU_MIN_TILES = 180
 WIDE_SWIGLU_MIN_ROWS = 1024
 WIDE_SWIGLU_SMALL_WEIGHTS = 64 << 20    # elements of [gate; up] up to which 512 rows are enough
@@ -520,32 +537,28 @@ def wide_swiglu_pays(M: int, two_i: int, K: int, ldx: int) -> bool:
 
 
 @contextlib.contextmanager
-def library_tuning():
+def library_tuning(policy: "ProductPolicy | None" = None):
     """While active, a library product of a shape not seen before is timed over the library's
     candidate kernels and the fastest is remembered; afterwards the remembered choices stay in
-    use and unseen shapes take the library's own default again. The choices are kept in a file
-    in the temporary folder (or where PYTORCH_TUNABLEOP_FILENAME points), which later processes
-    of the same user read. Not to be left active during HIP-graph capture."""
+    use and unseen shapes take the library's own default again. The library keeps its choices in a
+    file in the temporary folder (or where PYTORCH_TUNABLEOP_FILENAME points), which later
+    processes of the same user read. ``policy``: the engine whose own kernels are timed against the
+    library's meanwhile. Not to be left active during HIP-graph capture."""
     import torch.cuda.tunable as tunable
 
+    policy = policy if policy is not None else DEFAULT_POLICY
     if not os.environ.get("PYTORCH_TUNABLEOP_FILENAME"):
         tunable.set_filename(os.path.join(tempfile.gettempdir(), f"clockwork_amd_products_{os.getuid()}.csv"), True)
-    global _tuning
     tunable.enable(True)
     tunable.tuning_enable(True)
-    _tuning = True
+    policy.tuning = True
     try:
         yield
     finally:
-        _tuning = False
+        policy.tuning = False
         tunable.tuning_enable(False)
 
 
-_tuning = False
-# (rows of [gate; up], K) -> was the wide-tile kernel the faster way when both were timed?
-_swiglu_choices: dict = {}
-# (N, K, with bias) -> the same for a plain product; shapes that were never timed take the library
-_product_choices: dict = {}
 # a plain product is timed against the library's only with this many rows and tiles (half the
 # compute units busy): below that the library has always been the faster one
 WIDE_PRODUCT_MIN_ROWS = 1024
@@ -556,23 +569,23 @@ def _library_product(x, weight, bias):
     return torch.mm(x, weight.t()) if bias is None else torch.addmm(bias, x, weight.t())
 
 
-def _wide_product_chosen(x: torch.Tensor, weight: torch.Tensor, bias) -> bool:
+def _wide_product_chosen(x: torch.Tensor, weight: torch.Tensor, bias, policy: ProductPolicy) -> bool:
     """Does a plain product of many bfloat16 rows go through the wide-tile kernel? Only where a
     tuning start-up has timed it against the library's tuned kernel on these very shapes and
     found it faster (measured: the 7B shape's down product, 279 against 351 us)."""
     M, K = x.shape
-    if M < WIDE_PRODUCT_MIN_ROWS or not _product_choices and not _tuning:
+    if M < WIDE_PRODUCT_MIN_ROWS or not policy.product_choices and not policy.tuning:
         return False
     key = (weight.shape[0], K, bias is not None)
-    choice = _product_choices.get(key)
-    if choice is None and _tuning and x.is_contiguous():
+    choice = policy.product_choices.get(key)
+    if choice is None and policy.tuning and x.is_contiguous():
         if _load("gemm_tile").cw_gemm_bf16_wide_tiles(0, M, key[0], K, K) >= WIDE_PRODUCT_MIN_TILES:
             library = _timed_us(lambda: _library_product(x, weight, bias))
             own = _timed_us(lambda: linear_tiled(x, weight, bias, wide=True))
             choice = own <= library
         else:
             choice = False
-        _product_choices[key] = choice
+        policy.product_choices[key] = choice
     return bool(choice) and x.is_contiguous()
 
 
@@ -650,11 +663,13 @@ def swiglu_norm_fusable(M: int, two_i: int, K: int, dtype, gate_up_weight, delta
             and bool(_load("gemm").cw_gemm_bf16_swiglu_normed_ok(M, two_i, K)))
 
 
-def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
+def linear_swiglu(x, gate_up_weight: torch.Tensor, policy: "ProductPolicy | None" = None) -> torch.Tensor:
     """silu(x @ gate.T) * (x @ up.T) for gate_up_weight = [gate; up] stacked along dim 0.
 
     Few bfloat16 rows: one kernel that streams the weights once and applies the gate in its
-    epilogue. Otherwise the product followed by the gate kernel."""
+    epilogue. Otherwise the product followed by the gate kernel, or (``policy``, see ``linear``)
+    a tiled kernel with the gate in its epilogue."""
+    policy = policy if policy is not None else DEFAULT_POLICY
     if isinstance(x, LazyAddNorm):
         M, K = x.shape
         two_i = gate_up_weight.shape[0]
@@ -683,17 +698,17 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
                "gemm_bf16_skinny(swiglu)")
         return out
     if x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and K % 8 == 0 and x.is_contiguous():
-        if HIP_PRODUCTS:
+        if policy.hip_products:
             return linear_tiled(x, gate_up_weight, swiglu=True)
         if wide_swiglu_pays(M, two_i, K, K):
             # with enough rows the shape of the weights decides, and a start-up that tunes the
             # library's products has measured it for this model's
             measured = M >= WIDE_SWIGLU_MIN_ROWS
-            if measured and _tuning and (two_i, K) not in _swiglu_choices:
-                _swiglu_choices[(two_i, K)] = _measure_swiglu(x, gate_up_weight, out)
-            if not measured or _swiglu_choices.get((two_i, K), True):
+            if measured and policy.tuning and (two_i, K) not in policy.swiglu_choices:
+                policy.swiglu_choices[(two_i, K)] = _measure_swiglu(x, gate_up_weight, out)
+            if not measured or policy.swiglu_choices.get((two_i, K), True):
                 return linear_tiled(x, gate_up_weight, swiglu=True, wide=True)
-    return silu_mul(linear(x, gate_up_weight), out)
+    return silu_mul(linear(x, gate_up_weight, policy=policy), out)
 
 
 _zero_rows: dict = {}

@@ -238,6 +238,7 @@ class PagedAttention(Part):
         s = self.spec
         nh, nkv, hd = s.num_heads, s.num_kv_heads, s.head_dim
         T = x.shape[0]
+        policy = getattr(ctx, "products", None)
         fused = getattr(self.position, "project_rotate_store", None) if cache.writes else None
         qkv = None
         if fused is not None:
@@ -245,13 +246,13 @@ class PagedAttention(Part):
         if qkv is not None:
             pass  # q only, [T, nh * hd]: keys and values are in the cache already
         elif cache.writes:
-            qkv = ops.linear(x, self.qkv_weight)
+            qkv = ops.linear(x, self.qkv_weight, policy=policy)
             self.position.rotate_and_store(
                 qkv, self.qkv_bias, ctx.positions, ctx.slots[cache.group], nh, nkv, hd, cache.k, cache.v
             )
         else:
             # the keys and values of another entry are read: only queries are made here
-            qkv = ops.linear(x, self.qkv_weight[: self.q_width])
+            qkv = ops.linear(x, self.qkv_weight[: self.q_width], policy=policy)
             bias = self.qkv_bias[: self.q_width] if self.qkv_bias is not None else None
             self.position.rotate_and_store(qkv, bias, ctx.positions, None, nh, 0, hd, None, None)
         out = torch.empty((T, self.q_width), dtype=x.dtype, device=x.device)
@@ -292,4 +293,4 @@ class PagedAttention(Part):
                 workspace = torch.empty(need, dtype=torch.float32, device=x.device)
             ops.attention(items=plan.single_items, n_items=plan.n_single, rows=16, gh=plan.gh_single,
                           n_splits=plan.single_splits, workspace=workspace, **common)
-        return ops.linear(out, self.out_weight, self.out_bias, partial_ok=True)
+        return ops.linear(out, self.out_weight, self.out_bias, partial_ok=True, policy=policy)

@@ -82,4 +82,4 @@ class LinearHead(Part):
         return [self.weight]
 
     def forward(self, rows: torch.Tensor, ctx) -> torch.Tensor:
-        return ops.linear(rows, self.weight, out_dtype=torch.float32)
+        return ops.linear(rows, self.weight, out_dtype=torch.float32, policy=getattr(ctx, "products", None))

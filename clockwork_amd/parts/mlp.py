@@ -33,4 +33,5 @@ class SwiGLU(Part):
         return ops.swiglu_norm_fusable(n_tokens, 2 * I, H, dtype, self.gate_up, delta)
 
     def forward(self, x, ctx) -> torch.Tensor:
-        return ops.linear(ops.linear_swiglu(x, self.gate_up), self.down, partial_ok=True)
+        policy = getattr(ctx, "products", None)
+        return ops.linear(ops.linear_swiglu(x, self.gate_up, policy=policy), self.down, partial_ok=True, policy=policy)

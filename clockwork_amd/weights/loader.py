@@ -14,12 +14,17 @@ from pathlib import Path
 
 from clockwork_amd.config.spec import ParamSpec, WeightTarget
 from clockwork_amd.weights.checkpoint import CheckpointIndex, WeightMismatchError
+from clockwork_amd.weights.transforms import apply_transform, transformed_shape
 
 
-def read_config_json(model_dir: str | Path) -> dict:
-    path = Path(model_dir) / "config.json"
+def read_config_json(model: str | Path) -> dict:
+    """The architecture's configuration: ``model`` is a folder that holds a config.json, or (for
+    a model that needs no checkpoint: random weights) such a file itself."""
+    path = Path(model)
+    if path.is_dir():
+        path = path / "config.json"
     if not path.is_file():
-        raise FileNotFoundError(f"no config.json in {model_dir}")
+        raise FileNotFoundError(f"no config.json in {model}")
     return json.loads(path.read_text(encoding="utf-8"))
 
 
@@ -88,8 +93,11 @@ def load_parameters(
         if not all(present):
             continue  # optional and absent
         spec = param_specs[target.param]
-        rows = sum(shape[0] for shape in target.source_shapes)
-        full_shape = (rows, *target.source_shapes[0][1:])
+        # the sources as they are after the target's transform (a transpose, a slice of rows): these
+        # are what is stacked along dim 0
+        shapes = [transformed_shape(target.transform, shape) for shape in target.source_shapes]
+        rows = sum(shape[0] for shape in shapes)
+        full_shape = (rows, *shapes[0][1:])
         if tuple(spec.shape) != full_shape:
             raise RuntimeError(
                 f"weight plan for {target.param} yields {full_shape}, the part declares {spec.shape}"
@@ -100,8 +108,8 @@ def load_parameters(
         dtype = _target_dtype(spec, stored, compute_dtype)
         out = torch.empty(full_shape, dtype=dtype, device=device)
         row = 0
-        for name, shape in zip(target.sources, target.source_shapes):
-            out[row : row + shape[0]].copy_(index.read(name))
+        for name, shape in zip(target.sources, shapes):
+            out[row : row + shape[0]].copy_(apply_transform(target.transform, index.read(name)))
             row += shape[0]
         params[target.param] = out
     if hasattr(index, "close"):

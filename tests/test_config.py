@@ -74,6 +74,45 @@ def test_dtype_whitelist():
         EngineConfig.defaults("m", dtype="float16").model.torch_dtype()
 
 
+def test_random_weights_are_a_mode_of_the_configuration_and_of_the_command_line(tmp_path):
+    """clockwork/engine/loader.py:82-103 builds a model from a seed without a checkpoint; here that
+    is ``weights: random`` + ``weight_seed`` in the model section, ``--random-weights SEED`` on
+    the command line, and ``model`` may then name a bare config.json."""
+    import json
+
+    from clockwork_amd import cli
+    from clockwork_amd.weights.loader import read_config_json
+
+    cfg = EngineConfig.defaults("m")
+    assert (cfg.model.weights, cfg.model.weight_seed) == ("checkpoint", 0)
+    cfg.apply_overrides(["weights=random", "weight_seed=7"])
+    assert (cfg.model.weights, cfg.model.weight_seed) == ("random", 7)
+    with pytest.raises(ValueError, match="weights 'noise'"):
+        cfg.set("weights", "noise")
+    assert cfg.model.weights == "random"  # a refused value changes nothing
+    with pytest.raises(ValueError, match="weights 'noise'"):
+        EngineConfig.defaults("m", weights="noise")
+    path = tmp_path / "engine.yaml"
+    path.write_text("model:\n  model: /m/config.json\n  weights: random_device\n  weight_seed: 3\n")
+    from_yaml = EngineConfig.from_yaml(path)
+    assert (from_yaml.model.weights, from_yaml.model.weight_seed) == ("random_device", 3)
+
+    config_json = tmp_path / "tiny.json"
+    config_json.write_text(json.dumps(TINY_B))
+    args, cfg, prompts = cli.parse_generate(["--model", str(config_json), "--random-weights", "2", "--prompt-ids", "5,17,3",
+                                             "--max-tokens", "8"])
+    assert (cfg.model.model, cfg.model.weights, cfg.model.weight_seed) == (str(config_json), "random", 2)
+    assert prompts == [[5, 17, 3]] and args.max_tokens == 8
+    _, cfg, _ = cli.parse_generate(["--model", "/some/dir", "--prompt-ids", "1"])
+    assert cfg.model.weights == "checkpoint"
+    # a file stands for itself, a folder for the config.json inside it
+    assert read_config_json(config_json) == TINY_B
+    (tmp_path / "config.json").write_text(json.dumps(TINY_A))
+    assert read_config_json(tmp_path) == TINY_A
+    with pytest.raises(FileNotFoundError):
+        read_config_json(tmp_path / "nothing")
+
+
 # ------------------------------------------------------------------ the model's own keys
 def test_qwen2_config_reads_every_size_from_the_dict():
     for d in (TINY_A, TINY_B, TINY_C):

@@ -322,6 +322,36 @@ def test_command_line(model_dirs, tmp_path, capsys):
         cli.main(["--config", str(yaml_path), "--set", "nonsense=1", "--prompt-ids", "1"])
 
 
+def test_command_line_with_random_weights_equals_the_written_folder(tmp_path, capsys):
+    """``--model config.json --random-weights SEED`` serves the very model that ``make-random``
+    writes into a folder from the same file and seed: the same tokens, and the plain
+    implementation's on that folder."""
+    import json
+
+    from clockwork_amd import cli
+    from tests.configs import TINY_B
+
+    config_json = tmp_path / "tiny_b.json"
+    config_json.write_text(json.dumps(TINY_B))
+    common = ["--set", "block_size=8", "--set", "num_blocks=64", "--prompt-ids", "5,17,3", "--max-tokens", "8", "--ignore-eos"]
+    assert cli.main(["--model", str(config_json), "--random-weights", "2", *common]) == 0
+    from_seed = json.loads(capsys.readouterr().out.strip().splitlines()[-1])["token_ids"]
+    folder = tmp_path / "written"
+    assert cli.main(["make-random", "--config-json", str(config_json), "--seed", "2", "--out", str(folder)]) == 0
+    capsys.readouterr()
+    assert cli.main(["--model", str(folder), *common]) == 0
+    from_folder = json.loads(capsys.readouterr().out.strip().splitlines()[-1])["token_ids"]
+    assert from_seed == from_folder == PlainQwen2(folder).greedy([5, 17, 3], 8)
+    # another seed is another model
+    assert cli.main(["--model", str(config_json), "--random-weights", "3", *common]) == 0
+    assert json.loads(capsys.readouterr().out.strip().splitlines()[-1])["token_ids"] != from_seed
+    # and the configuration key does the same through the Python entry point
+    from clockwork_amd.engine.llm_engine import LLMEngine
+
+    cfg = EngineConfig.defaults(str(config_json), weights="random", weight_seed=2, block_size=8, num_blocks=64)
+    assert LLMEngine(cfg).generate([[5, 17, 3]], greedy(8))[0].token_ids == from_seed
+
+
 def test_cache_size_left_open_is_what_the_scheduler_can_use(model_dirs):
     # a tiny model on a large card: the cap (twice max_num_seqs requests of max_model_len tokens) decides
     eng = engine(model_dirs["A"], num_blocks=0, max_num_seqs=4, max_model_len=64)

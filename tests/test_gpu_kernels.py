@@ -605,38 +605,40 @@ def test_gate_up_of_a_long_portion_goes_through_the_wide_tile_kernel():
 
 def test_a_tuning_start_up_measures_which_gate_up_product_is_faster():
     """While the library tunes, the first long portion of a weight shape times both ways and the
-    choice is kept: later products of that shape follow it."""
+    choice is kept by the engine's own policy: later products of that shape follow it, and a
+    call on behalf of another engine (another policy) knows nothing of it."""
     from clockwork_amd import ops
 
     x = torch.randn(1024, 1536, device=DEV).to(torch.bfloat16)
     w = (torch.randn(2 * 8960, 1536, device=DEV) / 40).to(torch.bfloat16)
     key = (2 * 8960, 1536)
-    kept = ops._swiglu_choices.pop(key, None)
+    policy = ops.ProductPolicy()
     calls = []
     real = ops.linear_tiled
     ops.linear_tiled = lambda *a, **k: (calls.append(k), real(*a, **k))[1]
     try:
-        ops._tuning = True   # what library_tuning() sets, without touching the library's own tuner
-        first = ops.linear_swiglu(x, w)
-        ops._tuning = False
-        assert key in ops._swiglu_choices
+        policy.tuning = True   # what library_tuning(policy) sets, without touching the library's own tuner
+        first = ops.linear_swiglu(x, w, policy=policy)
+        policy.tuning = False
+        assert key in policy.swiglu_choices and not ops.DEFAULT_POLICY.swiglu_choices
         for choice in (False, True):
-            ops._swiglu_choices[key] = choice
+            policy.swiglu_choices[key] = choice
             calls.clear()
-            again = ops.linear_swiglu(x, w)
+            again = ops.linear_swiglu(x, w, policy=policy)
             assert bool(calls) == choice
             torch.testing.assert_close(again.float(), first.float(), rtol=2e-2, atol=2e-2)
         # fewer rows than the measurement speaks for: the rule, not the choice
-        ops._swiglu_choices[key] = False
+        policy.swiglu_choices[key] = False
         calls.clear()
-        ops.linear_swiglu(x[:512], w)
+        ops.linear_swiglu(x[:512], w, policy=policy)
         assert calls
+        # another engine's calls follow the rule too, whatever this one has measured
+        calls.clear()
+        ops.linear_swiglu(x, w, policy=ops.ProductPolicy())
+        ops.linear_swiglu(x, w)
+        assert len(calls) == 2
     finally:
-        ops._tuning = False
         ops.linear_tiled = real
-        ops._swiglu_choices.pop(key, None)
-        if kept is not None:
-            ops._swiglu_choices[key] = kept
 
 
 def test_a_tuning_start_up_times_plain_products_too():
@@ -648,35 +650,33 @@ def test_a_tuning_start_up_times_plain_products_too():
     w = (torch.randn(3584, 1024, device=DEV) / 32).to(torch.bfloat16)     # 8 x 19 tiles
     small = (torch.randn(512, 1024, device=DEV) / 32).to(torch.bfloat16)  # 8 x 3 tiles
     b = torch.randn(3584, device=DEV).to(torch.bfloat16)
-    kept = dict(ops._product_choices)
-    ops._product_choices.clear()
+    policy = ops.ProductPolicy()
     calls = []
     real = ops.linear_tiled
     ops.linear_tiled = lambda *a, **k: (calls.append(k), real(*a, **k))[1]
     try:
-        want = ops.linear(x, w, b)
-        assert not calls and not ops._product_choices       # nothing is timed outside a tuning start-up
-        ops._tuning = True
-        ops.linear(x, w, b)
-        ops.linear(x, small)
-        ops._tuning = False
-        assert (3584, 1024, True) in ops._product_choices and ops._product_choices[(512, 1024, False)] is False
+        want = ops.linear(x, w, b, policy=policy)
+        assert not calls and not policy.product_choices       # nothing is timed outside a tuning start-up
+        policy.tuning = True
+        ops.linear(x, w, b, policy=policy)
+        ops.linear(x, small, policy=policy)
+        policy.tuning = False
+        assert (3584, 1024, True) in policy.product_choices and policy.product_choices[(512, 1024, False)] is False
+        assert not ops.DEFAULT_POLICY.product_choices
         for choice in (True, False):
-            ops._product_choices[(3584, 1024, True)] = choice
+            policy.product_choices[(3584, 1024, True)] = choice
             calls.clear()
-            got = ops.linear(x, w, b)
+            got = ops.linear(x, w, b, policy=policy)
             assert bool(calls) == choice
             torch.testing.assert_close(got.float(), want.float(), rtol=2e-2, atol=2e-2)
         calls.clear()
-        ops._product_choices[(3584, 1024, True)] = True
-        ops.linear(x[:512], w, b)          # too few rows for the measurement to speak for
-        ops.linear(x, w)                   # another shape (no bias): never timed
+        policy.product_choices[(3584, 1024, True)] = True
+        ops.linear(x[:512], w, b, policy=policy)          # too few rows for the measurement to speak for
+        ops.linear(x, w, policy=policy)                   # another shape (no bias): never timed
+        ops.linear(x, w, b)                               # no engine behind the call: the library
         assert not calls
     finally:
-        ops._tuning = False
         ops.linear_tiled = real
-        ops._product_choices.clear()
-        ops._product_choices.update(kept)
 
 
 def test_hip_products_switch_routes_large_products_to_the_tiled_kernel():
@@ -689,14 +689,16 @@ def test_hip_products_switch_routes_large_products_to_the_tiled_kernel():
     calls = []
     real = ops.linear_tiled
     ops.linear_tiled = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
-    ops.use_hip_products(True)
+    own = ops.ProductPolicy(hip_products=True)
     try:
-        own_y, own_g = ops.linear(x, w, b), ops.linear_swiglu(x, w)
-        logits = ops.linear(x, w, out_dtype=torch.float32)
+        own_y, own_g = ops.linear(x, w, b, policy=own), ops.linear_swiglu(x, w, policy=own)
+        logits = ops.linear(x, w, out_dtype=torch.float32, policy=own)
+        assert len(calls) == 3
+        ops.linear(x, w, b)   # a call of another engine, or of none, stays with the library
+        assert len(calls) == 3
     finally:
-        ops.use_hip_products(False)
         ops.linear_tiled = real
-    assert len(calls) == 3 and logits.dtype == torch.float32
+    assert logits.dtype == torch.float32
     torch.testing.assert_close(own_y.float(), lib_y.float(), rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(own_g.float(), lib_g.float(), rtol=2e-2, atol=2e-2)
 

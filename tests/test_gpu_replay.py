@@ -488,8 +488,7 @@ def test_replay_with_the_tiled_products_instead_of_the_library(model_dirs):
         got = replay.run_trace(runner, replay.mixed(requests))
     finally:
         ops.linear_tiled = real
-        ops.use_hip_products(False)
-    assert calls
+    assert calls and runner.products.hip_products and not ops.DEFAULT_POLICY.hip_products
     _check(got, _plain(name, model_dirs), "bfloat16")
 
 
@@ -882,43 +881,33 @@ def test_captured_graphs_hold_kernel_nodes_only(tmp_path, tuned):
         assert set(kinds) == {"kernel"} and kinds["kernel"] > 10, f"graph {key} holds {kinds}"
 
 
-def test_a_graph_with_a_memset_node_is_not_kept(model_dirs):
-    """A part whose step clears a buffer with a memset (torch's zero_ of a large tensor is one):
-    the captured graph holds a node that is no kernel, so the runner drops it and runs that
-    batch shape eagerly from then on, with the same logits."""
-    from clockwork_amd.engine.graph_nodes import node_kinds
+def test_a_graph_with_a_memset_node_is_not_kept(model_dirs, monkeypatch):
+    """A captured step in which something recorded a node that is no kernel launch (a library
+    product that clears a workspace with a memset) is not kept: the runner drops the graph and
+    runs that batch shape eagerly from then on, with the same logits. No memset is put under a
+    capture here: the walk over the captured graph's nodes is made to report one."""
+    from clockwork_amd.engine import model_runner
 
     name = "B"
     cfg, _, block_size = TINY_CONFIGS[name]
-    # what the walk reports for a capture with a memset in it
-    scratch = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
-    import ctypes
-
-    from clockwork_amd.engine import graph_nodes
-
-    hip = graph_nodes._runtime()
-    hip.hipMemsetAsync.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p]
-    graph = torch.cuda.CUDAGraph(keep_graph=True)
-    with torch.cuda.graph(graph):
-        scratch.add_(1)
-        assert hip.hipMemsetAsync(scratch.data_ptr(), 0, scratch.numel(), torch.cuda.current_stream().cuda_stream) == 0
-    kinds = node_kinds(graph)
-    assert kinds["kernel"] >= 1 and kinds["memset"] == 1
-    graph.reset()   # never replayed
-
     toks = torch.randint(0, cfg["vocab_size"], (40,), generator=torch.Generator().manual_seed(2)).tolist()
     steps = [{"entries": [{"id": "x", "tokens": [t], "want": [0]}], "end": []} for t in toks]
-    clean = replay.run_trace(replay.make_runner(model_dirs[name], "float32", block_size, 8), [dict(s) for s in steps])
+    clean_runner = replay.make_runner(model_dirs[name], "float32", block_size, 8)
+    clean = replay.run_trace(clean_runner, [dict(s) for s in steps])
+    assert isinstance(clean_runner._graphs[(1, 512)], tuple)  # the same steps do replay a graph otherwise
+    real_walk = model_runner.node_kinds
+    walked = []
+
+    def walk_that_finds_a_memset(graph):
+        kinds = dict(real_walk(graph))
+        walked.append(dict(kinds))
+        kinds["memset"] = 1
+        return kinds
+
+    monkeypatch.setattr(model_runner, "node_kinds", walk_that_finds_a_memset)
     runner = replay.make_runner(model_dirs[name], "float32", block_size, 8)
-    norm = runner.model.final_norm
-    real = norm.forward
-
-    def with_memset(resid, delta, rows=None):
-        hip.hipMemsetAsync(scratch.data_ptr(), 0, scratch.numel(), torch.cuda.current_stream().cuda_stream)
-        return real(resid, delta, rows)
-
-    norm.forward = with_memset
     got = replay.run_trace(runner, [dict(s) for s in steps])
+    assert len(walked) == 1 and set(walked[0]) == {"kernel"}   # captured once, never again
     assert runner._graphs[(1, 512)] == "eager" and runner.graph_nodes[(1, 512)].get("memset") == 1
     for key in clean:
         torch.testing.assert_close(got[key], clean[key], rtol=2e-6, atol=2e-6)
@@ -945,11 +934,11 @@ def test_negative_control_a_small_weight_change_breaks_the_match(model_dirs, tmp
         replay.compare(got, {"r0": _plain(name, model_dirs)["r3"]}, **TOL["float32"])
 
 
-def _run_program(model_dir, dtype, steps, out, max_tokens):
+def _run_program(model_dir, dtype, steps, out, max_tokens, page=None):
     lines = [json.dumps({"step": i, **s}) for i, s in enumerate(steps)]
     proc = subprocess.run(
         [sys.executable, str(REPO / "bin" / "trace_run"), "--model", str(model_dir), "--dtype", dtype,
-         "--out", str(out), "--max-tokens", str(max_tokens)],
+         "--out", str(out), "--max-tokens", str(max_tokens), *([] if page is None else ["--page", str(page)])],
         input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600,
     )
     assert proc.returncode == 0, proc.stderr[-2000:]
@@ -980,13 +969,14 @@ def _read_program_output(out, steps, vocab, starts=None) -> dict:
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(model_dirs, tmp_path, dtype):
-    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and 'done <step>' out."""
+    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and 'done <step>' out;
+    once with its own page size, once with pages of 8 tokens (``--page``)."""
     name = "A"
     requests = {k: v for k, v in list(_requests(name).items())[:5]}
     steps = replay.mixed(requests)
     max_tokens = 4 * 64 * -(-max(len(t) for t in requests.values()) // 64)
     out = tmp_path / "out"
-    _run_program(model_dirs[name], dtype, steps, out, max_tokens)
+    _run_program(model_dirs[name], dtype, steps, out, max_tokens, page=None if dtype == "float32" else 8)
     got = _read_program_output(out, steps, TINY_CONFIGS[name][0]["vocab_size"])
     assert len(got) == sum(len(t) for t in requests.values())
     _check(got, _plain(name, model_dirs), dtype)

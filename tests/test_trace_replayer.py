@@ -128,3 +128,15 @@ def test_random_traces_are_what_they_say():
                 assert lengths.pop(rid) == len(seqs[rid])
         assert not lengths
     assert min(kinds.values()) > 50
+
+
+def test_the_program_sizes_its_pool_for_max_tokens_in_pages_of_the_given_size():
+    from clockwork_amd.engine.trace_run import PAGE, replay_config
+
+    cfg = replay_config("m", "float32", 256)
+    assert (cfg.cache.block_size, cfg.cache.num_blocks) == (PAGE, 256 // PAGE) and PAGE == 16
+    assert cfg.model.max_model_len == cfg.scheduler.max_model_len == 256   # one request may hold every page
+    assert not cfg.cache.enable_prefix_cache and cfg.cache.watermark == 0.0
+    cfg = replay_config("m", "bfloat16", 250, page=24)
+    assert (cfg.cache.block_size, cfg.cache.num_blocks, cfg.model.max_model_len) == (24, 11, 264)
+    assert replay_config("m", "float32", 0, page=8).cache.num_blocks == 1

@@ -36,13 +36,6 @@ def _with_workspace(lib, logits, stream):
     return out
 
 
-def _static(lib, logits, stream):
-    n, V = logits.shape
-    out = torch.full((n,), -7, dtype=torch.int32, device=logits.device)
-    assert lib.cw_argmax_static(logits.data_ptr(), logits.stride(0), n, V, out.data_ptr(), stream) == 0
-    return out
-
-
 def test_argmax_without_allocation_equals_the_one_with_a_workspace():
     lib = _library()
     device = torch.device("cuda", torch.cuda.current_device())
@@ -60,17 +53,48 @@ def test_argmax_without_allocation_equals_the_one_with_a_workspace():
     small[2, 4_096] = 40.0                 # the last element, alone in the second chunk
     outputs = []
     for logits in (big, small):
-        before = torch.cuda.memory_stats(device)["allocation.all.allocated"]
-        got = _static(lib, logits, stream)
-        # ``out`` above is the test's own tensor; the call itself asked torch for nothing
-        assert torch.cuda.memory_stats(device)["allocation.all.allocated"] - before == 1
-        outputs.append((got, _with_workspace(lib, logits, stream), logits))
+        n, V = logits.shape
+        out = torch.full((n,), -7, dtype=torch.int32, device=device)
+        torch.cuda.synchronize()
+        # neither torch's allocator nor the runtime's (hipMalloc: the device's free memory) is asked
+        before = torch.cuda.memory_stats(device)["allocation.all.allocated"], torch.cuda.mem_get_info(device)[0]
+        assert lib.cw_argmax_static(logits.data_ptr(), logits.stride(0), n, V, out.data_ptr(), stream) == 0
+        torch.cuda.synchronize()
+        assert (torch.cuda.memory_stats(device)["allocation.all.allocated"], torch.cuda.mem_get_info(device)[0]) == before
+        outputs.append((out, _with_workspace(lib, logits, stream), logits))
     torch.cuda.synchronize()
     for got, want, logits in outputs:
         assert torch.equal(got.cpu(), want.cpu())
         ref = torch.where(torch.isnan(logits), torch.full_like(logits, float("-inf")), logits).argmax(dim=1)
         assert torch.equal(got.cpu().long(), ref.cpu())
     assert int(outputs[0][0][3]) == 5 and int(outputs[0][0][5]) == 0 and int(outputs[1][0][2]) == 4_096
+
+
+def test_argmax_without_allocation_inside_a_captured_graph():
+    """What the entry point is for: a caller under HIP-graph capture, where an allocation is an
+    error. The call is captured (after ``cw_argmax_static_init``, which looks the array up and may
+    not run under capture), replayed several times over changing inputs with eager work between
+    the replays, and every replay is checked against the ordinary entry point."""
+    lib = _library()
+    device = torch.device("cuda", torch.cuda.current_device())
+    assert lib.cw_argmax_static_init() == 0
+    gen = torch.Generator().manual_seed(23)
+    logits = torch.randn(9, 70_001, generator=gen).to(device)
+    out = torch.full((9,), -7, dtype=torch.int32, device=device)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        code = lib.cw_argmax_static(logits.data_ptr(), logits.stride(0), 9, 70_001, out.data_ptr(),
+                                    torch.cuda.current_stream().cuda_stream)
+    assert code == 0
+    for trial in range(3):
+        logits.copy_(torch.randn(9, 70_001, generator=gen))
+        logits[trial, 70_000 - trial] = 30.0
+        graph.replay()
+        torch.cuda.synchronize()
+        want = _with_workspace(lib, logits, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), want.cpu()) and int(out[trial]) == 70_000 - trial
 
 
 def test_argmax_without_allocation_refuses_more_rows_than_its_array_holds():
