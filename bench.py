@@ -134,18 +134,21 @@ def time_decode(cfg, runner, batch: int, steps: int, warmup: int, sampling=None,
 
 # per-step times of the last ``time_decode`` run, from events on the GPU's queue (milliseconds)
 LAST_STEP_TIMES: dict = {}
+# how the last ``time_prefill`` chose its time, and the fastest and slowest of its runs
+LAST_PREFILL_TIMES: dict = {}
 
 
 def time_prefill(cfg, runner, repeats: int = 6, total: int = PROMPT_LEN):
     """Seconds for one prompt of ``total`` tokens, in portions of PROMPT_LEN tokens (one step when
-    total is PROMPT_LEN, the recorded measurement): the best of ``repeats`` runs."""
+    total is PROMPT_LEN, the recorded measurement): the median of ``repeats`` runs after one that
+    is not counted; ``LAST_PREFILL_TIMES`` keeps the runs' best and worst beside it."""
     import torch
 
     from clockwork_amd.engine.batch import StepEntry
 
     vocab = runner.spec.vocab_size
     tokens = torch.randint(0, vocab, (total,), generator=torch.Generator().manual_seed(99)).tolist()
-    best = None
+    runs = []
     for i in range(repeats + 1):
         _sync()
         t0 = time.perf_counter()
@@ -157,9 +160,13 @@ def time_prefill(cfg, runner, repeats: int = 6, total: int = PROMPT_LEN):
         dt = time.perf_counter() - t0
         runner.release("prefill")
         if i > 0:  # the first run pays for library heuristics and allocations
-            best = dt if best is None else min(best, dt)
+            runs.append(dt)
     assert logits.shape == (1, vocab)
-    return best
+    runs.sort()
+    median = runs[len(runs) // 2] if len(runs) % 2 else 0.5 * (runs[len(runs) // 2 - 1] + runs[len(runs) // 2])
+    LAST_PREFILL_TIMES.clear()
+    LAST_PREFILL_TIMES.update(stat=f"median of {len(runs)} runs", best_ms=round(1e3 * runs[0], 3), worst_ms=round(1e3 * runs[-1], 3))
+    return median
 
 
 def run_mixed(args) -> dict:
@@ -473,7 +480,7 @@ def main() -> int:
     if args.only_prefill:
         t = time_prefill(cfg, runner, total=args.prompt_len)
         print(json.dumps({"prefill_ms": round(1e3 * t, 3), "tokens": args.prompt_len, "portion": PROMPT_LEN,
-                          "tokens_per_s": round(args.prompt_len / t, 1)}))
+                          "tokens_per_s": round(args.prompt_len / t, 1), **LAST_PREFILL_TIMES}))
         return 0
     sampling = (args.temperature, args.top_k, args.top_p) if args.temperature > 0 else None
     elapsed, mean_ctx = time_decode(cfg, runner, args.batch, args.steps, args.warmup, sampling, args.prompt_len)
@@ -531,6 +538,7 @@ def main() -> int:
             "tokens": PROMPT_LEN,
             "ms": round(1e3 * t, 3),
             "frac": round(flops / t / PEAK_FLOPS[args.dtype], 4),
+            **LAST_PREFILL_TIMES,
         }
         points = {}
         for b in (1, 64):

@@ -536,27 +536,32 @@ CW_EXPORT int cw_copy_pages(void* pool, int planes, int64_t num_blocks, int64_t 
 
 // ---------------------------------------------------------------- fresh state slots
 // The state pool of a group is [entries, slots, row_bytes]. A request whose first token runs in
-// this step (starts[r] == 0) begins from an empty state: its slot's row is cleared in every
-// entry, by a kernel (no memset: the launch is part of steps that are captured as graphs).
-// slots[r] < 0 or >= num_slots: the row belongs to no request, nothing is cleared.
-__global__ void zero_state_rows_kernel(uint32_t* __restrict__ pool, int64_t entry_words, int64_t row_words,
-                                       int num_slots, const int* __restrict__ slots,
-                                       const int* __restrict__ starts) {
+// this step (starts[r] == 0) begins from the fresh state: its slot's row is set, in every entry, to
+// the row of the pool's template slot, by a kernel (no memset or copy node: the launch is part of
+// steps that are captured as graphs). slots[r] < 0 or >= num_slots: the row belongs to no request,
+// nothing is written.
+__global__ void fresh_state_rows_kernel(uint32_t* __restrict__ pool, int64_t entry_words, int64_t row_words,
+                                        int num_slots, int fresh_slot, const int* __restrict__ slots,
+                                        const int* __restrict__ starts) {
   const int r = blockIdx.x, entry = blockIdx.y;
   const int slot = slots[r];
   if (starts[r] != 0 || slot < 0 || slot >= num_slots) return;
   uint32_t* row = pool + entry * entry_words + (int64_t)slot * row_words;
-  for (int64_t i = threadIdx.x; i < row_words; i += blockDim.x) row[i] = 0u;
+  const uint32_t* fresh = pool + entry * entry_words + (int64_t)fresh_slot * row_words;
+  for (int64_t i = threadIdx.x; i < row_words; i += blockDim.x) row[i] = fresh[i];
 }
 
-CW_EXPORT int cw_zero_state_rows(void* pool, int entries, int num_slots, int64_t row_bytes, const int* slots,
-                                 const int* starts, int n, hipStream_t stream) {
+// pool [entries, pool_slots, row_bytes]: slots [0, num_slots) may be set, slot ``fresh_slot`` (one of
+// the pool's, outside that range) holds what a fresh state is.
+CW_EXPORT int cw_fresh_state_rows(void* pool, int entries, int pool_slots, int num_slots, int fresh_slot,
+                                  int64_t row_bytes, const int* slots, const int* starts, int n, hipStream_t stream) {
   if (entries <= 0 || num_slots <= 0 || row_bytes <= 0 || (row_bytes & 3) || n < 0 || !pool || !slots || !starts)
     return CW_ERR_ARG;
+  if (num_slots > pool_slots || fresh_slot < num_slots || fresh_slot >= pool_slots) return CW_ERR_ARG;
   if (n == 0) return CW_OK;
   if (entries > 65535) return CW_ERR_SIZE;
-  hipLaunchKernelGGL(zero_state_rows_kernel, dim3(n, entries), dim3(256), 0, stream, (uint32_t*)pool,
-                     (int64_t)num_slots * (row_bytes / 4), row_bytes / 4, num_slots, slots, starts);
+  hipLaunchKernelGGL(fresh_state_rows_kernel, dim3(n, entries), dim3(256), 0, stream, (uint32_t*)pool,
+                     (int64_t)pool_slots * (row_bytes / 4), row_bytes / 4, num_slots, fresh_slot, slots, starts);
   return cw_launch_status();
 }
 

@@ -62,7 +62,8 @@ class StepContext:
         self.block_size = 0
         # device int32 tensors
         self.token_ids = None
-        self.positions = None
+        self.positions = None            # [T] what the parts read as positions (the embedding part may replace it)
+        self.sequence_positions = None   # [T] each token's index in its request: start + i
         self.cu_q = None          # [R + 1]
         self.ctx_lens = None      # [R]  keys of each request once this step's tokens are cached
         self.starts = None        # [R]  position of each request's first token in this step
@@ -148,6 +149,7 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int
     views = packer.upload(device)
     ctx._packer = packer
     ctx.token_ids, ctx.positions, ctx.cu_q = views[i_tok], views[i_pos], views[i_cu]
+    ctx.sequence_positions = ctx.positions
     ctx.ctx_lens, ctx.starts = views[i_ctx], views[i_start]
     ctx.state_slots, ctx.logit_rows = views[i_state], views[i_rows]
     for i_slots, i_table, width in group_idx:
@@ -200,6 +202,7 @@ class StaticDecodeBatch:
         ctx.block_size = manager.block_size
         ctx.num_tokens = ctx.num_requests = ctx.num_logit_rows = size
         ctx.token_ids, ctx.positions = view("token_ids"), view("positions")
+        ctx.sequence_positions = ctx.positions
         ctx.ctx_lens, ctx.starts, ctx.state_slots = view("ctx_lens"), view("starts"), view("state_slots")
         ctx.cu_q = torch.arange(size + 1, dtype=torch.int32, device=device)
         ctx.logit_rows = torch.arange(size, dtype=torch.int32, device=device)
@@ -343,6 +346,7 @@ class StaticPortionBatch:
         ctx.block_size = manager.block_size
         ctx.num_tokens, ctx.num_requests, ctx.num_logit_rows = n, 1, int(wanted)
         ctx.token_ids, ctx.positions = view("token_ids"), view("positions")
+        ctx.sequence_positions = ctx.positions
         ctx.ctx_lens, ctx.starts, ctx.state_slots = view("ctx_lens"), view("starts"), view("state_slots")
         ctx.cu_q = view("cu_q")
         ctx.logit_rows = view("logit_rows") if wanted else torch.empty(0, dtype=torch.int32, device=device)
@@ -454,6 +458,7 @@ class StaticMixedBatch:
         ctx.block_size = manager.block_size
         ctx.num_tokens, ctx.num_requests, ctx.num_logit_rows = rows, requests, requests
         ctx.token_ids, ctx.positions = view("token_ids"), view("positions")
+        ctx.sequence_positions = ctx.positions
         ctx.ctx_lens, ctx.starts, ctx.state_slots = view("ctx_lens"), view("starts"), view("state_slots")
         ctx.cu_q, ctx.logit_rows = view("cu_q"), view("logit_rows")
         for g in range(n_groups):

@@ -434,7 +434,7 @@ class ModelRunner:
         captured step does it too), then the parts run."""
         ctx.products = self.products
         if self.pools.state:
-            self.pools.zero_fresh_state(ctx.state_slots, ctx.starts, ctx.num_requests)
+            self.pools.set_fresh_states(ctx.state_slots, ctx.starts, ctx.num_requests)
         return self.model.forward(ctx, self.caches)
 
     @torch.no_grad()

@@ -95,7 +95,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_rope_kv_write": [P, I, P, I, P, P, P, I, I, I, I, I, P, P, L, P],
             "cw_silu_mul": [P, P, I, I, I, P],
             "cw_copy_pages": [P, I, L, L, P, I, P],
-            "cw_zero_state_rows": [P, I, I, L, P, P, I, P],
+            "cw_fresh_state_rows": [P, I, I, I, I, L, P, P, I, P],
             "cw_bf16_to_f32": [P, P, L, P],
         },
         "gemm": {
@@ -361,18 +361,20 @@ def copy_pages(pool: torch.Tensor, pairs: torch.Tensor) -> None:
     _check(_load("core").cw_copy_pages(_ptr(pool), planes, num_blocks, block_bytes, _ptr(pairs), pairs.shape[0], _stream()), "copy_pages")
 
 
-def zero_state_rows(pool: torch.Tensor, slots: torch.Tensor, starts: torch.Tensor, n: int) -> None:
-    """pool [entries, num_slots, ...]: for each of the first ``n`` requests of a step that starts at
-    position 0 (``starts[r] == 0``), clear row ``slots[r]`` in every entry; a slot outside
-    [0, num_slots) clears nothing. A kernel, so a captured step may hold it."""
+def fresh_state_rows(pool: torch.Tensor, slots: torch.Tensor, starts: torch.Tensor, n: int) -> None:
+    """pool [entries, slots, ...], its last slot the template of a fresh state: for each of the
+    first ``n`` requests of a step that starts at position 0 (``starts[r] == 0``), set row
+    ``slots[r]`` to the template in every entry; a slot outside [0, slots - 1) writes nothing. A
+    kernel, so a captured step may hold it."""
     _gpu(pool, slots, starts)
     _i32(slots, n, "slots")
     _i32(starts, n, "starts")
-    if pool.dim() < 2:
-        raise KernelError("a state pool is [entries, slots, ...]")
+    if pool.dim() < 2 or pool.shape[1] < 2:
+        raise KernelError("a state pool is [entries, slots, ...] with the template as its last slot")
     row_bytes = (pool[0, 0].numel() if pool.dim() > 2 else 1) * pool.element_size()
-    _check(_load("core").cw_zero_state_rows(_ptr(pool), pool.shape[0], pool.shape[1], row_bytes, _ptr(slots),
-                                            _ptr(starts), int(n), _stream()), "zero_state_rows")
+    pool_slots = pool.shape[1]
+    _check(_load("core").cw_fresh_state_rows(_ptr(pool), pool.shape[0], pool_slots, pool_slots - 1, pool_slots - 1,
+                                             row_bytes, _ptr(slots), _ptr(starts), int(n), _stream()), "fresh_state_rows")
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, partial_ok: bool = False,

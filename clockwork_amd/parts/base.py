@@ -12,7 +12,11 @@ Roles and their run methods:
 
 * embedding:     ``forward(ctx) -> resid``: the float32 residual stream [T, H] of the step's
                  tokens (``ctx.token_ids``, ``ctx.positions``). May offer ``table()``, the
-                 [vocab, H] matrix a tied head uses.
+                 [vocab, H] matrix a tied head uses, and ``positions(ctx) -> tensor``: what
+                 ``ctx.positions`` holds for the parts of this step (an offset, several axes a
+                 token), made on the device from ``ctx.sequence_positions`` (int32 [T], each
+                 token's index in its request) before anything else runs; without it
+                 ``ctx.positions`` is ``ctx.sequence_positions``.
 * norm:          ``forward(resid, delta, rows=None) -> normed`` - ``resid`` is the
                  float32 residual stream [T, H]; ``delta`` (activation type, an
                  ``ops.PartialSums`` of that shape, or None)
@@ -34,7 +38,9 @@ Roles and their run methods:
                  ``forward(resid, delta, ctx, cache) -> delta`` wires norms, mixer and
                  feed-forward around the residual stream; the returned ``delta`` is the last
                  branch output, not yet added. The part named ``mixer`` owns the block's
-                 cache; the part named ``mixer_norm`` is the first to take the delta handed on.
+                 cache. Optional ``first_norm() -> part``: the norm that takes the delta handed
+                 on; if it has ``accepts_pending`` the block before may hand on two outputs
+                 (``ops.PendingPair``), without the hook it hands on one.
 * head:          ``forward(rows, ctx) -> logits``: float32 [n, vocab] for the final norm's rows.
                  A head whose spec has ``tied`` set gets ``use_embedding(embedding part)``
                  before ``bind``. ``matrices()``: what a step streams through it (byte counts).
@@ -84,13 +90,15 @@ class EntryCache:
     Key/value kind: ``k`` and ``v`` are flat [num_blocks * block_size, kv_heads, head_dim]
     views of the entry's pages, ``group`` indexes the step context's per-group block
     tables and slot mappings, ``writes`` is False when the entry reads another entry's
-    cache. State kind: ``state`` is [max_num_seqs, *shape]; the request's row is
-    ``ctx.state_slots[r]``.
+    cache. A mixer with planes of its own (``PagedRowsSpec``) finds each in ``planes`` by name,
+    a flat [num_blocks * block_size, *row shape] view addressed the same way. State kind:
+    ``state`` is [slots, *shape]; the request's row is ``ctx.state_slots[r]``.
     """
 
     group: int = -1
     k: Any = None
     v: Any = None
+    planes: Any = None   # {plane name: flat view}: ``k`` and ``v`` among them, or a mixer's own
     state: Any = None
     writes: bool = True
     block_size: int = 0

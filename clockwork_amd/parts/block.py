@@ -27,6 +27,10 @@ class PreNormBlock:
             "ffn_norm": self.ffn_norm,
         }
 
+    def first_norm(self):
+        """The norm that takes what the block before hands on (may it be two pending outputs?)."""
+        return self.mixer_norm
+
     def forward(self, resid, delta, ctx, cache):
         x = self.mixer_norm.forward(resid, delta)
         a = self.mixer.forward(x, ctx, cache)

@@ -139,12 +139,22 @@ class DecoderModel:
     def forward(self, ctx, caches) -> Optional[torch.Tensor]:
         """Run the step's tokens; returns float32 logits [len(ctx.logit_rows), vocab] or None
         when no logits are wanted. ``caches[i]`` is the EntryCache of run entry i."""
+        # what ``ctx.positions`` holds is the embedding part's to say: without its word every token
+        # carries its index in its request (``ctx.sequence_positions``, which stays what it is)
+        positions_of = getattr(self.embedding, "positions", None)
+        if positions_of is not None:
+            ctx.positions = positions_of(ctx)
         resid = self.embedding.forward(ctx)
         delta = None
         run = self.spec.run
         for i, entry in enumerate(run):
-            # may this block hand on two pending outputs? Only if the norm that comes next takes them
-            nxt = self.layers[run[i + 1].layer].parts().get("mixer_norm") if i + 1 < len(run) else self.final_norm
+            # may this block hand on two pending outputs? Only if the norm that takes them next (the
+            # next block's first norm, as that block's arrangement names it, or the final norm) can
+            if i + 1 < len(run):
+                first_norm = getattr(self.layers[run[i + 1].layer], "first_norm", None)
+                nxt = first_norm() if first_norm is not None else None
+            else:
+                nxt = self.final_norm
             ctx.next_norm_accepts_pending = bool(getattr(nxt, "accepts_pending", False))
             delta = self.layers[entry.layer].forward(resid, delta, ctx, caches[i])
         if ctx.num_logit_rows == 0:

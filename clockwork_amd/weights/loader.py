@@ -98,6 +98,8 @@ def load_parameters(
         shapes = [transformed_shape(target.transform, shape) for shape in target.source_shapes]
         rows = sum(shape[0] for shape in shapes)
         full_shape = (rows, *shapes[0][1:])
+        if any(shape[1:] != shapes[0][1:] for shape in shapes):
+            raise RuntimeError(f"weight plan for {target.param} stacks sources whose rows differ: {shapes}")
         if tuple(spec.shape) != full_shape:
             raise RuntimeError(
                 f"weight plan for {target.param} yields {full_shape}, the part declares {spec.shape}"

@@ -359,3 +359,66 @@ def test_pages_that_fit_follows_the_reference_arithmetic_and_its_caps():
     assert page_bytes(two, 4, torch.float32) == 3 * 2 * 4 * 2 * 16 * 4
     # a model without paged state needs no pages
     assert pages_that_fit(plan_groups([StateSpec((4,), "float32")]), 16, torch.float32, 10, 1.0, most=5) == 1
+
+
+# ------------------------------------------------------------------ pages of a mixer's own rows
+def test_a_mixer_may_keep_planes_of_its_own_in_pages():
+    """Keys and values of one shape are one case; a mixer may cache one latent vector a token
+    and no values, or planes of different widths. The manager pages them all alike, the pools
+    size every plane from the spec."""
+    import torch
+
+    from clockwork_amd.cache.pools import CachePools, page_bytes
+    from clockwork_amd.config.spec import PagedRowsSpec
+
+    latent = PagedRowsSpec((("latent", (24,)),))
+    uneven = PagedRowsSpec((("k", (2, 16)), ("v", (2, 8))), window=8)
+    assert KVPagesSpec(2, 16).planes == (("k", (2, 16)), ("v", (2, 16)))
+    assert latent.group_key() != PagedRowsSpec((("latent", (32,)),)).group_key()
+    with pytest.raises(ValueError, match="names of their own"):
+        PagedRowsSpec((("a", (4,)), ("a", (4,))))
+    with pytest.raises(ValueError, match="row shape"):
+        PagedRowsSpec((("a", ()),))
+    groups = plan_groups([latent, KVPagesSpec(2, 16), latent, uneven, StateSpec((4,), "float32")])
+    assert [(g.is_kv, g.window, g.entries) for g in groups] == [
+        (True, None, (0, 2)), (True, None, (1,)), (True, 8, (3,)), (False, None, (4,))]
+    # a page number costs: two entries of 24, one of 2 x 2 x 16, one of 2 x 16 + 2 x 8, times the page's tokens
+    assert page_bytes(groups, 4, torch.float32) == 4 * 4 * (2 * 24 + 64 + 48)
+    m = CacheManager(groups, block_size=4, num_blocks=6, max_num_seqs=2)
+    m.admit("a", 9)
+    assert [len(m.block_table("a", g)) for g in range(3)] == [3, 3, 3]
+    m.free("a")
+    assert all(p.num_free == 6 for p in m.pools)
+
+    pools = CachePools(groups, 4, 6, 2, torch.float32, "cpu", fill=7.0)
+    assert tuple(pools.kv[0].shape) == (2, 1, 6, 4, 24) and tuple(pools.kv[1].shape) == (1, 2, 6, 4, 2, 16)
+    assert pools.kv[2] is None   # planes of different shapes have a tensor each
+    assert {n: tuple(t.shape) for n, t in pools.planes[2].items()} == {"k": (1, 6, 4, 2, 16), "v": (1, 6, 4, 2, 8)}
+    assert pools.kv_bytes_per_token() == 4 * (2 * 24 + 64 + 48)
+    assert pools.bytes() == 6 * 4 * pools.kv_bytes_per_token() + 4 * 4 * 4
+    cache = pools.entry_cache(2)     # the second entry of the latent group
+    assert cache.group == 0 and cache.k is None and cache.v is None and tuple(cache.planes["latent"].shape) == (24, 24)
+    cache.planes["latent"][5] = 1.0  # a view of the pool: page 1, token 1 of entry row 1
+    assert float(pools.kv[0][1, 0, 1, 1].sum()) == 24.0 and float(pools.kv[0][0].sum()) == 7.0 * 6 * 4 * 24
+    kv = pools.entry_cache(1)
+    assert tuple(kv.k.shape) == tuple(kv.v.shape) == (24, 2, 16) and kv.planes["k"] is kv.k
+    odd = pools.entry_cache(3)
+    assert tuple(odd.k.shape) == (24, 2, 16) and tuple(odd.v.shape) == (24, 2, 8) and odd.block_size == 4
+
+
+def test_a_fresh_state_is_what_the_spec_says():
+    import torch
+
+    from clockwork_amd.cache.pools import CachePools
+
+    with pytest.raises(ValueError, match="fresh state"):
+        StateSpec((4,), "float32", init=("ones",))
+    filled, zeros = StateSpec((4,), "float32", init=("fill", 0.5)), StateSpec((4,), "float32")
+    assert filled.group_key() != zeros.group_key()   # other beginnings, other pools
+    groups = plan_groups([filled, zeros, filled])
+    pools = CachePools(groups, 4, 2, 3, torch.float32, "cpu")
+    # three slots for requests, the spare one, the template
+    assert tuple(pools.state[0].shape) == (2, 5, 4) and tuple(pools.state[1].shape) == (1, 5, 4)
+    assert bool((pools.state[0] == 0.5).all()) and bool((pools.state[1] == 0).all())
+    pools.set_fresh_state(2, torch.arange(4.0))
+    assert pools.state[0][1, 4].tolist() == [0.0, 1.0, 2.0, 3.0] and pools.state[0][0, 4].tolist() == [0.5] * 4

@@ -1322,3 +1322,30 @@ def test_sampling_is_reproducible_and_follows_the_distribution():
     assert not torch.equal(a, c)
     freq = torch.bincount(a.long(), minlength=V).float() / n
     torch.testing.assert_close(freq.cpu(), torch.softmax(row, -1).cpu(), rtol=0, atol=0.03)
+
+
+def test_fresh_state_rows_copies_the_template_into_the_slots_of_requests_that_begin():
+    """pool [entries, slots, row]: the last slot is the template; a request whose step starts at
+    position 0 gets it, every other row of the pool stays as it is."""
+    from clockwork_amd import ops
+
+    entries, slots, width = 3, 7, 10            # 5 request slots, the spare one, the template
+    pool = torch.randn(entries, slots, width, device=DEV)
+    before = pool.clone()
+    rows = torch.tensor([4, 1, -1, 9, 5, 2, 6], dtype=torch.int32, device=DEV)     # -1 / 9: no request; 5: the spare slot
+    starts = torch.tensor([0, 3, 0, 0, 0, 0, 0], dtype=torch.int32, device=DEV)    # slot 1 is in the middle of its request
+    ops.fresh_state_rows(pool, rows, starts, 6)                                    # the seventh row is not part of the step
+    torch.cuda.synchronize()
+    want = before.clone()
+    for slot in (4, 5, 2):
+        want[:, slot] = before[:, 6]
+    assert torch.equal(pool, want)   # slot 6 itself (the template) is never a target
+    # half precision rows of an even width are whole words too
+    half = torch.randn(2, 4, 6, device=DEV).to(torch.bfloat16)
+    kept = half.clone()
+    ops.fresh_state_rows(half, torch.tensor([0], dtype=torch.int32, device=DEV), torch.tensor([0], dtype=torch.int32, device=DEV), 1)
+    torch.cuda.synchronize()
+    kept[:, 0] = kept[:, 3]
+    assert torch.equal(half, kept)
+    with pytest.raises(ops.KernelError):
+        ops.fresh_state_rows(pool[:, :1], rows, starts, 1)   # no room for a template

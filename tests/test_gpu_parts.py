@@ -11,7 +11,7 @@ from dataclasses import dataclass
 import pytest
 import torch
 
-from clockwork_amd.config.spec import LayerSpec, ModelSpec, ParamSpec, RunEntry, StateSpec, WeightTarget
+from clockwork_amd.config.spec import LayerSpec, ModelSpec, PagedRowsSpec, ParamSpec, RunEntry, StateSpec, WeightTarget
 from clockwork_amd.parts.specs import AttentionSpec, RMSNormSpec, RopeNeoxSpec, SwiGLUSpec
 from clockwork_amd.registry import Architecture, build_part, register_architecture, register_part
 from tests import replay
@@ -619,6 +619,279 @@ def test_a_second_toy_with_its_own_embedding_head_and_block(toy2_dir, dtype, mod
     assert not runner.manager.live_requests()
     # slots come back, and a slot that another request used is cleared for the next one
     assert len(runner.manager._free_slots) == runner.manager.max_num_seqs
+
+
+# ---------------------------------------------------------------------------------- a third toy
+# What the first two leave to the framework's defaults: a mixer that pages rows of its own (one
+# 24-wide latent a token, no values), checkpoint tensors that are stored transposed and fused,
+# positions that the embedding part decides, a block whose parts have other names, a state that
+# does not begin at zero.
+@dataclass(frozen=True)
+class OffsetEmbeddingSpec:
+    """A table lookup whose tokens count their positions from ``offset``, not from 0."""
+
+    vocab_size: int
+    hidden_size: int
+    offset: int
+
+
+class OffsetEmbedding:
+    def __init__(self, spec):
+        self.spec = spec
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.spec.vocab_size, self.spec.hidden_size))}
+
+    def bind(self, params, device, dtype):
+        self.weight = params["weight"]
+
+    def table(self):
+        return self.weight
+
+    def positions(self, ctx):
+        return ctx.sequence_positions + self.spec.offset
+
+    def forward(self, ctx):
+        return self.weight[ctx.token_ids.long()].float()
+
+
+@dataclass(frozen=True)
+class LatentMixerSpec:
+    """c_t = x_t Wc^T + 0.3 sin(pos_t / (j + 1)) is cached, 24 wide, one row a token; a token
+    attends over the latents up to its own: y_t = softmax_s(scale (x_t Wq^T) . c_s) c_s Wo^T."""
+
+    hidden_size: int
+    latent: int
+    scale: float
+
+
+class LatentMixer:
+    def __init__(self, spec):
+        self.spec = spec
+
+    def param_specs(self):
+        s = self.spec
+        return {"w_c": ParamSpec((s.latent, s.hidden_size), init=("normal", 0.2)),
+                "w_q": ParamSpec((s.latent, s.hidden_size), init=("normal", 0.2)),
+                "w_o": ParamSpec((s.hidden_size, s.latent), init=("normal", 0.1))}
+
+    def cache_need(self):
+        return PagedRowsSpec((("latent", (self.spec.latent,)),))
+
+    def bind(self, params, device, dtype):
+        self.w_c, self.w_q, self.w_o = (params[k].float() for k in ("w_c", "w_q", "w_o"))
+
+    def forward(self, x, ctx, cache):
+        xf = x.float()
+        j = torch.arange(self.spec.latent, device=x.device, dtype=torch.float32)
+        c = xf @ self.w_c.t() + 0.3 * torch.sin(ctx.positions.float()[:, None] / (j + 1.0))
+        pages = cache.planes["latent"]                     # [pages * page size, latent]
+        slots = ctx.slots[cache.group]
+        keep = slots >= 0
+        pages[slots[keep].long()] = c[keep].to(pages.dtype)
+        q = xf @ self.w_q.t()
+        out = torch.empty_like(q)
+        at = 0
+        for r, n in enumerate(ctx.h_q_lens):
+            have, start = ctx.h_ctx_lens[r], ctx.h_starts[r]
+            at_token = torch.arange(have, device=x.device)
+            table = ctx.block_tables[cache.group][r].long()
+            rows = table[at_token // cache.block_size] * cache.block_size + at_token % cache.block_size
+            latents = pages[rows].float()                  # what the request has cached, through its block table
+            scores = self.spec.scale * q[at : at + n] @ latents.t()
+            seen = at_token[None, :] <= (start + torch.arange(n, device=x.device))[:, None]
+            out[at : at + n] = torch.softmax(scores.masked_fill(~seen, float("-inf")), dim=-1) @ latents
+            at += n
+        return (out @ self.w_o.t()).to(x.dtype)
+
+
+@dataclass(frozen=True)
+class WarmDecayMixerSpec:
+    """DecayMixer's recurrence, begun at s = ``begin`` in every element instead of at zero."""
+
+    hidden_size: int
+    decay: float
+    begin: float
+
+
+class WarmDecayMixer(DecayMixer):
+    graph_safe = False
+
+    def cache_need(self):
+        return StateSpec((self.spec.hidden_size,), "float32", init=("fill", self.spec.begin))
+
+
+class RenamedBlock:
+    """The pre-norm wiring under names of its own: nothing in it is called ``mixer_norm``."""
+
+    def __init__(self, mixer, feed_forward, norm_a, norm_b):
+        self.mixer, self.feed_forward, self.norm_a, self.norm_b = mixer, feed_forward, norm_a, norm_b
+
+    def parts(self):
+        return {"mixer": self.mixer, "feed_forward": self.feed_forward, "norm_a": self.norm_a, "norm_b": self.norm_b}
+
+    def first_norm(self):
+        return self.norm_a
+
+    def forward(self, resid, delta, ctx, cache):
+        a = self.mixer.forward(self.norm_a.forward(resid, delta), ctx, cache)
+        return self.feed_forward.forward(self.norm_b.forward(resid, a), ctx)
+
+
+@dataclass(frozen=True)
+class Toy3Config:
+    vocab: int
+    hidden: int
+    latent: int
+    offset: int
+    begin: float
+    eps: float
+
+
+def _toy3_spec(cfg: Toy3Config) -> ModelSpec:
+    norm = RMSNormSpec(cfg.hidden, cfg.eps)
+    ffn = SwiGLUSpec(cfg.hidden, 2 * cfg.hidden)
+    norms = (("norm_a", norm), ("norm_b", norm))
+    layers = [
+        LayerSpec("renamed", mixer=LatentMixerSpec(cfg.hidden, cfg.latent, 0.1), feed_forward=ffn, extra=norms),
+        LayerSpec("renamed", mixer=WarmDecayMixerSpec(cfg.hidden, 0.7, cfg.begin), feed_forward=ffn, extra=norms),
+    ]
+    return ModelSpec("Toy3ForCausalLM", cfg.vocab, cfg.hidden, layers, [RunEntry(0), RunEntry(1), RunEntry(0)], norm,
+                     tie_embeddings=True, embedding=OffsetEmbeddingSpec(cfg.vocab, cfg.hidden, cfg.offset))
+
+
+def _toy3_plan(cfg: Toy3Config, spec: ModelSpec):
+    """The latent mixer's checkpoint holds Wc and Wq as one tensor [2 latent, hidden] and Wo the
+    other way round, [latent, hidden]; everything else under the model's own names."""
+    plan = []
+    for target in _toy_plan(cfg, spec):
+        if target.param.endswith(".mixer.w_c"):
+            fused = target.param[:-3] + "cq"
+            plan.append(WeightTarget(target.param, (fused,), ((2 * cfg.latent, cfg.hidden),), transform=("split_rows", 0, 2)))
+        elif target.param.endswith(".mixer.w_q"):
+            fused = target.param[:-3] + "cq"
+            plan.append(WeightTarget(target.param, (fused,), ((2 * cfg.latent, cfg.hidden),), transform=("split_rows", 1, 2)))
+        elif target.param.endswith(".mixer.w_o"):
+            plan.append(WeightTarget(target.param, (target.param + "_t",), ((cfg.latent, cfg.hidden),), transform=("transpose",)))
+        else:
+            plan.append(target)
+    return plan
+
+
+@pytest.fixture(scope="module")
+def toy3_dir(tmp_path_factory):
+    from clockwork_amd.registry import register_arrangement
+    from clockwork_amd.weights.random_init import write_random_model
+
+    register_part(OffsetEmbeddingSpec, OffsetEmbedding)
+    register_part(LatentMixerSpec, LatentMixer)
+    register_part(WarmDecayMixerSpec, WarmDecayMixer)
+    register_arrangement("renamed", RenamedBlock)
+    register_architecture(
+        ["Toy3ForCausalLM"],
+        Architecture(
+            "Toy3ForCausalLM",
+            parse_config=lambda d: Toy3Config(d["vocab"], d["hidden"], d["latent"], d["offset"], d["begin"], d["eps"]),
+            build_spec=_toy3_spec,
+            weight_plan=_toy3_plan,
+        ),
+    )
+    config = {"architectures": ["Toy3ForCausalLM"], "vocab": 190, "hidden": 48, "latent": 24, "offset": 11, "begin": 0.5,
+              "eps": 1e-5}
+    return write_random_model(tmp_path_factory.mktemp("toy3") / "toy3", config, seed=21)
+
+
+def _toy3_plain_logits(model_dir, tokens, offset=None):
+    from safetensors.torch import load_file
+
+    cfg = json.loads((model_dir / "config.json").read_text())
+    w = {k: v.float() for k, v in load_file(str(model_dir / "model.safetensors")).items()}
+    # the checkpoint's own layout: the fused and the transposed tensors, no model-side names
+    assert tuple(w["layers.0.mixer.cq"].shape) == (48, 48) and tuple(w["layers.0.mixer.w_o_t"].shape) == (24, 48)
+    assert not any(k.endswith(("mixer.w_c", "mixer.w_q", "mixer.w_o")) for k in w)
+    T, H, L = len(tokens), cfg["hidden"], cfg["latent"]
+    pos = torch.arange(T).float() + (cfg["offset"] if offset is None else offset)
+    h = plain.embedding(w["embed.weight"], torch.tensor(tokens))
+    for layer in (0, 1, 0):
+        p = f"layers.{layer}."
+        x = plain.rmsnorm(h, w[p + "norm_a.weight"], cfg["eps"])
+        if layer == 0:
+            wc, wq = w[p + "mixer.cq"][:L], w[p + "mixer.cq"][L:]
+            c = x @ wc.t() + 0.3 * torch.sin(pos[:, None] / (torch.arange(L).float() + 1.0))
+            scores = 0.1 * (x @ wq.t()) @ c.t()
+            scores = scores.masked_fill(torch.ones(T, T).triu(1).bool(), float("-inf"))
+            a = torch.softmax(scores, dim=-1) @ c @ w[p + "mixer.w_o_t"]   # Wo^T as stored
+        else:
+            s, rows = torch.full((H,), cfg["begin"]), []
+            for t in range(T):
+                s = 0.7 * s + x[t]
+                rows.append(s)
+            a = torch.stack(rows) @ w[p + "mixer.weight"].t()
+        h = h + a
+        x = plain.rmsnorm(h, w[p + "norm_b.weight"], cfg["eps"])
+        gu = w[p + "feed_forward.gate_up_weight"]
+        h = h + plain.swiglu(x, gu[: 2 * H], gu[2 * H :], w[p + "feed_forward.down_weight"])
+    return plain.linear(plain.rmsnorm(h, w["final_norm.weight"], cfg["eps"]), w["embed.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["whole", "prefill_then_decode", "portions", "mixed"])
+def test_a_third_toy_pages_latents_and_loads_transposed_and_fused_tensors(toy3_dir, dtype, mode):
+    """One latent row a token in pages (no value plane), a layer run twice with a page pool entry
+    each, weights that the checkpoint holds fused and transposed, positions that begin at 11
+    because the embedding part says so, a state that begins at 0.5, a block without a
+    ``mixer_norm``: registered from this file, no framework file knows of any of it."""
+    gen = torch.Generator().manual_seed(9)
+    requests = {f"v{i}": torch.randint(0, 190, (n,), generator=gen).tolist() for i, n in enumerate([50, 9, 77, 1, 64])}
+    runner = replay.make_runner(toy3_dir, dtype, 8, 40)
+    assert [(g.is_kv, g.entries) for g in runner.manager.groups] == [(True, (0, 2)), (False, (1,))]
+    assert tuple(runner.pools.kv[0].shape) == (2, 1, 40, 8, 24)
+    # the loader has split the fused tensor and turned the transposed one round
+    assert tuple(runner.model.params["layers.0.mixer.w_o"].shape) == (48, 24)
+    got = replay.run_trace(runner, getattr(replay, mode)(requests))
+    ref = {rid: _toy3_plain_logits(toy3_dir, toks) for rid, toks in requests.items()}
+    if dtype == "float32":
+        replay.compare(got, ref, rtol=1e-5, atol=1e-5)
+        # the offset and the warm state are not idle: without either the logits are others
+        first = next(iter(requests))
+        for other in (_toy3_plain_logits(toy3_dir, requests[first], offset=0),):
+            assert not torch.allclose(other, ref[first], rtol=1e-3, atol=1e-3)
+    else:
+        replay.compare_to_scale(got, ref)
+    assert not runner.manager.live_requests()
+    assert [p.num_free for p in runner.manager.pools] == [40]
+
+
+def test_random_traces_of_the_third_toy_fork_and_copy_latent_pages(toy3_dir):
+    """Random traces with forks (shared pages of latents copied on the first write, the warm state
+    copied at the fork) on pools that hold little more than four requests."""
+    for seed in range(8):
+        steps, seqs = replay.random_trace(seed, 190, kinds=("fork",))
+        block_size = (4, 8, 16)[seed % 3]
+        longest = sorted((-(-len(t) // block_size) for t in seqs.values()), reverse=True)[:4]
+        runner = replay.make_runner(toy3_dir, "float32", block_size, sum(longest) + len(seqs) + 2, max_model_len=1024)
+        got = replay.run_trace(runner, steps)
+        ref = {rid: _toy3_plain_logits(toy3_dir, toks) for rid, toks in seqs.items()}
+        replay.compare(got, ref, rtol=1e-5, atol=1e-5)
+        assert not runner.manager.live_requests()
+        assert all(p.num_free == runner.manager.num_blocks for p in runner.manager.pools)
+
+
+def test_pages_of_planes_with_different_widths_are_copied_plane_by_plane():
+    from clockwork_amd.cache import plan_groups
+    from clockwork_amd.cache.pools import CachePools
+
+    groups = plan_groups([PagedRowsSpec((("k", (2, 16)), ("v", (2, 8)))), PagedRowsSpec((("k", (2, 16)), ("v", (2, 8))))])
+    pools = CachePools(groups, 4, 6, 2, torch.bfloat16, torch.device(DEV))
+    for t in pools.planes[0].values():
+        t.copy_(torch.randn(t.shape))
+    before = {n: t.clone() for n, t in pools.planes[0].items()}
+    pools.copy_pages(0, [(1, 4), (2, 0)])
+    torch.cuda.synchronize()
+    for name, t in pools.planes[0].items():
+        want = before[name].clone()
+        want[:, 4], want[:, 0] = before[name][:, 1], before[name][:, 2]
+        assert torch.equal(t, want), name
 
 
 def test_windowed_group_uses_few_pages_for_a_long_request(toy_dir):

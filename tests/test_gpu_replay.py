@@ -344,7 +344,7 @@ def test_the_whole_benchmark_model(benchmark_model, mode, dtype):
     every way of cutting the work, against the plain implementation in float64 on the CPU.
     float32: the 1e-5 bar and the same arg-max at every position. bfloat16: the rounding of 28
     layers adds up to about 2% of the logits' scale (root mean square; bound 4%, the largest of 25
-    million within 25%), and wherever the arg-max differs the plain logits of the two tokens lie
+    million within 15%: 12% was measured), and wherever the arg-max differs the plain logits of the two tokens lie
     closer than a tenth of the scale (random weights give many near-ties)."""
     model_dir, requests, want = benchmark_model
     live = 3 if mode == "mixed" else 1
@@ -363,7 +363,7 @@ def test_the_whole_benchmark_model(benchmark_model, mode, dtype):
         assert not gaps
         print(f"whole model float32 {mode}: largest error {worst:.3e}")
     else:
-        scale, rms, worst = replay.compare_to_scale(got, want, rms_bound=4e-2, worst_bound=2.5e-1)
+        scale, rms, worst = replay.compare_to_scale(got, want, rms_bound=4e-2, worst_bound=1.5e-1)
         print(f"whole model bfloat16 {mode}: scale {scale:.3f}, rms {rms:.3e}, largest {worst:.3e}, arg-max differs at {len(gaps)} of 165")
         assert all(g < 1e-1 * scale for g in gaps) and len(gaps) < 30
 
@@ -619,7 +619,9 @@ def test_graph_replays_equal_eager_steps(model_dirs, dtype, graph_limit, monkeyp
     # the graph plans its attention splits for a padded batch and a context bucket, so sums may be
     # taken in another order than in the eager step: equal up to that rounding, far inside the
     # bar that both must meet against the plain implementation
-    close = dict(rtol=2e-6, atol=2e-6) if dtype == "float32" else dict(rtol=1e-2, atol=1e-2)
+    # (bfloat16: within 3% of the logits' own scale, whatever that scale is)
+    scale = torch.stack(list(got_e.values())).square().mean().sqrt().item()
+    close = dict(rtol=2e-6, atol=2e-6) if dtype == "float32" else dict(rtol=0.0, atol=3e-2 * scale)
     for key in got_e:
         torch.testing.assert_close(got_g[key], got_e[key], **close, msg=lambda m: f"graph replay differs from the eager step at {key}: {m}")
     model = PlainQwen2(model_dirs[name])

@@ -164,3 +164,49 @@ def test_several_files_are_merged_and_an_empty_folder_is_an_error(tmp_path):
     empty.mkdir()
     with pytest.raises(FileNotFoundError, match="no .safetensors files"):
         _load(empty, TINY_A)
+
+
+def test_a_checkpoint_tensor_may_be_transposed_or_split_on_its_way_in(tmp_path):
+    """A parameter's sources go through the target's ``transform`` before they are stacked: a
+    matrix the file holds the other way round, a slice of a tensor that holds several
+    projections, or both; an architecture may register steps of its own."""
+    from clockwork_amd.config.spec import ParamSpec, WeightTarget
+    from clockwork_amd.weights.transforms import apply_transform, register_transform, steps_of, transformed_shape
+
+    stored = {"down_t": torch.arange(24.0).reshape(4, 6), "qkv": torch.arange(36.0).reshape(9, 4),
+              "a": torch.arange(8.0).reshape(2, 4), "b_t": torch.full((4, 3), 2.0)}
+    save_file({k: v.to(torch.bfloat16) for k, v in stored.items()}, str(tmp_path / "model.safetensors"))
+    specs = {"down": ParamSpec((6, 4)), "k": ParamSpec((3, 4)), "v_t": ParamSpec((4, 3)), "ab": ParamSpec((5, 4)),
+             "reversed": ParamSpec((2, 4))}
+    plan = [
+        WeightTarget("down", ("down_t",), ((4, 6),), transform=("transpose",)),
+        WeightTarget("k", ("qkv",), ((9, 4),), transform=("split_rows", 1, 3)),
+        WeightTarget("v_t", ("qkv",), ((9, 4),), transform=(("split_rows", 2, 3), ("transpose",))),
+        WeightTarget("reversed", ("a",), ((2, 4),), transform=("flip_rows",)),
+    ]
+    assert transformed_shape(("transpose",), (4, 6)) == (6, 4) and steps_of(("transpose",)) == (("transpose",),)
+    assert transformed_shape((("split_rows", 2, 3), ("transpose",)), (9, 4)) == (4, 3)
+    del specs["ab"]
+    with pytest.raises(KeyError, match="no weight transform is registered under 'flip_rows'"):
+        load_parameters(tmp_path, plan + [WeightTarget("ab", ("b_t",), ((4, 3),), optional=True)], specs, torch.float32, "cpu")
+    register_transform("flip_rows", lambda t: t.flip(0))   # an architecture's own step
+    # the steps apply to every source, then the sources are stacked; sources that do not stack
+    # afterwards are a fault of the plan, said as such
+    unstackable = WeightTarget("ab", ("a", "b_t"), ((2, 4), (4, 3)), transform=("transpose",))
+    with pytest.raises(RuntimeError, match="weight plan for ab stacks sources whose rows differ"):
+        load_parameters(tmp_path, plan + [unstackable], dict(specs, ab=ParamSpec((7, 2))), torch.float32, "cpu")
+    params = load_parameters(tmp_path, plan + [WeightTarget("ab", ("b_t",), ((4, 3),), optional=True)],
+                             dict(specs, ab=ParamSpec((4, 3))), torch.float32, "cpu")
+    assert torch.equal(params["reversed"], stored["a"].flip(0)) and torch.equal(params["ab"], stored["b_t"])
+    assert torch.equal(params["down"], stored["down_t"].t())
+    assert torch.equal(params["k"], stored["qkv"][3:6]) and torch.equal(params["v_t"], stored["qkv"][6:9].t())
+    assert params["down"].is_contiguous() and params["v_t"].is_contiguous()
+    with pytest.raises(KeyError, match="no weight transform is registered under 'rotate'"):
+        apply_transform(("rotate",), stored["a"])
+    with pytest.raises(ValueError, match="does not divide"):
+        apply_transform(("split_rows", 0, 2), stored["qkv"])
+    # a shape that differs from the file's is still named, in the file's terms
+    bad = [WeightTarget("down", ("down_t",), ((6, 4),), transform=("transpose",))]
+    with pytest.raises(WeightMismatchError) as err:
+        load_parameters(tmp_path, bad, {"down": ParamSpec((4, 6))}, torch.float32, "cpu")
+    assert "down_t: checkpoint (4, 6), model (6, 4)" in str(err.value)
