@@ -26,6 +26,8 @@ class Sampler:
     # pinned buffers the rows' options travel through, used in turn: a step's copy may still be
     # under way when the next step's options are written
     _RING = 4
+    # batches whose packed options are kept
+    _KEPT = 64
 
     def __init__(self, device, default_seed: int = 0) -> None:
         self.device = device
@@ -61,9 +63,13 @@ class Sampler:
             return None
         if logits.shape[0] != n:
             raise ValueError(f"{logits.shape[0]} logits rows for {n} sequences")
-        # (the entry keeps the sequences, so an id in a key cannot come to mean another object)
-        key = tuple(id(s) for s in seqs)
+        # the options of a batch that comes again step after step are packed once: kept under the
+        # requests' ids (the entry holds the sequences themselves, and serves only them: an id that
+        # has come to mean another request finds nothing), the least recently used entry goes
+        key = tuple(s.seq_id for s in seqs)
         fixed = self._fixed.get(key)
+        if fixed is not None and not all(a is b for a, b in zip(fixed[3], seqs)):
+            fixed = None
         if fixed is None:
             params = [s.sampling_params for s in seqs]
             if all(p.greedy for p in params):
@@ -78,9 +84,12 @@ class Sampler:
                 packed = np.concatenate([seeds.view(np.int32), np.zeros(2 * n, dtype=np.int32),
                                          temperature.view(np.int32), top_p.view(np.int32), top_k])
                 fixed = packed, bool((top_k > 0).any()), bool((top_p < 1.0).any()), list(seqs)
-            if len(self._fixed) > 64:
-                self._fixed.clear()
-            self._fixed[key] = fixed
+            self._fixed.pop(key, None)
+            while len(self._fixed) >= self._KEPT:
+                self._fixed.pop(next(iter(self._fixed)))
+        else:
+            self._fixed.pop(key)
+        self._fixed[key] = fixed   # the newest entry last
         packed, any_top_k, any_top_p, _ = fixed
         if packed is None:
             return ops.argmax(logits)

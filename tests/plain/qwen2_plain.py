@@ -36,6 +36,18 @@ def rope_tables(positions: torch.Tensor, head_dim: int, theta: float, dtype=torc
     return emb.cos().to(dtype), emb.sin().to(dtype)
 
 
+def reference_rope_tables(positions: torch.Tensor, head_dim: int, theta: float, dtype=torch.float32):
+    """The tables as the reference's model has them whatever ``dtype`` the rest of the arithmetic
+    runs in: the angle of a position is the float32 product pos * inv_freq (model.py:186-191;
+    at position 2000 its rounding is 1e-4 of a radian, which a model with peaked attention
+    shows in its logits), and only its cosine and sine are taken in ``dtype``. In float32 this
+    is ``rope_tables``; in float64 it measures an engine against the reference's angles with
+    everything else exact, where ``rope_tables`` would hold the engine's float32 angles against it."""
+    freqs = positions.to(torch.float32)[:, None] * inv_frequencies(head_dim, theta)[None, :]
+    emb = torch.cat((freqs, freqs), dim=-1).to(torch.float64 if dtype == torch.float64 else torch.float32)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
 def rotate_half(x: torch.Tensor) -> torch.Tensor:
     """clockwork/engine/model.py:32-35 - (-second half, first half)."""
     half = x.shape[-1] // 2
@@ -130,7 +142,7 @@ class PlainQwen2:
         """All-position logits [T, vocab] of one whole sequence (model.py:200-204, 228-233)."""
         ids = torch.as_tensor(token_ids, dtype=torch.long)
         h = embedding(self.w["model.embed_tokens.weight"], ids)
-        cos, sin = rope_tables(torch.arange(len(ids)), self.hd, self.theta, self.dtype)
+        cos, sin = reference_rope_tables(torch.arange(len(ids)), self.hd, self.theta, self.dtype)
         for i in range(self.L):
             h = self.layer(i, h, cos, sin)
         h = rmsnorm(h, self.w["model.norm.weight"], self.eps)

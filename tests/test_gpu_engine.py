@@ -249,6 +249,73 @@ def test_seeded_sampling_is_reproducible_and_seeds_differ(model_dirs):
     assert got == run(1)
 
 
+def test_the_stated_sampling_workload_token_by_token_against_the_plain_sampler(model_dirs):
+    """The tiny model B's workload as the benchmark description states it: five prompts of 1, 9,
+    40, 64 and 100 tokens, two of which share their first 32, at most 24 tokens a step, twelve
+    tokens each at temperature 0.8; seeds given for three requests, left to the engine's for two;
+    so few pages that a request is preempted and computed again. In float32 every sampled token
+    is the one the plain sampler draws (clockwork/engine/model_runner.py:134-164: logits /
+    temperature, softmax, one draw) from the plain logits of the tokens so far with the request's
+    n-th uniform number, n being the outputs it has (a preempted request draws the same numbers
+    again); draws that land within 1e-4 of an interval's edge are not judged."""
+    from tests.plain import qwen2_plain as plain_sampling
+
+    name, vocab = "B", TINY_CONFIGS["B"][0]["vocab_size"]
+    gen = torch.Generator().manual_seed(77)
+    draw = lambda n: torch.randint(0, vocab, (n,), generator=gen).tolist()
+    shared = draw(32)
+    prompts = [draw(1), draw(9), draw(40), shared + draw(32), shared + draw(68)]
+    assert [len(p) for p in prompts] == [1, 9, 40, 64, 100]
+    seeds = [21, None, 23, None, 25]
+    plain = PlainQwen2(model_dirs[name])
+
+    def run(num_blocks):
+        e = engine(model_dirs[name], dtype="float32", block_size=8, num_blocks=num_blocks, max_num_batched_tokens=24,
+                   seed=5, enable_prefix_cache=True)
+
+        def add(i):
+            e.add_request(f"s{i}", prompt_token_ids=prompts[i],
+                          sampling_params=SamplingParams(max_tokens=12, temperature=0.8, seed=seeds[i], ignore_eos=True))
+
+        for i in range(4):
+            add(i)
+        finals = {}
+        late = [4]   # the longest prompt arrives once the prompt whose beginning it shares has been computed
+        while e.has_unfinished_requests() or late:
+            if late and (e._seqs["s3"].output_token_ids if "s3" in e._seqs else True):
+                add(late.pop())
+            for out in e.step():
+                if out.finished:
+                    finals[out.request_id] = out
+        return finals, e.stats()
+
+    def judge(finals):
+        judged = 0
+        for i, (prompt, seed) in enumerate(zip(prompts, seeds)):
+            tokens = finals[f"s{i}"].token_ids
+            assert len(tokens) == 12
+            rows = plain.logits(prompt + tokens)[len(prompt) - 1 : -1]    # the logits each output token was drawn from
+            for n, token in enumerate(tokens):
+                probs = plain_sampling.sampling_probs(rows[n], 0.8)
+                want, margin = plain_sampling.draw(probs, plain_sampling.uniform01(5 if seed is None else seed, n))
+                if margin > 1e-4:
+                    judged += 1
+                    assert token == want, f"request s{i}, output {n}: sampled {token}, the plain sampler draws {want}"
+        return judged
+
+    # the same workload on ever fewer pages: roomy, then so tight that requests are preempted (the
+    # five hold 36 pages at their ends, the longest prompt alone 13)
+    preempted = hits = 0
+    for num_blocks in (64, 30, 26, 22, 18):
+        finals, stats = run(num_blocks)
+        assert judge(finals) >= 40   # of 60: near-uniform probabilities of 1e-3 leave a fifth within 1e-4 of an edge
+        preempted += stats["num_preempted_total"]
+        hits += stats["prefix_cache_hit_tokens"]
+        print(f"{num_blocks} pages: preempted {stats['num_preempted_total']}, prefix hits {stats['prefix_cache_hit_tokens']} tokens")
+    assert preempted > 0, "no pool was small enough to preempt a request"
+    assert hits >= 32
+
+
 def test_finish_rules(model_dirs):
     # tests/test_llm_engine.py:239-296
     name = "A"

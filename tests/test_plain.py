@@ -92,6 +92,15 @@ def test_rope_tables_are_float32_exact_like_the_reference():
     cos64, sin64 = plain.rope_tables(pos, 32, 1e6, torch.float64)
     assert cos.shape == (3, 32) and torch.equal(cos[:, :16], cos[:, 16:])
     assert float((cos.double() - cos64).abs().max()) < 8e-3 and float((sin.double() - sin64).abs().max()) < 8e-3
+    # the whole model's tables keep the reference's float32 angles in every precision: in float32
+    # they are these tables, in float64 the exact cosines of the same float32 angles
+    ref_cos, ref_sin = plain.reference_rope_tables(pos, 32, 1e6)
+    assert torch.equal(ref_cos, cos) and torch.equal(ref_sin, sin)
+    angles = pos.float()[:, None] * inv[None, :]
+    cos_of_f32_angles, _ = plain.reference_rope_tables(pos, 32, 1e6, torch.float64)
+    assert torch.equal(cos_of_f32_angles[:, :16], angles.double().cos())
+    assert float((cos_of_f32_angles - cos.double()).abs().max()) < 2e-7     # float32's own cosine of the same angle
+    assert float((cos_of_f32_angles - cos64).abs().max()) > 1e-5            # the angle's rounding at position 4000
 
 
 # ------------------------------------------------------------------ attention
@@ -155,6 +164,38 @@ def test_logits_are_causal_and_deterministic(tiny):
     other = toks[:11] + [(t + 1) % 1000 for t in toks[11:]]
     torch.testing.assert_close(model.logits(other)[:11], full[:11], rtol=1e-5, atol=1e-5)
     assert not torch.allclose(model.logits(other)[12], full[12], atol=1e-4)
+
+
+def test_the_models_score_scale_is_the_library_default_for_its_head_size(tmp_path, monkeypatch):
+    """clockwork/engine/model.py:73: scale = head_dim ** -0.5, head_dim being the explicit key
+    where a config has one (model.py:17-18), not hidden_size / heads. With the model's attention
+    swapped for the library routine at its *default* scale (1 / sqrt of the queries' last
+    dimension), configuration C (head_dim 48, hidden 80, 3 heads: 80 / 3 would give another
+    scale) yields the same logits."""
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests.configs import TINY_C
+
+    model = plain.PlainQwen2(write_random_model(tmp_path / "C", TINY_C, 5), dtype=torch.float64)
+    # sharper scores, so that the scale shows: with N(0, 0.02) weights every softmax is nearly flat
+    for i in range(model.L):
+        model.w[f"model.layers.{i}.self_attn.q_proj.weight"] *= 40.0
+    toks = torch.randint(0, 777, (15,), generator=torch.Generator().manual_seed(2)).tolist()
+    own = model.logits(toks)
+    scales = []
+
+    def library_attention(q, k, v, scale, window=None):
+        scales.append(scale)
+        assert q.shape[1] == k.shape[1] and window is None   # no groups in this configuration
+        out = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), is_causal=True)
+        return out.transpose(0, 1)
+
+    monkeypatch.setattr(plain, "attention_dense", library_attention)
+    torch.testing.assert_close(model.logits(toks), own, rtol=1e-9, atol=1e-9)
+    assert scales == [48 ** -0.5] * model.L
+    # the bar bites: the scale that hidden_size / heads would give moves the logits
+    model.scale = (80 / 3) ** -0.5
+    monkeypatch.undo()
+    assert not torch.allclose(model.logits(toks), own, rtol=1e-4, atol=1e-4)
 
 
 def test_shifting_all_positions_changes_nothing(tiny):
