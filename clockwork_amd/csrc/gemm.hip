@@ -206,6 +206,24 @@ CW_EXPORT int cw_gemm_f32(const float* A, int64_t lda, const float* W, const flo
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
+// How these kernels load operands. An MFMA operand wants lane l to hold row l % 16 of a tile and
+// the 8 k-values of slot l / 16: loaded that way every lane asks for 16 bytes of a row of its own,
+// 64 requests an instruction to a compute unit's load path, which takes in about 30 GB/s of such.
+// So a lane loads row l / 4, slot l % 4 instead (four neighbouring lanes cover 64 bytes of one row:
+// 16 requests an instruction), and the lanes swap what they hold afterwards, lane (r, s) taking
+// from lane 4 r + s (ds_bpermute: through the LDS unit's crossbar, no memory). Measured on the
+// 1.5B shape's gate/up product: 12.8 -> 11.7 us with 8 rows of x, 19.8 -> 17.5 us with 64.
+typedef __attribute__((ext_vector_type(4))) int cw_i32x4_t;
+__device__ __forceinline__ bf16x8_t cw_to_operand_layout(const bf16x8_t& v, int lane) {
+  const int r = lane & 15, s = lane >> 4;
+  const int from = (r * 4 + s) * 4;  // byte address of the lane that loaded what lane (r, s) multiplies
+  const cw_i32x4_t q = __builtin_bit_cast(cw_i32x4_t, v);
+  cw_i32x4_t t;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) t[d] = __builtin_amdgcn_ds_bpermute(from, q[d]);
+  return __builtin_bit_cast(bf16x8_t, t);
+}
+
 // ROWS (16, 8 or 4) is the number of weight rows a tile really holds: a narrow output with a long K
 // is cut into more, smaller tiles so that every compute unit streams a share of the matrix (the
 // unused rows of the MFMA tile are zeros). MODE 2 needs ROWS == 16.
@@ -217,29 +235,34 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
   __shared__ float red[WAVES][RT * MT * 256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, s = lane >> 4;
+  const int lr = lane >> 2, ls = lane & 3;  // the row of a tile and the slot of a k-step that this lane loads
   const int I = N / 2;  // MODE 2 only
 
-  // weight rows of this lane, one per row tile
+  // weight rows that this lane loads, one per row tile
   const bf16_t* wrow[RT];
   bool wok[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     int64_t n;
     if (MODE == 2) {
-      const int64_t i = ((int64_t)blockIdx.x * RT + rt) * 8 + (r & 7);
-      n = (r < 8) ? i : I + i;
+      const int64_t i = ((int64_t)blockIdx.x * RT + rt) * 8 + (lr & 7);
+      n = (lr < 8) ? i : I + i;
       wok[rt] = i < I;
     } else {
-      n = ((int64_t)blockIdx.x * RT + rt) * ROWS + r;
-      wok[rt] = r < ROWS && n < N;
+      n = ((int64_t)blockIdx.x * RT + rt) * ROWS + lr;
+      wok[rt] = lr < ROWS && n < N;
     }
     wrow[rt] = W + (wok[rt] ? n : 0) * K;
   }
+  // x: one tile of tokens is few bytes beside the weights and is loaded in operand layout as it is
+  // (a swap would only add to the wait before the first product); several tiles are loaded like the weights
+  constexpr bool X_SWAP = MT > 1;
+  const int xr = X_SWAP ? lr : r, xs = X_SWAP ? ls : s;
   const bf16_t* xrow[MT];
   bool xok[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + r;
+    const int m = mt * 16 + xr;
     xok[mt] = m < M;
     xrow[mt] = X + (int64_t)(xok[mt] ? m : 0) * ldx;
   }
@@ -261,22 +284,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
     bf16x8_t wf[U][RT], xf[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int k = (ks0 + u) * 32 + s * 8;
+      const int k = (ks0 + u) * 32 + ls * 8;
       const bool kok = (ks0 + u) < k_steps && k + 8 <= K;
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
         wf[u][rt] = (kok && wok[rt]) ? *reinterpret_cast<const bf16x8_t*>(wrow[rt] + k) : zero;
+      const int kx = (ks0 + u) * 32 + xs * 8;
+      const bool kxok = (ks0 + u) < k_steps && kx + 8 <= K;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
-        xf[u][mt] = (kok && xok[mt]) ? *reinterpret_cast<const bf16x8_t*>(xrow[mt] + k) : zero;
+        xf[u][mt] = (kxok && xok[mt]) ? *reinterpret_cast<const bf16x8_t*>(xrow[mt] + kx) : zero;
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
+      bf16x8_t xo[MT];
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
+      for (int mt = 0; mt < MT; ++mt) xo[mt] = X_SWAP ? cw_to_operand_layout(xf[u][mt], lane) : xf[u][mt];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const bf16x8_t wo = cw_to_operand_layout(wf[u][rt], lane);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][rt], xf[u][mt], acc[rt][mt], 0, 0, 0);
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wo, xo[mt], acc[rt][mt], 0, 0, 0);
+      }
+    }
   }
 
   // D tile of (rt, mt): lane (r, s) holds weight rows 4s..4s+3 of token r -> red[wave][tile][row][token]
@@ -358,19 +389,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
   const int r = lane & 15, s = lane >> 4;
   const int I = N / 2;  // MODE 2 only
 
-  int koff[SPW];  // the lane's 8 k-values of each step; a step outside K reads k = 0 and meets zeros in x
+  // Loads as cw_to_operand_layout describes: this lane loads row lr of a tile, slot ls of a k-step.
+  const int lr = lane >> 2, ls = lane & 3;
+  auto to_operand = [&](const bf16x8_t& v) __attribute__((always_inline)) -> bf16x8_t {
+    return cw_to_operand_layout(v, lane);
+  };
+  int koff[SPW];  // the loading lane's 8 k-values of each step; a step outside K reads k = 0 and meets zeros in x
 #pragma unroll
   for (int u = 0; u < SPW; ++u) {
-    const int k = ((blockIdx.y * WAVES + wave) * SPW + u) * 32 + s * 8;
+    const int k = ((blockIdx.y * WAVES + wave) * SPW + u) * 32 + ls * 8;
     koff[u] = k + 8 <= K ? k : 0;
   }
   auto wrow = [&](int tile) __attribute__((always_inline)) -> const bf16_t* {
     int64_t n;
     if (MODE == 2) {  // gate and up rows alternate, so that a pair lies side by side in the tile
-      const int64_t i = min((int64_t)tile * 8 + (r >> 1), (int64_t)I - 1);
-      n = (r & 1) ? I + i : i;
+      const int64_t i = min((int64_t)tile * 8 + (lr >> 1), (int64_t)I - 1);
+      n = (lr & 1) ? I + i : i;
     } else {
-      n = min((int64_t)tile * 16 + r, (int64_t)N - 1);
+      n = min((int64_t)tile * 16 + lr, (int64_t)N - 1);
     }
     return W + n * K;
   };
@@ -425,28 +461,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
 #pragma unroll
       for (int e = 0; e < 8; ++e) xf[u][0][e] = (__bf16)(wv[u][e] * (float)(__bf16)(v[u][e] * inv));
   } else {
-    // Token tile by token tile, a row's k-steps one after the other: a lane's 16 bytes of step u
-    // and of step u + 1 are halves of one 128-byte line, and asked for back to back the second
-    // finds the line in the compute unit's own cache. The loads are unconditional, from clamped
-    // addresses; what lies past M or K is zeroed afterwards. (Every workgroup pulls all of x from
-    // L2: with 64 rows that is 44 MB beside the 55 MB of a gate/up matrix, and the kernel takes
-    // both in at about 5.7 TB/s: 13 us with 8 rows, 19 us with 64.)
+    // Every workgroup pulls all of x from L2 (with 64 rows that is as many bytes as its weights),
+    // loaded like the weights, four lanes to a row's step, and swapped into operand layout. The
+    // loads are unconditional, from clamped addresses; what lies past M or K is zeroed first.
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      const bf16_t* xrow = X + (int64_t)min(mt * 16 + r, M - 1) * ldx;
+      const int m = mt * 16 + lr;
+      const bf16_t* xrow = X + (int64_t)min(m, M - 1) * ldx;
 #pragma unroll
-      for (int u = 0; u < SPW; ++u)
-        xf[u][mt] = *reinterpret_cast<const bf16x8_t*>(xrow + koff[u]);
-    }
+      for (int u = 0; u < SPW; ++u) {
+        const bool ok = ((blockIdx.y * WAVES + wave) * SPW + u) * 32 + ls * 8 + 8 <= K && m < M;
+        bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(xrow + koff[u]);
+        if (!ok) {
 #pragma unroll
-    for (int u = 0; u < SPW; ++u) {
-      const bool kok = ((blockIdx.y * WAVES + wave) * SPW + u) * 32 + s * 8 + 8 <= K;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        if (!kok || mt * 16 + r >= M) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) xf[u][mt][e] = (__bf16)0.0f;
+          for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.0f;
         }
+        xf[u][mt] = to_operand(v);
+      }
     }
   }
   // what the waves' partial tiles of ``tile`` (in red[buf]) become: summed over the waves, then
@@ -503,10 +534,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-      for (int u = 0; u < CH; ++u)
+      for (int u = 0; u < CH; ++u) {
+        const bf16x8_t wu = to_operand(w[u]);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], xf[u][mt], acc[mt], 0, 0, 0);
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu, xf[u][mt], acc[mt], 0, 0, 0);
+      }
     };
     const int stride = (int)gridDim.x;
     while (tile < n_tiles) {
@@ -538,10 +571,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
         for (int u = 0; u < CH; ++u)
           nxt[u] = *reinterpret_cast<const bf16x8_t*>((c + 1 < NC ? w_tile + koff[(c + 1) * CH + u] : w_next + koff[u]));
 #pragma unroll
-        for (int u = 0; u < CH; ++u)
+        for (int u = 0; u < CH; ++u) {
+          const bf16x8_t wu = to_operand(cur[u]);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], xf[c * CH + u][mt], acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu, xf[c * CH + u][mt], acc[mt], 0, 0, 0);
+        }
 #pragma unroll
         for (int u = 0; u < CH; ++u) cur[u] = nxt[u];
       }
@@ -806,15 +841,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_qkv_rope_bf16_kernel(
   const int head = blockIdx.x / tiles_per_head;   // 0 .. nh + 2 nkv - 1
   const int tile = blockIdx.x % tiles_per_head;
   const bool is_v = head >= nh + nkv;
-  // weight row of this lane inside the head
-  const int row_in_head = is_v ? tile * 16 + r : (r < 8 ? tile * 8 + r : half + tile * 8 + (r - 8));
+  // the weight row inside the head that this lane loads: row lr of the tile (see cw_to_operand_layout)
+  const int lr = lane >> 2, ls = lane & 3;
+  const int row_in_head = is_v ? tile * 16 + lr : (lr < 8 ? tile * 8 + lr : half + tile * 8 + (lr - 8));
   const bf16_t* wrow = W + ((int64_t)head * hd + row_in_head) * K;
+  constexpr bool X_SWAP = MT > 1;  // one tile of tokens is loaded in operand layout as it is (see gemm_skinny_bf16_kernel)
+  const int xr = X_SWAP ? lr : r, xs = X_SWAP ? ls : s;
   bool xok[MT];
   const bf16_t* xrow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    xok[mt] = mt * 16 + r < M;
-    xrow[mt] = X + (int64_t)(xok[mt] ? mt * 16 + r : 0) * ldx;
+    xok[mt] = mt * 16 + xr < M;
+    xrow[mt] = X + (int64_t)(xok[mt] ? mt * 16 + xr : 0) * ldx;
   }
 
   auto bias_at = [&](int col) -> float {
@@ -859,17 +897,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_qkv_rope_bf16_kernel(
     bf16x8_t wf[U], xf[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int k = (ks0 + u) * 32 + s * 8;
+      const int k = (ks0 + u) * 32 + ls * 8;
       const bool kok = (ks0 + u) < k_steps && k + 8 <= K;
       wf[u] = kok ? *reinterpret_cast<const bf16x8_t*>(wrow + k) : zero;
+      const int kx = (ks0 + u) * 32 + xs * 8;
+      const bool kxok = (ks0 + u) < k_steps && kx + 8 <= K;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
-        xf[u][mt] = (kok && xok[mt]) ? *reinterpret_cast<const bf16x8_t*>(xrow[mt] + k) : zero;
+        xf[u][mt] = (kxok && xok[mt]) ? *reinterpret_cast<const bf16x8_t*>(xrow[mt] + kx) : zero;
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
+      const bf16x8_t wo = cw_to_operand_layout(wf[u], lane);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u][mt], acc[mt], 0, 0, 0);
+      for (int mt = 0; mt < MT; ++mt)
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wo, X_SWAP ? cw_to_operand_layout(xf[u][mt], lane) : xf[u][mt],
+                                                          acc[mt], 0, 0, 0);
+    }
   }
   // lane (r, s) holds tile rows 4s..4s+3 of token r: one 16-byte store, no bank hit twice
 #pragma unroll
