@@ -721,7 +721,16 @@ CW_EXPORT int cw_gemm_bf16_skinny_ksplits(int M, int N, int K) {
   if (s < for_registers) s = for_registers;
   if (s > 16) s = 16;
   while (s > 1 && K / s < 1024) --s;
-  return s < 1 ? 1 : s;
+  if (s < 1) s = 1;
+  // One split more if that is what brings the streaming kernel in (two tiles for every compute unit):
+  // it keeps x in registers and its next tile's weights in flight, which the one-tile kernel does not
+  // (the 1.5B shape's down product with the norm behind it: 13.2 us with 5 splits, 11.3 with 6).
+  int mt, spw, n_tiles;
+  dim3 grid;
+  if (s < 16 && K / (s + 1) >= 1024 && !plan_stream(3, M, N, K, s, &mt, &spw, &grid, &n_tiles) &&
+      plan_stream(3, M, N, K, s + 1, &mt, &spw, &grid, &n_tiles))
+    ++s;
+  return s;
 }
 
 // 1 if cw_gemm_bf16_skinny streams the weights once for this shape at full speed: every shape
@@ -777,10 +786,11 @@ CW_EXPORT int cw_gemm_bf16_swiglu_normed(const float* resid, const void* delta, 
 
 // y = x W^T for M <= 64 rows of bfloat16 x [M, K] (row stride ldx) and bfloat16 W [N, K].
 // mode 0: y bfloat16 [M, N]; 1: y float32 [M, N]; 2: y = silu(gate) * up, bfloat16 [M, N / 2];
-// 3: float32 partial products [cw_gemm_bf16_skinny_ksplits(M, N, K), M, N] (M <= 16).
-// K must be a multiple of 8 (16-byte rows).
+// 3: float32 partial products [splits, M, N], splits = ``k_splits`` if that is positive (up to 16
+// rows of x; what a caller has measured to be the best for the shape), else
+// cw_gemm_bf16_skinny_ksplits(M, N, K). K must be a multiple of 8 (16-byte rows).
 CW_EXPORT int cw_gemm_bf16_skinny(int mode, const void* X, int64_t ldx, const void* W, void* C,
-                                  int64_t ldc, int M, int N, int K, hipStream_t stream) {
+                                  int64_t ldc, int M, int N, int K, int k_splits, hipStream_t stream) {
   if (M < 0 || N <= 0 || K <= 0 || mode < 0 || mode > 3) return CW_ERR_ARG;
   if (M > CW_SKINNY_MAX_M) return CW_ERR_SIZE;
   if ((K & 7) || (ldx & 7) || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return CW_ERR_ARG;
@@ -792,7 +802,8 @@ CW_EXPORT int cw_gemm_bf16_skinny(int mode, const void* X, int64_t ldx, const vo
   const int rows = mode == 2 ? N / 2 : N;
   const int tiles = (rows + (mode == 2 ? 7 : 15)) / (mode == 2 ? 8 : 16);
   if (mode == 3) {
-    const int ks = cw_gemm_bf16_skinny_ksplits(M, N, K);
+    const int ks = k_splits > 0 ? k_splits : cw_gemm_bf16_skinny_ksplits(M, N, K);
+    if (ks > 16 || K / ks < 32) return CW_ERR_ARG;
     const int rc = try_stream(3, x, ldx, w, C, ldc, M, N, K, ks, stream);
     if (rc != CW_ERR_SIZE) return rc;
     if (M > 16) return CW_ERR_SIZE;

@@ -101,7 +101,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
         "gemm": {
             "cw_gemm_f32": [P, L, P, P, P, L, I, I, I, P, L, P],
             "cw_gemm_f32_workspace_floats": [I, I, I],
-            "cw_gemm_bf16_skinny": [I, P, L, P, P, L, I, I, I, P],
+            "cw_gemm_bf16_skinny": [I, P, L, P, P, L, I, I, I, I, P],
             "cw_gemm_bf16_skinny_ksplits": [I, I, I],
             "cw_gemm_bf16_skinny_fast": [I, I, I, I],
             "cw_gemm_bf16_swiglu_normed_ok": [I, I, I],
@@ -411,15 +411,22 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
         lib = _load("gemm")
         if partial_ok and out_dtype is None:
             splits = lib.cw_gemm_bf16_skinny_ksplits(M, N, K)
+            chosen = 0
+            if splits > 1 and M <= SKINNY_MAX_ROWS:
+                # a tuning start-up has timed the split counts for this shape, or does so now
+                if policy.tuning and (N, K) not in policy.k_split_choices:
+                    policy.k_split_choices[(N, K)] = _measure_k_splits(x, weight, splits)
+                chosen = policy.k_split_choices.get((N, K), 0)
+                splits = chosen or splits
             if splits > 1:
                 parts = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
-                _check(lib.cw_gemm_bf16_skinny(3, _ptr(x), K, _ptr(weight), _ptr(parts), N, M, N, K, _stream()),
+                _check(lib.cw_gemm_bf16_skinny(3, _ptr(x), K, _ptr(weight), _ptr(parts), N, M, N, K, chosen, _stream()),
                        "gemm_bf16_skinny(partial)")
                 return PartialSums(parts)
         want_f32 = out_dtype == torch.float32
         if lib.cw_gemm_bf16_skinny_fast(1 if want_f32 else 0, M, N, K):
             out = torch.empty((M, N), dtype=torch.float32 if want_f32 else torch.bfloat16, device=x.device)
-            _check(lib.cw_gemm_bf16_skinny(1 if want_f32 else 0, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, _stream()),
+            _check(lib.cw_gemm_bf16_skinny(1 if want_f32 else 0, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, 0, _stream()),
                    "gemm_bf16_skinny")
             return out
     if policy.hip_products and K % 8 == 0 and x.is_contiguous():
@@ -444,15 +451,18 @@ class ProductPolicy:
     library (about half as fast on an MI355X; for a run that must not depend on the library).
     ``swiglu_choices`` / ``product_choices``: for a weight shape that a tuning start-up has timed
     both ways, whether the wide-tile kernel was the faster one ((rows of [gate; up], K) and
-    (N, K, with bias)); shapes never timed follow the fixed rules. ``tuning``: such a start-up is
-    under way (``library_tuning``)."""
+    (N, K, with bias)); shapes never timed follow the fixed rules. ``k_split_choices``: for an
+    (N, K) whose product of few rows is summed in parts over K (a narrow output with a long K),
+    the number of parts that start-up found the fastest, the same for every step of up to 16 rows.
+    ``tuning``: such a start-up is under way (``library_tuning``)."""
 
-    __slots__ = ("hip_products", "swiglu_choices", "product_choices", "tuning")
+    __slots__ = ("hip_products", "swiglu_choices", "product_choices", "k_split_choices", "tuning")
 
     def __init__(self, hip_products: bool = False) -> None:
         self.hip_products = bool(hip_products)
         self.swiglu_choices: dict = {}
         self.product_choices: dict = {}
+        self.k_split_choices: dict = {}
         self.tuning = False
 
 
@@ -609,6 +619,32 @@ def _timed_us(fn, repeats: int = 5) -> float:
     return sorted(times)[len(times) // 2]
 
 
+def _measure_k_splits(x: torch.Tensor, weight: torch.Tensor, default: int) -> int:
+    """Into how many parts over K is the product of these few rows with ``weight`` [N, K] summed
+    the fastest, together with the norm kernel that adds the parts up? Which count lets the
+    streaming kernel in, fills the card evenly and leaves whole chunks to a wave differs from shape
+    to shape (the 7B shape's down product: 36.8 us with 5 parts, 30.9 with 7), so the candidates
+    are timed on the model's own weights, out of the caches."""
+    M, K = x.shape
+    N = weight.shape[0]
+    lib = _load("gemm")
+    resid = torch.zeros((M, N), dtype=torch.float32, device=x.device)
+    norm_weight = torch.ones(N, dtype=torch.bfloat16, device=x.device)
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+
+    def run(splits: int):
+        parts = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
+        _check(lib.cw_gemm_bf16_skinny(3, _ptr(x), K, _ptr(weight), _ptr(parts), N, M, N, K, splits, _stream()),
+               "gemm_bf16_skinny(partial)")
+        add_rmsnorm(resid, PartialSums(parts), norm_weight, 1e-6, out, write_back=False)
+
+    candidates = sorted({default, *(s for s in (2, 3, 4, 5, 6, 7, 8, 10, 12) if K // s >= 256)})
+    times = {splits: _timed_us(lambda: run(splits), repeats=7) for splits in candidates}
+    best = min(times, key=times.get)
+    # the fixed rule stays unless something is clearly faster: no flapping between equals
+    return best if times[best] < 0.97 * times[default] else default
+
+
 def _measure_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor, out: torch.Tensor) -> bool:
     """Time the two ways of a long portion's gate/up product on these operands (the library has
     just chosen its kernel for the shape): is this package's kernel at least as fast as the
@@ -696,7 +732,7 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor, policy: "ProductPolicy | None
             and _load("gemm").cw_gemm_bf16_skinny_fast(2, M, two_i, K)):
         if not (gate_up_weight.dtype == torch.bfloat16):
             raise KernelError("a bfloat16 product needs bfloat16 operands")
-        _check(_load("gemm").cw_gemm_bf16_skinny(2, _ptr(x), K, _ptr(gate_up_weight), _ptr(out), two_i // 2, M, two_i, K, _stream()),
+        _check(_load("gemm").cw_gemm_bf16_skinny(2, _ptr(x), K, _ptr(gate_up_weight), _ptr(out), two_i // 2, M, two_i, K, 0, _stream()),
                "gemm_bf16_skinny(swiglu)")
         return out
     if x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and K % 8 == 0 and x.is_contiguous():

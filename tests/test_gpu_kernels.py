@@ -1349,3 +1349,39 @@ def test_fresh_state_rows_copies_the_template_into_the_slots_of_requests_that_be
     assert torch.equal(half, kept)
     with pytest.raises(ops.KernelError):
         ops.fresh_state_rows(pool[:, :1], rows, starts, 1)   # no room for a template
+
+
+def test_the_parts_of_a_product_summed_over_k_are_as_many_as_the_engine_has_chosen():
+    """A narrow output with a long K and few rows comes back as partial sums over K. How many
+    parts is the kernel's rule, unless the engine's policy holds a count for the shape (what a
+    tuning start-up measures): every count gives the same product, and the count is the same for
+    every number of rows up to 16, so a row's sum does not depend on the rows beside it."""
+    from clockwork_amd import ops
+
+    N, K = 1536, 8960
+    gen = torch.Generator(device=DEV).manual_seed(6)
+    w = (torch.randn(N, K, device=DEV, generator=gen) / K ** 0.5).to(torch.bfloat16)
+    x = torch.randn(16, K, device=DEV, generator=gen).to(torch.bfloat16)
+    want = x.float() @ w.float().t()
+    default = ops.linear(x[:8].contiguous(), w, partial_ok=True)
+    assert isinstance(default, ops.PartialSums) and default.parts.shape[0] > 1
+    one, all_rows = ops.linear(x[:1].contiguous(), w, partial_ok=True), ops.linear(x, w, partial_ok=True)
+    assert one.parts.shape[0] == default.parts.shape[0] == all_rows.parts.shape[0]
+    for splits in (2, 3, 6, 7, 12):
+        policy = ops.ProductPolicy()
+        policy.k_split_choices[(N, K)] = splits
+        for rows in (1, 8, 16):
+            got = ops.linear(x[:rows].contiguous(), w, partial_ok=True, policy=policy)
+            assert got.parts.shape == (splits, rows, N)
+            torch.testing.assert_close(got.sum(), want[:rows], rtol=2e-2, atol=2e-2)
+        # one row alone and the same row in a batch: the same bits
+        assert torch.equal(ops.linear(x[:1].contiguous(), w, partial_ok=True, policy=policy).parts[:, 0], got.parts[:, 0])
+    # a tuning start-up measures the count once for the shape and keeps it
+    policy = ops.ProductPolicy()
+    policy.tuning = True
+    first = ops.linear(x[:8].contiguous(), w, partial_ok=True, policy=policy)
+    policy.tuning = False
+    assert (N, K) in policy.k_split_choices and not ops.DEFAULT_POLICY.k_split_choices
+    assert first.parts.shape[0] == policy.k_split_choices[(N, K)]
+    assert ops.linear(x, w, partial_ok=True, policy=policy).parts.shape[0] == first.parts.shape[0]
+    torch.testing.assert_close(first.sum(), want[:8], rtol=2e-2, atol=2e-2)
