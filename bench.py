@@ -530,6 +530,13 @@ def main() -> int:
             "frac": round(achieved / PEAK_HBM_GBS, 4),
         },
     }
+    # what the start-up's measurements chose for this model's shapes (``tune_products``)
+    products = runner.products
+    record["tuned"] = {
+        "gate_up_wide_tile": {f"{n}x{k}": bool(v) for (n, k), v in products.swiglu_choices.items()},
+        "decode_k_splits": {f"{n}x{k}": int(v) for (n, k), v in products.k_split_choices.items()},
+        "prefill_k_runs": {f"{n}x{k}": int(v) for (n, k), v in products.wide_partial_choices.items()},
+    }
     if not args.no_points:
         t = time_prefill(cfg, runner)
         flops = prefill_flops(runner.spec, runner.model, PROMPT_LEN)

@@ -273,7 +273,10 @@ CW_EXPORT int cw_gemm_bf16_tiled(int mode, const void* X, int64_t ldx, const voi
 // change places between lane rows (v_permlane16_swap) so that it stores 16 bytes and four lanes
 // 64 bytes of a row.
 //
-// MODE as above; K a multiple of 64, at least 256; both matrices below 4 GiB.
+// MODE as above; K a multiple of 64, at least 256; both matrices below 4 GiB. MODE 3: the product
+// of a narrow output with a long K (too few tiles to fill the card) summed in k_splits runs of K,
+// each run of every tile a work item of its own; the items write float32 planes of partial sums
+// [k_splits, M, N] that the next norm kernel adds up in their order.
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((address_space(3))) void lds_void_t;
@@ -300,6 +303,7 @@ struct WideArgs {
   int64_t ldc;
   int M, N, K;
   int tiles_m, tiles_n;
+  int k_splits;  // MODE 3: K is cut into this many runs, each a tile of its own with a float32 plane of partial sums
 };
 
 // Row of W that row ``rb`` of W tile ``tn`` is. MODE 2: a wave's 96 rows are 48 gate rows followed
@@ -342,13 +346,15 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
   const int wm = wave >> 1, wn = wave & 1;
   const int c = lane & 15, s = lane >> 4;
   const int M = a.M, N = a.N, K = a.K;
-  const int total = a.tiles_m * a.tiles_n;
+  const int per_split = a.tiles_m * a.tiles_n;
+  const int total = per_split * (MODE == 3 ? a.k_splits : 1);
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
   const int run = total >> 3, rest = total & 7;
   const int run_begin = xcd * run + min(xcd, rest), run_end = run_begin + run + (xcd < rest ? 1 : 0);
   // tile id -> (row tile, W tile): groups of W_GROUP_M row tiles, inside a group the row tiles
   // of one W tile next to each other
   auto tile_of = [&](int id, int* tm, int* tn) __attribute__((always_inline)) {
+    if (MODE == 3) id %= per_split;  // the runs of K one after the other, each over all tiles
     const int per_group = W_GROUP_M * a.tiles_n;
     const int group = id / per_group, within = id - group * per_group;
     const int rows = min(W_GROUP_M, a.tiles_m - group * W_GROUP_M);
@@ -365,17 +371,21 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
     const int64_t n = w_row_of<MODE>(0, wave * (W_BN / 4) + j * 16 + lrow, N);  // the same in every tile
     wo[j] = (uint32_t)((n * K + lsub * 8) * 2);
   }
-  const int k_tiles = K / W_BK;
+  const int k_run = MODE == 3 ? K / a.k_splits : K;  // elements of K that one work item sums
+  const int k_tiles = k_run / W_BK;
   __amdgpu_buffer_rsrc_t xr, wr;
   auto aim = [&](int id) __attribute__((always_inline)) {
     int tm, tn;
     tile_of(id, &tm, &tn);
+    const int64_t k0 = MODE == 3 ? (int64_t)(id / per_split) * k_run : 0;
     const int64_t x_row0 = (int64_t)tm * W_BM;
     const int64_t w_row0 = w_row_of<MODE>(tn, 0, N);
-    xr = __builtin_amdgcn_make_buffer_rsrc((void*)(a.X + x_row0 * a.ldx), 0,
-                                           (int)(uint32_t)(((M - x_row0 - 1) * a.ldx + K) * 2), 0x00020000);
-    wr = __builtin_amdgcn_make_buffer_rsrc((void*)(a.W + w_row0 * K), 0, (int)(uint32_t)((N - w_row0) * (int64_t)K * 2),
-                                           0x00020000);
+    // the descriptors begin at the run's first element of the tile's first row and end with the
+    // run's last element of the matrix's last row: rows past the end read as zeros
+    xr = __builtin_amdgcn_make_buffer_rsrc((void*)(a.X + x_row0 * a.ldx + k0), 0,
+                                           (int)(uint32_t)(((M - x_row0 - 1) * a.ldx + k_run) * 2), 0x00020000);
+    wr = __builtin_amdgcn_make_buffer_rsrc((void*)(a.W + w_row0 * K + k0), 0,
+                                           (int)(uint32_t)(((N - w_row0 - 1) * (int64_t)K + k_run) * 2), 0x00020000);
   };
   // load i of a wave's W_LOADS for stage kt: its four x blocks, then its three W blocks
   auto fetch_one = [&](int kt, int i) __attribute__((always_inline)) {
@@ -501,6 +511,30 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
       *lo = w_pack_bf16(v[0], v[1]);
       *hi = w_pack_bf16(v[2], v[3]);
     };
+    if constexpr (MODE == 3) {
+      // the lane's four neighbouring columns of a row as they are: 16 bytes of the run's plane
+      float* plane = (float*)a.C + (int64_t)(id / per_split) * M * a.ldc;
+      const bool vec_ok = !(a.ldc & 3) && !((uintptr_t)a.C & 15);
+#pragma unroll
+      for (int mi = 0; mi < 8; ++mi) {
+        const int64_t m = (int64_t)tm * W_BM + wm * 128 + mi * 16 + c;
+        if (m >= M) continue;
+#pragma unroll
+        for (int ni = 0; ni < W_NB; ++ni) {
+          const int64_t n0 = col0 + ni * 16 + 4 * s;
+          if (n0 >= N) continue;
+          float* dst = plane + m * a.ldc + n0;
+          if (n0 + 4 <= N && vec_ok) {
+            *reinterpret_cast<f32x4_t*>(dst) = acc[mi][ni];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n0 + e < N) dst[e] = acc[mi][ni][e];
+          }
+        }
+      }
+      continue;
+    }
     const bool wide_ok = !(a.ldc & 7) && !((uintptr_t)a.C & 15);
 #pragma unroll
     for (int mi = 0; mi < 8; ++mi) {
@@ -562,6 +596,12 @@ CW_EXPORT int cw_gemm_bf16_wide_tiles(int mode, int M, int N, int K, int64_t ldx
   return w_tiles(mode, M, N);
 }
 
+// 1 if the wide-tile kernel sums this product in ``k_splits`` runs of K (cw_gemm_bf16_wide_partial).
+CW_EXPORT int cw_gemm_bf16_wide_partial_ok(int M, int N, int K, int64_t ldx, int k_splits) {
+  if (k_splits < 2 || k_splits > 16 || K % (64 * k_splits) || K / k_splits < 256) return 0;
+  return cw_gemm_bf16_wide_tiles(0, M, N, K, ldx) > 0 ? 1 : 0;
+}
+
 template <int MODE>
 static int w_launch(WideArgs a, int workgroups, hipStream_t stream) {
   static bool raised = false;
@@ -575,7 +615,7 @@ static int w_launch(WideArgs a, int workgroups, hipStream_t stream) {
   const int per_tile = MODE == 2 ? W_BN / 2 : W_BN;
   a.tiles_n = (out_cols + per_tile - 1) / per_tile;
   a.tiles_m = (a.M + W_BM - 1) / W_BM;
-  const int total = a.tiles_m * a.tiles_n;
+  const int total = a.tiles_m * a.tiles_n * (MODE == 3 ? a.k_splits : 1);
   // a multiple of 8 workgroups, so that every XCD gets the same number of them
   int grid = total < workgroups ? total : workgroups;
   grid = (grid + 7) & ~7;
@@ -594,6 +634,19 @@ CW_EXPORT int cw_gemm_bf16_wide(int mode, const void* X, int64_t ldx, const void
   if (ldc < (mode == 2 ? N / 2 : N)) return CW_ERR_ARG;
   if (M == 0) return CW_OK;
   if (cw_gemm_bf16_wide_tiles(mode, M, N, K, ldx) == 0) return CW_ERR_SIZE;
-  WideArgs a{(const bf16_t*)X, ldx, (const bf16_t*)W, bias, bias_f32, C, ldc, M, N, K, 0, 0};
+  WideArgs a{(const bf16_t*)X, ldx, (const bf16_t*)W, bias, bias_f32, C, ldc, M, N, K, 0, 0, 1};
   return mode == 2 ? w_launch<2>(a, workgroups, stream) : w_launch<0>(a, workgroups, stream);
+}
+
+// parts[z] = x[:, run z of K] W[:, run z of K]^T for z < k_splits: float32 planes [k_splits, M, N]
+// (rows ldc floats apart) whose sum, taken in the order of z, is the product. For the shapes that
+// cw_gemm_bf16_wide_partial_ok takes.
+CW_EXPORT int cw_gemm_bf16_wide_partial(const void* X, int64_t ldx, const void* W, float* parts, int64_t ldc, int M,
+                                        int N, int K, int k_splits, int workgroups, hipStream_t stream) {
+  if (M < 0 || N <= 0 || K <= 0 || workgroups < 8 || !parts || ldc < N) return CW_ERR_ARG;
+  if (((uintptr_t)X & 15) || ((uintptr_t)W & 15) || ((uintptr_t)parts & 15)) return CW_ERR_ARG;
+  if (M == 0) return CW_OK;
+  if (!cw_gemm_bf16_wide_partial_ok(M, N, K, ldx, k_splits)) return CW_ERR_SIZE;
+  WideArgs a{(const bf16_t*)X, ldx, (const bf16_t*)W, nullptr, 0, parts, ldc, M, N, K, 0, 0, k_splits};
+  return w_launch<3>(a, workgroups, stream);
 }

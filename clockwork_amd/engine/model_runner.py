@@ -74,6 +74,9 @@ def require_gpu() -> torch.device:
 
 
 class ModelRunner:
+    # the step of few rows that a tuning start-up runs for all of them
+    FEW_ROWS_SAMPLE = 8
+
     def __init__(self, cfg: EngineConfig, weight_source=None, config_dict: Optional[dict] = None,
                  cache_fill: float = 0.0, use_graphs: bool = True) -> None:
         self.cfg = cfg
@@ -181,14 +184,19 @@ class ModelRunner:
     def tune_products(self, token_counts: Sequence[int]) -> list[int]:
         """Let the matrix library choose its fastest kernel for the products of steps with these
         token counts: each count runs once as a throwaway request while tuning is on. Counts the
-        hand-written narrow products serve, float32 models (no library product) and counts that
-        the cache cannot hold are skipped. Returns the counts that ran."""
+        hand-written narrow products serve (but for one step of 8 tokens, which stands for all
+        steps of few rows: the engine times its own choices for them on it, such as into how many
+        parts over K a product is summed), float32 models (no library product) and counts that the
+        cache cannot hold are skipped. Returns the counts that ran."""
         done: list[int] = []
         if self.dtype != torch.bfloat16:
             return done
         limit = min(self.cfg.model.max_model_len, self._table_width * self.manager.block_size)
-        for n in sorted({int(c) for c in token_counts}, reverse=True):
-            if n <= ops.SKINNY_MAX_ROWS or n > limit:
+        counts = {int(c) for c in token_counts}
+        if any(c <= ops.SKINNY_MAX_ROWS for c in counts):
+            counts.add(self.FEW_ROWS_SAMPLE)
+        for n in sorted(counts, reverse=True):
+            if (n <= ops.SKINNY_MAX_ROWS and n != self.FEW_ROWS_SAMPLE) or n > limit:
                 continue
             seq_id = "__tune_products__"
             if not self.manager.can_admit(n, n):

@@ -112,6 +112,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_gemm_bf16_tiled": [I, P, L, P, P, I, P, L, I, I, I, P],
             "cw_gemm_bf16_wide_tiles": [I, I, I, I, L],
             "cw_gemm_bf16_wide": [I, P, L, P, P, I, P, L, I, I, I, I, P],
+            "cw_gemm_bf16_wide_partial_ok": [I, I, I, L, I],
+            "cw_gemm_bf16_wide_partial": [P, L, P, P, L, I, I, I, I, I, P],
         },
         "sampling": {
             "cw_argmax_chunks": [I],
@@ -429,6 +431,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
             _check(lib.cw_gemm_bf16_skinny(1 if want_f32 else 0, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, 0, _stream()),
                    "gemm_bf16_skinny")
             return out
+    if partial_ok and out_dtype is None and bias is None and M >= WIDE_PRODUCT_MIN_ROWS and x.is_contiguous():
+        splits = _wide_partial_chosen(x, weight, policy)
+        if splits:
+            return linear_wide_partial(x, weight, splits)
     if policy.hip_products and K % 8 == 0 and x.is_contiguous():
         y = linear_tiled(x, weight, bias)
     elif _wide_product_chosen(x, weight, bias, policy):
@@ -454,15 +460,18 @@ class ProductPolicy:
     (N, K, with bias)); shapes never timed follow the fixed rules. ``k_split_choices``: for an
     (N, K) whose product of few rows is summed in parts over K (a narrow output with a long K),
     the number of parts that start-up found the fastest, the same for every step of up to 16 rows.
+    ``wide_partial_choices``: for an (N, K) of a long portion's product with a narrow output and a
+    long K, into how many runs of K the wide-tile kernel sums it (0: the library's product stays).
     ``tuning``: such a start-up is under way (``library_tuning``)."""
 
-    __slots__ = ("hip_products", "swiglu_choices", "product_choices", "k_split_choices", "tuning")
+    __slots__ = ("hip_products", "swiglu_choices", "product_choices", "k_split_choices", "wide_partial_choices", "tuning")
 
     def __init__(self, hip_products: bool = False) -> None:
         self.hip_products = bool(hip_products)
         self.swiglu_choices: dict = {}
         self.product_choices: dict = {}
         self.k_split_choices: dict = {}
+        self.wide_partial_choices: dict = {}
         self.tuning = False
 
 
@@ -617,6 +626,58 @@ def _timed_us(fn, repeats: int = 5) -> float:
         end.synchronize()
         times.append(begin.elapsed_time(end) * 1e3)
     return sorted(times)[len(times) // 2]
+
+
+def linear_wide_partial(x: torch.Tensor, weight: torch.Tensor, k_splits: int) -> PartialSums:
+    """x @ weight.T as ``k_splits`` float32 planes of partial sums over runs of K, through the
+    wide-tile kernel (csrc/gemm_tile.hip): for a long portion's product whose output is too narrow
+    to fill the card with whole tiles (the down product: 64 tiles of 256 x 192 for 2048 rows of the
+    1.5B shape), and whose result goes straight into ``add_rmsnorm``."""
+    _gpu(x, weight)
+    M, K = x.shape
+    N = weight.shape[0]
+    lib = _load("gemm_tile")
+    if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and weight.shape[1] == K
+            and lib.cw_gemm_bf16_wide_partial_ok(M, N, K, x.stride(0), int(k_splits))):
+        raise KernelError("the wide-tile kernel does not sum this product in parts")
+    parts = torch.empty((int(k_splits), M, N), dtype=torch.float32, device=x.device)
+    _check(lib.cw_gemm_bf16_wide_partial(_ptr(x), x.stride(0), _ptr(weight), _ptr(parts), N, M, N, K, int(k_splits),
+                                         _compute_units(x.device), _stream()), "gemm_bf16_wide_partial")
+    return PartialSums(parts)
+
+
+# a long portion's product is a candidate for the wide-tile kernel's partial sums when whole tiles
+# would leave most compute units idle and K is long enough to cut
+WIDE_PARTIAL_MAX_TILES = 128
+WIDE_PARTIAL_MIN_K = 1024
+
+
+def _wide_partial_chosen(x: torch.Tensor, weight: torch.Tensor, policy: ProductPolicy) -> int:
+    """Into how many runs of K does the wide-tile kernel sum this product of many rows (0: it
+    does not, the library's product runs)? Only what a tuning start-up has measured on these very
+    shapes: the kernel's partial sums and the norm that adds them against the library's product and
+    the norm of its bfloat16 result."""
+    M, K = x.shape
+    N = weight.shape[0]
+    key = (N, K)
+    choice = policy.wide_partial_choices.get(key)
+    if choice is None and policy.tuning:
+        lib = _load("gemm_tile")
+        tiles = lib.cw_gemm_bf16_wide_tiles(0, M, N, K, K)
+        choice = 0
+        if 0 < tiles <= WIDE_PARTIAL_MAX_TILES and K >= WIDE_PARTIAL_MIN_K:
+            resid = torch.zeros((M, N), dtype=torch.float32, device=x.device)
+            norm_weight = torch.ones(N, dtype=torch.bfloat16, device=x.device)
+            out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            best = _timed_us(lambda: add_rmsnorm(resid, _library_product(x, weight, None), norm_weight, 1e-6, out, write_back=False))
+            for splits in (2, 3, 4, 5, 6, 7, 8):
+                if not lib.cw_gemm_bf16_wide_partial_ok(M, N, K, K, splits):
+                    continue
+                t = _timed_us(lambda: add_rmsnorm(resid, linear_wide_partial(x, weight, splits), norm_weight, 1e-6, out, write_back=False))
+                if t < 0.97 * best:
+                    best, choice = t, splits
+        policy.wide_partial_choices[key] = choice
+    return int(choice or 0)
 
 
 def _measure_k_splits(x: torch.Tensor, weight: torch.Tensor, default: int) -> int:

@@ -1385,3 +1385,47 @@ def test_the_parts_of_a_product_summed_over_k_are_as_many_as_the_engine_has_chos
     assert first.parts.shape[0] == policy.k_split_choices[(N, K)]
     assert ops.linear(x, w, partial_ok=True, policy=policy).parts.shape[0] == first.parts.shape[0]
     torch.testing.assert_close(first.sum(), want[:8], rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("M,N,K,splits", [(2048, 1536, 8960, 4), (1300, 1536, 8960, 5), (1030, 200, 2560, 2), (2048, 3584, 18944, 8),
+                                          (257, 1536, 8960, 7)])
+def test_wide_tile_product_in_partial_sums_over_k(M, N, K, splits):
+    """The wide-tile kernel with K cut into runs, every run of every tile a work item that writes
+    a float32 plane of partial sums: the planes add up to the product; rows and columns that end
+    inside a tile, a width that is no multiple of 4 floats' alignment, several runs a workgroup."""
+    from clockwork_amd import ops
+
+    gen = torch.Generator(device=DEV).manual_seed(M + splits)
+    x = torch.randn(M, K, device=DEV, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV, generator=gen) / K ** 0.5).to(torch.bfloat16)
+    got = ops.linear_wide_partial(x, w, splits)
+    assert got.parts.shape == (splits, M, N) and got.parts.dtype == torch.float32
+    run = K // splits
+    for z in (0, splits - 1):
+        want = x[:, z * run : (z + 1) * run].float() @ w[:, z * run : (z + 1) * run].float().t()
+        torch.testing.assert_close(got.parts[z], want, rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(got.sum(), x.float() @ w.float().t(), rtol=1e-3, atol=2e-3)
+    # and through the norm that adds the planes up
+    resid = torch.randn(M, N, device=DEV, generator=gen)
+    before = resid.clone()
+    weight = torch.ones(N, device=DEV)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.add_rmsnorm(resid, got, weight, 1e-6, out)
+    torch.testing.assert_close(resid, before + x.float() @ w.float().t(), rtol=1e-3, atol=3e-3)
+
+
+def test_wide_tile_partial_sums_refuse_what_they_do_not_take():
+    from clockwork_amd import ops
+
+    x = torch.zeros(1024, 8960, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(1536, 8960, device=DEV, dtype=torch.bfloat16)
+    for splits in (1, 3, 6, 17):   # 8960 is no multiple of 64 * 3 or 64 * 6
+        with pytest.raises(ops.KernelError):
+            ops.linear_wide_partial(x, w, splits)
+    # the engine takes the kernel only where a tuning start-up has measured it to be the faster way
+    policy = ops.ProductPolicy()
+    assert isinstance(ops.linear(x, w, partial_ok=True, policy=policy), torch.Tensor)
+    policy.wide_partial_choices[(1536, 8960)] = 4
+    assert ops.linear(x, w, partial_ok=True, policy=policy).parts.shape == (4, 1024, 1536)
+    assert isinstance(ops.linear(x[:512], w, partial_ok=True, policy=policy), torch.Tensor)   # too few rows
+    assert isinstance(ops.linear(x, w, policy=policy), torch.Tensor)                           # a caller that wants a tensor
