@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
+import json
 import os
 import tempfile
 from ctypes import c_float, c_int, c_int64, c_void_p
@@ -466,6 +467,8 @@ class ProductPolicy:
 
     __slots__ = ("hip_products", "swiglu_choices", "product_choices", "k_split_choices", "wide_partial_choices", "tuning")
 
+    TABLES = ("swiglu_choices", "product_choices", "k_split_choices", "wide_partial_choices")
+
     def __init__(self, hip_products: bool = False) -> None:
         self.hip_products = bool(hip_products)
         self.swiglu_choices: dict = {}
@@ -473,6 +476,54 @@ class ProductPolicy:
         self.k_split_choices: dict = {}
         self.wide_partial_choices: dict = {}
         self.tuning = False
+
+    def read_choices(self, path: str) -> int:
+        """Take over what an earlier start-up on this card and kernel build measured and left in
+        ``path`` (entries this policy already holds stay). A file that is missing, unreadable or
+        from another card or build is passed over. Returns the number of entries taken."""
+        try:
+            with open(path) as f:
+                record = json.load(f)
+            if record.get("made_for") != _choices_made_for():
+                return 0
+            taken = 0
+            for name in self.TABLES:
+                table = getattr(self, name)
+                for key, value in record.get(name, []):
+                    key = tuple(key)
+                    if key not in table:
+                        table[key] = value
+                        taken += 1
+            return taken
+        except (OSError, ValueError, TypeError, AttributeError):
+            return 0
+
+    def write_choices(self, path: str) -> None:
+        """Leave this policy's measured choices in ``path`` (written beside it and moved over it,
+        so a reader never sees half a file); where the folder cannot be written nothing is kept."""
+        record = {"made_for": _choices_made_for()}
+        for name in self.TABLES:
+            record[name] = [[list(key), value] for key, value in getattr(self, name).items()]
+        try:
+            fd, tmp = tempfile.mkstemp(dir=os.path.dirname(path) or ".", prefix=".choices-")
+            with os.fdopen(fd, "w") as f:
+                json.dump(record, f)
+            os.replace(tmp, path)
+        except OSError:
+            pass
+
+
+def choices_file() -> str:
+    """Where a tuning start-up keeps what it measured for this package's own kernels: a file in
+    the temporary folder, one per user, or where CLOCKWORK_AMD_CHOICES_FILE points."""
+    return os.environ.get("CLOCKWORK_AMD_CHOICES_FILE") or os.path.join(
+        tempfile.gettempdir(), f"clockwork_amd_choices_{os.getuid()}.json")
+
+
+def _choices_made_for() -> list:
+    """What measured choices hold for: the card and the builds of the kernels that were timed."""
+    card = torch.cuda.get_device_name() if torch.cuda.is_available() else "none"
+    return [card, torch.__version__] + [build.library_path(n).name for n in ("gemm", "gemm_tile", "core")]
 
 
 # what a call without an engine behind it runs by: the library for large products, nothing timed
@@ -564,7 +615,10 @@ def library_tuning(policy: "ProductPolicy | None" = None):
     use and unseen shapes take the library's own default again. The library keeps its choices in a
     file in the temporary folder (or where PYTORCH_TUNABLEOP_FILENAME points), which later
     processes of the same user read. ``policy``: the engine whose own kernels are timed against the
-    library's meanwhile. Not to be left active during HIP-graph capture."""
+    library's meanwhile; what it measures is kept in a file beside the library's
+    (``choices_file``), so that a later process on the same card and build, a profiled run among
+    them, takes the same kernels without timing them again. Not to be left active during
+    HIP-graph capture."""
     import torch.cuda.tunable as tunable
 
     policy = policy if policy is not None else DEFAULT_POLICY
@@ -573,11 +627,13 @@ def library_tuning(policy: "ProductPolicy | None" = None):
     tunable.enable(True)
     tunable.tuning_enable(True)
     policy.tuning = True
+    policy.read_choices(choices_file())
     try:
         yield
     finally:
         policy.tuning = False
         tunable.tuning_enable(False)
+        policy.write_choices(choices_file())
 
 
 # a plain product is timed against the library's only with this many rows and tiles (half the

@@ -1,0 +1,48 @@
+"""What a tuning start-up measured for the package's own kernels is kept in a file and read again."""
+
+import json
+
+from clockwork_amd import ops
+
+
+def test_choices_written_and_read_back(tmp_path):
+    path = str(tmp_path / "choices.json")
+    first = ops.ProductPolicy()
+    first.k_split_choices[(1536, 8960)] = 6
+    first.wide_partial_choices[(1536, 8960)] = 4
+    first.swiglu_choices[(17920, 1536)] = False
+    first.product_choices[(3584, 1024, True)] = True
+    first.write_choices(path)
+
+    later = ops.ProductPolicy()
+    later.k_split_choices[(1536, 8960)] = 3          # what this process measured itself stays
+    assert later.read_choices(path) == 3
+    assert later.k_split_choices == {(1536, 8960): 3}
+    assert later.wide_partial_choices == {(1536, 8960): 4}
+    assert later.swiglu_choices == {(17920, 1536): False}
+    assert later.product_choices == {(3584, 1024, True): True}
+    assert not ops.DEFAULT_POLICY.k_split_choices
+
+
+def test_choices_of_another_build_or_a_broken_file_are_passed_over(tmp_path):
+    path = tmp_path / "choices.json"
+    policy = ops.ProductPolicy()
+    assert policy.read_choices(str(path)) == 0                      # no file
+    path.write_text("{ not json")
+    assert policy.read_choices(str(path)) == 0
+    record = {"made_for": ["another card", "0.0", "gemm-0.so", "gemm_tile-0.so", "core-0.so"],
+              "k_split_choices": [[[1536, 8960], 6]]}
+    path.write_text(json.dumps(record))
+    assert policy.read_choices(str(path)) == 0 and not policy.k_split_choices
+    record["made_for"] = ops._choices_made_for()
+    path.write_text(json.dumps(record))
+    assert policy.read_choices(str(path)) == 1 and policy.k_split_choices == {(1536, 8960): 6}
+    # a folder that cannot be written: nothing is kept, nothing is raised
+    policy.write_choices(str(tmp_path / "missing" / "choices.json"))
+
+
+def test_choices_file_follows_the_environment(monkeypatch, tmp_path):
+    monkeypatch.setenv("CLOCKWORK_AMD_CHOICES_FILE", str(tmp_path / "c.json"))
+    assert ops.choices_file() == str(tmp_path / "c.json")
+    monkeypatch.delenv("CLOCKWORK_AMD_CHOICES_FILE")
+    assert "clockwork_amd_choices_" in ops.choices_file()
