@@ -1115,21 +1115,29 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
     if (t_first + 1 <= t_last) fetch(t_first + 1, gk, gv);
     if (t_first + 2 <= t_last) fetch(t_first + 2, gk1, gv1);
     __syncthreads();
+    // The two waves of a SIMD (sets h and h + NH / 2) would walk through a round in step, both in
+    // the score product, then both in the softmax, each waiting for the unit the other holds. The
+    // later sets move their tile traffic to the start of the round (the buffer it writes was last
+    // read before the barrier), so their phases fall beside other ones of the earlier sets:
+    // 2048 tokens of 12 heads on 2 key/value heads 44.5 -> 42.6 us.
+    const bool late = half >= NH / 2;
     for (int t = t_first; t <= t_last; t += 2) {
-      compute(t, 0);
+      if (!late) compute(t, 0);
       if (t + 1 <= t_last) stash(1, gk, gv);
       if (t + 3 <= t_last) {
         window_for(t + 3);
         fetch(t + 3, gk, gv);
       }
+      if (late) compute(t, 0);
       __syncthreads();
       if (t + 1 > t_last) break;
-      compute(t + 1, 1);
+      if (!late) compute(t + 1, 1);
       if (t + 2 <= t_last) stash(0, gk1, gv1);
       if (t + 4 <= t_last) {
         window_for(t + 4);
         fetch(t + 4, gk1, gv1);
       }
+      if (late) compute(t + 1, 1);
       __syncthreads();
     }
   } else {
