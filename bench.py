@@ -422,6 +422,75 @@ def measure_peaks() -> dict:
     }
 
 
+# The reference's only kernel-level figures: its paged decode attention alone, on its own card
+# (/root/reference/docs/results.md:83-94: Tesla T4, float16, 12 query heads on 2 key/value heads,
+# head size 128, pages of 16; milliseconds by (batch, context)).
+REFERENCE_DECODE_ATTENTION_MS = {
+    (1, 128): 0.0607, (1, 512): 0.1602, (1, 2048): 0.6219, (4, 128): 0.0737, (4, 512): 0.2735, (4, 2048): 0.5802,
+    (16, 128): 0.0979, (16, 512): 0.4182, (16, 2048): 1.4058, (64, 128): 0.4079, (64, 512): 1.4359, (64, 2048): 5.3783,
+}
+
+
+def measure_decode_attention_grid() -> dict:
+    """The engine's attention part alone on batches of single tokens, over the grid of batch sizes
+    and context lengths that the reference times its decode kernel on (its method: 10 warm-up
+    calls, then 50 timed ones, /root/reference/notebooks/bench_t4.ipynb:236-250; here the 50 calls
+    are one captured graph, so the time is the kernels', the merge of the key splits included).
+    Pages lie in random order; bytes are the keys and values read."""
+    import torch
+
+    from clockwork_amd.engine.batch import StepContext
+    from clockwork_amd.parts.attention import PagedAttention
+    from clockwork_amd.parts.specs import AttentionSpec
+
+    dev = torch.device("cuda:0")
+    nh, nkv, hd, bs = 12, 2, 128, BLOCK
+    part = PagedAttention(AttentionSpec(hidden_size=nh * hd, num_heads=nh, num_kv_heads=nkv, head_dim=hd,
+                                        qkv_bias=False, out_bias=False, scale=hd ** -0.5))
+    part.dtype = torch.bfloat16
+    units = torch.cuda.get_device_properties(dev).multi_processor_count
+    grid = {}
+    for (batch, context), ref_ms in REFERENCE_DECODE_ATTENTION_MS.items():
+        pages_each = -(-context // bs)
+        pages = batch * pages_each
+        gen = torch.Generator(device="cpu").manual_seed(batch * 100003 + context)
+        k = torch.randn((pages, bs, nkv, hd), generator=gen).to(dev, torch.bfloat16)
+        v = torch.randn((pages, bs, nkv, hd), generator=gen).to(dev, torch.bfloat16)
+        q = torch.randn((batch, nh * hd), generator=gen).to(dev, torch.bfloat16)
+        ctx = StepContext()
+        ctx.device, ctx.block_size, ctx.num_compute_units = dev, bs, units
+        ctx.num_tokens = ctx.num_requests = batch
+        ctx.h_q_lens, ctx.h_ctx_lens = [1] * batch, [context] * batch
+        ctx.block_tables = [torch.randperm(pages, generator=gen).to(dev, torch.int32).view(batch, pages_each)]
+        ctx.ctx_lens = torch.full((batch,), context, dtype=torch.int32, device=dev)
+        ctx.cu_q = torch.arange(batch + 1, dtype=torch.int32, device=dev)
+        cache = argparse.Namespace(k=k, v=v, group=0, block_size=bs)
+        part.prepare(ctx)
+        for _ in range(10):
+            part.attend(q, ctx, cache)
+        _sync()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(50):
+                part.attend(q, ctx, cache)
+        graph.replay()
+        _sync()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        graph.replay()
+        end.record()
+        end.synchronize()
+        ms = begin.elapsed_time(end) / 50
+        plan = part._plan(ctx, torch.bfloat16)
+        read = 2 * batch * context * nkv * hd * 2
+        grid[f"batch{batch}_ctx{context}"] = {"ms": round(ms, 5), "reference_t4_ms": ref_ms, "key_splits": plan.decode_splits,
+                                              "GB_per_s": round(read / ms / 1e6, 1)}
+    return {"metric": "paged decode attention alone, 12 query heads on 2 key/value heads, head size 128, pages of 16",
+            "unit": "ms", "dtype": "bf16", "stat": "mean of 50 calls in one graph after 10 warm-up calls",
+            "reference": "Tesla T4, float16 (docs/results.md:83-94 of the reference): other hardware, for orientation",
+            "grid": grid}
+
+
 def prefill_flops(spec, model, T: int) -> float:
     """2 * T * (matrix parameters of the layers) + causal attention + one row of the output head."""
     layer_params = 0
@@ -457,6 +526,8 @@ def main() -> int:
     ap.add_argument("--no-prefix-cache", action="store_true", help="--workload agent: the same traffic without the prefix cache")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--peaks", action="store_true", help="measure a device copy and a large library product instead")
+    ap.add_argument("--decode-attention-grid", action="store_true",
+                    help="time the attention part alone over the reference's grid of batch sizes and context lengths instead")
     ap.add_argument("--temperature", type=float, default=0.0, help="sample instead of the greedy decoding of the recorded benchmark")
     ap.add_argument("--top-k", type=int, default=-1)
     ap.add_argument("--top-p", type=float, default=1.0)
@@ -469,6 +540,9 @@ def main() -> int:
 
     if args.peaks:
         print(json.dumps(measure_peaks()))
+        return 0
+    if args.decode_attention_grid:
+        print(json.dumps(measure_decode_attention_grid()))
         return 0
     if args.workload == "agent":
         print(json.dumps(run_agent(args)))

@@ -237,7 +237,6 @@ class PagedAttention(Part):
     def forward(self, x: torch.Tensor, ctx, cache: EntryCache) -> torch.Tensor:
         s = self.spec
         nh, nkv, hd = s.num_heads, s.num_kv_heads, s.head_dim
-        T = x.shape[0]
         policy = getattr(ctx, "products", None)
         fused = getattr(self.position, "project_rotate_store", None) if cache.writes else None
         qkv = None
@@ -255,11 +254,21 @@ class PagedAttention(Part):
             qkv = ops.linear(x, self.qkv_weight[: self.q_width], policy=policy)
             bias = self.qkv_bias[: self.q_width] if self.qkv_bias is not None else None
             self.position.rotate_and_store(qkv, bias, ctx.positions, None, nh, 0, hd, None, None)
-        out = torch.empty((T, self.q_width), dtype=x.dtype, device=x.device)
-        mfma = ops.prefill_attention_supported(hd, x.dtype)
-        plan = self._plan(ctx, x.dtype)
+        out = self.attend(qkv, ctx, cache)
+        return ops.linear(out, self.out_weight, self.out_bias, partial_ok=True, policy=policy)
+
+    def attend(self, q: torch.Tensor, ctx, cache: EntryCache) -> torch.Tensor:
+        """Attention of the step's rotated queries (the first ``num_heads * head_dim`` columns of
+        ``q``, one row a token) over the keys and values that ``cache`` holds, [T, heads * head_dim]:
+        the kernels and work items that the step's plan names, and nothing else of the layer."""
+        s = self.spec
+        nh, nkv, hd = s.num_heads, s.num_kv_heads, s.head_dim
+        T = q.shape[0]
+        out = torch.empty((T, self.q_width), dtype=q.dtype, device=q.device)
+        mfma = ops.prefill_attention_supported(hd, q.dtype)
+        plan = self._plan(ctx, q.dtype)
         common = dict(
-            q=qkv, q_stride=qkv.shape[1], out=out, k_cache=cache.k, v_cache=cache.v,
+            q=q, q_stride=q.shape[1], out=out, k_cache=cache.k, v_cache=cache.v,
             block_tables=ctx.block_tables[cache.group], ctx_lens=ctx.ctx_lens, cu_q=ctx.cu_q,
             nh=nh, nkv=nkv, hd=hd, block_size=cache.block_size, window=s.window or 0,
             scale=s.scale, n_tokens=T, n_requests=ctx.num_requests,
@@ -268,21 +277,21 @@ class PagedAttention(Part):
             workspace = None
             if plan.mfma_parts > 1:
                 need = ops.prefill_attention_workspace_floats(hd, plan.n_mfma, nh, nkv, plan.mfma_row_blocks)
-                workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+                workspace = torch.empty(need, dtype=torch.float32, device=q.device)
             ops.attention_prefill(items=plan.mfma_items, n_items=plan.n_mfma, row_blocks=plan.mfma_row_blocks,
                                   workspace=workspace, **common)
         elif plan.n_wide:
             workspace = None
             if plan.wide_splits > 1:
                 need = ops.attention_workspace_floats(hd, 64, plan.n_wide, nkv, -(-(nh // nkv) // plan.gh_wide), plan.wide_splits)
-                workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+                workspace = torch.empty(need, dtype=torch.float32, device=q.device)
             ops.attention(items=plan.wide_items, n_items=plan.n_wide, rows=64, gh=plan.gh_wide,
                           n_splits=plan.wide_splits, workspace=workspace, **common)
-        if plan.n_single and ops.decode_attention_supported(hd, x.dtype):
+        if plan.n_single and ops.decode_attention_supported(hd, q.dtype):
             workspace = None
             if plan.decode_splits > 1:
                 need = ops.decode_attention_workspace_floats(hd, plan.n_single, nh, nkv, plan.decode_splits)
-                workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+                workspace = torch.empty(need, dtype=torch.float32, device=q.device)
             ops.attention_decode(items=plan.single_items, n_items=plan.n_single, n_splits=plan.decode_splits,
                                  workspace=workspace, identity=plan.single_identity,
                                  split_keys=plan.decode_split_keys, max_ctx=plan.decode_max_ctx, **common)
@@ -290,7 +299,7 @@ class PagedAttention(Part):
             workspace = None
             if plan.single_splits > 1:
                 need = ops.attention_workspace_floats(hd, 16, plan.n_single, nkv, plan.chunks_single, plan.single_splits)
-                workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+                workspace = torch.empty(need, dtype=torch.float32, device=q.device)
             ops.attention(items=plan.single_items, n_items=plan.n_single, rows=16, gh=plan.gh_single,
                           n_splits=plan.single_splits, workspace=workspace, **common)
-        return ops.linear(out, self.out_weight, self.out_bias, partial_ok=True, policy=policy)
+        return out

@@ -1429,3 +1429,47 @@ def test_wide_tile_partial_sums_refuse_what_they_do_not_take():
     assert ops.linear(x, w, partial_ok=True, policy=policy).parts.shape == (4, 1024, 1536)
     assert isinstance(ops.linear(x[:512], w, partial_ok=True, policy=policy), torch.Tensor)   # too few rows
     assert isinstance(ops.linear(x, w, policy=policy), torch.Tensor)                           # a caller that wants a tensor
+
+
+def test_attention_part_alone_as_the_benchmark_times_it(monkeypatch):
+    """``bench.py --decode-attention-grid`` times ``PagedAttention.attend`` on a hand-made step of
+    single tokens: the same call must give dense attention over each request's own pages, and the
+    benchmark's record must hold a time for every point of its grid."""
+    import argparse
+
+    import bench
+    from clockwork_amd.engine.batch import StepContext
+    from clockwork_amd.parts.attention import PagedAttention
+    from clockwork_amd.parts.specs import AttentionSpec
+
+    nh, nkv, hd, bs = 12, 2, 128, 16
+    part = PagedAttention(AttentionSpec(hidden_size=nh * hd, num_heads=nh, num_kv_heads=nkv, head_dim=hd,
+                                        qkv_bias=False, out_bias=False, scale=hd ** -0.5))
+    part.dtype = torch.bfloat16
+    batch, context = 5, 700
+    pages_each = -(-context // bs)
+    gen = torch.Generator().manual_seed(11)
+    k = torch.randn((batch * pages_each, bs, nkv, hd), generator=gen).to(DEV, torch.bfloat16)
+    v = torch.randn((batch * pages_each, bs, nkv, hd), generator=gen).to(DEV, torch.bfloat16)
+    q = torch.randn((batch, nh * hd), generator=gen).to(DEV, torch.bfloat16)
+    tables = torch.randperm(batch * pages_each, generator=gen).view(batch, pages_each)
+    ctx = StepContext()
+    ctx.device, ctx.block_size = torch.device(DEV), bs
+    ctx.num_tokens = ctx.num_requests = batch
+    ctx.h_q_lens, ctx.h_ctx_lens = [1] * batch, [context] * batch
+    ctx.block_tables = [tables.to(DEV, torch.int32)]
+    ctx.ctx_lens = torch.full((batch,), context, dtype=torch.int32, device=DEV)
+    ctx.cu_q = torch.arange(batch + 1, dtype=torch.int32, device=DEV)
+    part.prepare(ctx)
+    out = part.attend(q, ctx, argparse.Namespace(k=k, v=v, group=0, block_size=bs)).float().cpu().view(batch, 1, nh, hd)
+    for r in range(batch):
+        keys = k[tables[r]].reshape(-1, nkv, hd)[:context].float().cpu()
+        values = v[tables[r]].reshape(-1, nkv, hd)[:context].float().cpu()
+        want = plain.attention_dense(q[r].view(1, nh, hd).float().cpu(), keys, values, hd ** -0.5)
+        torch.testing.assert_close(out[r], want, **tol(torch.bfloat16))
+
+    monkeypatch.setattr(bench, "REFERENCE_DECODE_ATTENTION_MS", {(2, 128): 0.07, (4, 512): 0.27})
+    record = bench.measure_decode_attention_grid()
+    assert set(record["grid"]) == {"batch2_ctx128", "batch4_ctx512"}
+    for point in record["grid"].values():
+        assert 0 < point["ms"] < 1 and point["key_splits"] >= 1 and point["GB_per_s"] > 0
