@@ -166,11 +166,13 @@ def _make_plan(ctx, nh: int, nkv: int, narrow_ok: bool) -> AttentionPlan:
         by_length = max(1, longest_single // 256)
         plan.single_splits = max(1, min(by_occupancy, by_length, 64))
         # decode kernel: a workgroup per (request, kv head, split); a split is at least 128 keys
-        # (one 32-key tile for each of its four waves), and about two workgroups per compute
-        # unit are enough to keep memory busy. More than 64 splits never paid: one request
+        # (one 32-key tile for each of its four waves). As many splits as still give every
+        # workgroup a compute unit of its own: one more and some units run a second round (24
+        # requests of 2100 keys on 2 kv heads, kernel and merge: 19.2 us with 4 splits, 22.4 with 6;
+        # 96 requests: 42.5 us with 1, 50.6 with 3). More than 64 splits never paid: one request
         # with 30000 keys takes 16 us with 64 to 128 splits and 19 us with 235.
         base = plan.n_single * nkv * -(-group // min(group, 16))
-        plan.decode_splits = max(1, min(-(-2 * ctx.num_compute_units // base), longest_single // 128, 64))
+        plan.decode_splits = max(1, min(ctx.num_compute_units // base, longest_single // 128, 64))
         # fixed places for the splits: a workgroup then knows its pages before it knows the
         # request's length, which saves it a trip to memory
         plan.decode_split_keys = 32 * -(-(-(-longest_single // plan.decode_splits)) // 32)

@@ -450,9 +450,10 @@ def test_decode_steps_of_eight_behind_2048_token_prompts(benchmark_steps, monkey
     assert (8, 2560) in captured and any(k[0] == "portion" and k[1] == 2048 for k in captured), captured
     if dtype == "bfloat16":
         cuts = [c for c in calls["decode"] if c[0] == 8]
-        # sixteen splits of 160 keys in the eager step, twenty of 128 in the graph (planned for its 2560-key bucket)
-        assert cuts and all(n_splits >= 16 and split_keys >= 128 and identity for _, n_splits, split_keys, identity in cuts), cuts
-        assert {c[1:3] for c in cuts} == {(16, 160), (20, 128)}, cuts
+        # sixteen splits (16 workgroups a split: one for every compute unit): of 160 keys in the
+        # eager step, which plans for its 2049 keys, and in the graph, planned for its 2560-key bucket
+        assert cuts and all(n_splits == 16 and split_keys == 160 and identity for _, n_splits, split_keys, identity in cuts), cuts
+        assert len(cuts) >= 2  # the eager step and the capture
     else:
         cuts = [c for c in calls["tile"] if c[0] == 8]
         assert cuts and all(n_splits > 1 for _, n_splits in cuts), cuts
@@ -485,7 +486,7 @@ def test_key_ranges_that_miss_keys_are_caught(benchmark_steps, monkeypatch):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_steps_of_sixty_four(benchmark_steps, monkeypatch, dtype):
     """The benchmark's wide batch: 64 requests that hold about 600 tokens decode side by side
-    (eager, captured, replayed twice), four splits a request in bfloat16."""
+    (eager, captured, replayed twice), two splits a request in bfloat16."""
     model_dir, _, many, want = benchmark_steps
     calls = _watch_attention(monkeypatch)
     runner = replay.make_runner(model_dir, dtype, 16, replay.pages_needed(many, 64, 16), max_model_len=4096)
