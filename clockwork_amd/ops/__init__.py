@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
+import gc
 import json
 import os
 import tempfile
@@ -417,7 +418,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias=None, out_dtype=None, par
             chosen = 0
             if splits > 1 and M <= SKINNY_MAX_ROWS:
                 # a tuning start-up has timed the split counts for this shape, or does so now
-                if policy.tuning and (N, K) not in policy.k_split_choices:
+                if policy.tuning and (N, K) not in policy.k_split_choices and policy.recall("k_split_choices", (N, K)) is None:
                     policy.k_split_choices[(N, K)] = _measure_k_splits(x, weight, splits)
                 chosen = policy.k_split_choices.get((N, K), 0)
                 splits = chosen or splits
@@ -465,7 +466,8 @@ class ProductPolicy:
     long K, into how many runs of K the wide-tile kernel sums it (0: the library's product stays).
     ``tuning``: such a start-up is under way (``library_tuning``)."""
 
-    __slots__ = ("hip_products", "swiglu_choices", "product_choices", "k_split_choices", "wide_partial_choices", "tuning")
+    __slots__ = ("hip_products", "swiglu_choices", "product_choices", "k_split_choices", "wide_partial_choices", "tuning",
+                 "_remembered")
 
     TABLES = ("swiglu_choices", "product_choices", "k_split_choices", "wide_partial_choices")
 
@@ -476,11 +478,14 @@ class ProductPolicy:
         self.k_split_choices: dict = {}
         self.wide_partial_choices: dict = {}
         self.tuning = False
+        self._remembered: dict = {name: {} for name in self.TABLES}
 
     def read_choices(self, path: str) -> int:
-        """Take over what an earlier start-up on this card and kernel build measured and left in
-        ``path`` (entries this policy already holds stay). A file that is missing, unreadable or
-        from another card or build is passed over. Returns the number of entries taken."""
+        """Remember what earlier start-ups on this card and kernel build measured and left in
+        ``path``: a shape's entry comes into use when this engine's own start-up asks for that
+        shape (``recall``), in place of measuring it again; other models' shapes stay aside. A file
+        that is missing, unreadable or from another card or build is passed over. Returns the number
+        of entries remembered."""
         try:
             with open(path) as f:
                 record = json.load(f)
@@ -488,22 +493,30 @@ class ProductPolicy:
                 return 0
             taken = 0
             for name in self.TABLES:
-                table = getattr(self, name)
                 for key, value in record.get(name, []):
-                    key = tuple(key)
-                    if key not in table:
-                        table[key] = value
-                        taken += 1
+                    self._remembered[name][tuple(key)] = value
+                    taken += 1
             return taken
         except (OSError, ValueError, TypeError, AttributeError):
             return 0
 
+    def recall(self, table: str, key):
+        """What an earlier start-up measured for ``key`` of ``table``, put into use; None if
+        nothing is remembered (or this policy holds a choice of its own already)."""
+        active = getattr(self, table)
+        if key in active or key not in self._remembered[table]:
+            return None
+        active[key] = self._remembered[table][key]
+        return active[key]
+
     def write_choices(self, path: str) -> None:
-        """Leave this policy's measured choices in ``path`` (written beside it and moved over it,
-        so a reader never sees half a file); where the folder cannot be written nothing is kept."""
+        """Leave what is remembered and this policy's own choices (which win) in ``path``, written
+        beside it and moved over it, so a reader never sees half a file; where the folder cannot be
+        written nothing is kept."""
         record = {"made_for": _choices_made_for()}
         for name in self.TABLES:
-            record[name] = [[list(key), value] for key, value in getattr(self, name).items()]
+            merged = {**self._remembered[name], **getattr(self, name)}
+            record[name] = [[list(key), value] for key, value in merged.items()]
         try:
             fd, tmp = tempfile.mkstemp(dir=os.path.dirname(path) or ".", prefix=".choices-")
             with os.fdopen(fd, "w") as f:
@@ -655,6 +668,8 @@ def _wide_product_chosen(x: torch.Tensor, weight: torch.Tensor, bias, policy: Pr
         return False
     key = (weight.shape[0], K, bias is not None)
     choice = policy.product_choices.get(key)
+    if choice is None and policy.tuning:
+        choice = policy.recall("product_choices", key)
     if choice is None and policy.tuning and x.is_contiguous():
         if _load("gemm_tile").cw_gemm_bf16_wide_tiles(0, M, key[0], K, K) >= WIDE_PRODUCT_MIN_TILES:
             library = _timed_us(lambda: _library_product(x, weight, bias))
@@ -682,6 +697,69 @@ def _timed_us(fn, repeats: int = 5) -> float:
         end.synchronize()
         times.append(begin.elapsed_time(end) * 1e3)
     return sorted(times)[len(times) // 2]
+
+
+def _replayed_us(candidates: dict, rounds: int, flush: bool, replays: int = 3) -> dict:
+    """The time of each of ``candidates`` (name -> a function of the round's number that launches
+    this package's own kernels only) as the kernels take it inside a captured graph of ``rounds``
+    rounds, replayed a few times. The operands have to come from memory as they do in a step:
+    either the candidate takes other copies of them from round to round, more than the caches
+    hold, or (``flush``) 512 MB are written before every round and what a graph of the writes
+    alone takes is subtracted. For kernels of a few microseconds, whose differences a timing of
+    eager launches blurs (the launches' own time lies on top and overlaps the kernels differently
+    from one candidate to the next: two counts of parts over K that differ by 5 us in the decode
+    step differed by 2 us timed that way)."""
+    wash = torch.empty(512 << 20, dtype=torch.uint8, device="cuda") if flush else None
+
+    def median_replay(fn) -> float:
+        def body():
+            for i in range(rounds):
+                if wash is not None:
+                    wash.zero_()
+                if fn is not None:
+                    fn(i)
+
+        body()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        was_enabled = gc.isenabled()
+        gc.disable()  # a collection must not destroy another graph while this capture is open
+        try:
+            with torch.cuda.graph(graph):
+                body()
+        finally:
+            if was_enabled:
+                gc.enable()
+        graph.replay()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(replays):
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record()
+            graph.replay()
+            end.record()
+            end.synchronize()
+            times.append(begin.elapsed_time(end) * 1e3)
+        del graph
+        return sorted(times)[len(times) // 2]
+
+    writes = median_replay(None) if flush else 0.0
+    return {name: (median_replay(fn) - writes) / rounds for name, fn in candidates.items()}
+
+
+# copies of a weight matrix that a timing walks through so that each comes from memory again:
+# together more than the memory-side cache holds
+_COLD_COPIES_BYTES = 320 << 20
+
+
+def _cold_copies(weight: torch.Tensor) -> list:
+    """``weight`` and as many copies of it as together exceed the caches (16 at most); the matrix
+    alone where the memory for them is not there."""
+    n = min(16, max(2, -(-_COLD_COPIES_BYTES // (weight.numel() * weight.element_size())) + 1))
+    try:
+        return [weight] + [weight.clone() for _ in range(n - 1)]
+    except torch.OutOfMemoryError:
+        return [weight]
 
 
 def linear_wide_partial(x: torch.Tensor, weight: torch.Tensor, k_splits: int) -> PartialSums:
@@ -718,6 +796,8 @@ def _wide_partial_chosen(x: torch.Tensor, weight: torch.Tensor, policy: ProductP
     key = (N, K)
     choice = policy.wide_partial_choices.get(key)
     if choice is None and policy.tuning:
+        choice = policy.recall("wide_partial_choices", key)
+    if choice is None and policy.tuning:
         lib = _load("gemm_tile")
         tiles = lib.cw_gemm_bf16_wide_tiles(0, M, N, K, K)
         choice = 0
@@ -740,8 +820,9 @@ def _measure_k_splits(x: torch.Tensor, weight: torch.Tensor, default: int) -> in
     """Into how many parts over K is the product of these few rows with ``weight`` [N, K] summed
     the fastest, together with the norm kernel that adds the parts up? Which count lets the
     streaming kernel in, fills the card evenly and leaves whole chunks to a wave differs from shape
-    to shape (the 7B shape's down product: 36.8 us with 5 parts, 30.9 with 7), so the candidates
-    are timed on the model's own weights, out of the caches."""
+    to shape (the 7B shape's down product with the norm: 38.4 us with 5 parts, 32.4 with 7; the 32B
+    shape's: 64.8 with 7, 59.2 with 6), so the candidates are timed on the model's own weights,
+    inside captured graphs that walk through copies of the matrix (each comes from memory again)."""
     M, K = x.shape
     N = weight.shape[0]
     lib = _load("gemm")
@@ -749,14 +830,19 @@ def _measure_k_splits(x: torch.Tensor, weight: torch.Tensor, default: int) -> in
     norm_weight = torch.ones(N, dtype=torch.bfloat16, device=x.device)
     out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
 
-    def run(splits: int):
+    weights = _cold_copies(weight)
+
+    def run(splits: int, round_no: int):
+        w = weights[round_no % len(weights)]
         parts = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
-        _check(lib.cw_gemm_bf16_skinny(3, _ptr(x), K, _ptr(weight), _ptr(parts), N, M, N, K, splits, _stream()),
+        _check(lib.cw_gemm_bf16_skinny(3, _ptr(x), K, _ptr(w), _ptr(parts), N, M, N, K, splits, _stream()),
                "gemm_bf16_skinny(partial)")
         add_rmsnorm(resid, PartialSums(parts), norm_weight, 1e-6, out, write_back=False)
 
     candidates = sorted({default, *(s for s in (2, 3, 4, 5, 6, 7, 8, 10, 12) if K // s >= 256)})
-    times = {splits: _timed_us(lambda: run(splits), repeats=7) for splits in candidates}
+    rounds = len(weights) * -(-12 // len(weights)) if len(weights) > 1 else 6
+    times = _replayed_us({splits: (lambda i, splits=splits: run(splits, i)) for splits in candidates},
+                         rounds=rounds, flush=len(weights) == 1)
     best = min(times, key=times.get)
     # the fixed rule stays unless something is clearly faster: no flapping between equals
     return best if times[best] < 0.97 * times[default] else default
@@ -859,7 +945,8 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor, policy: "ProductPolicy | None
             # with enough rows the shape of the weights decides, and a start-up that tunes the
             # library's products has measured it for this model's
             measured = M >= WIDE_SWIGLU_MIN_ROWS
-            if measured and policy.tuning and (two_i, K) not in policy.swiglu_choices:
+            if (measured and policy.tuning and (two_i, K) not in policy.swiglu_choices
+                    and policy.recall("swiglu_choices", (two_i, K)) is None):
                 policy.swiglu_choices[(two_i, K)] = _measure_swiglu(x, gate_up_weight, out)
             if not measured or policy.swiglu_choices.get((two_i, K), True):
                 return linear_tiled(x, gate_up_weight, swiglu=True, wide=True)

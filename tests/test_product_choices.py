@@ -16,12 +16,23 @@ def test_choices_written_and_read_back(tmp_path):
 
     later = ops.ProductPolicy()
     later.k_split_choices[(1536, 8960)] = 3          # what this process measured itself stays
-    assert later.read_choices(path) == 3
-    assert later.k_split_choices == {(1536, 8960): 3}
-    assert later.wide_partial_choices == {(1536, 8960): 4}
-    assert later.swiglu_choices == {(17920, 1536): False}
-    assert later.product_choices == {(3584, 1024, True): True}
-    assert not ops.DEFAULT_POLICY.k_split_choices
+    assert later.read_choices(path) == 4
+    # remembered, not in use: another model's shapes never show among this engine's choices
+    assert later.k_split_choices == {(1536, 8960): 3} and not later.wide_partial_choices and not later.swiglu_choices
+    assert later.recall("k_split_choices", (1536, 8960)) is None          # its own choice stands
+    assert later.recall("wide_partial_choices", (1536, 8960)) == 4
+    assert later.recall("wide_partial_choices", (1536, 8960)) is None     # in use now: nothing left to recall
+    assert later.recall("swiglu_choices", (17920, 1536)) is False
+    assert later.recall("swiglu_choices", (9, 9)) is None
+    assert later.wide_partial_choices == {(1536, 8960): 4} and later.swiglu_choices == {(17920, 1536): False}
+    assert not later.product_choices and not ops.DEFAULT_POLICY.k_split_choices
+    # what it leaves behind: everything remembered, its own choices on top
+    again = str(tmp_path / "again.json")
+    later.write_choices(again)
+    third = ops.ProductPolicy()
+    assert third.read_choices(again) == 4
+    assert third.recall("k_split_choices", (1536, 8960)) == 3
+    assert third.recall("product_choices", (3584, 1024, True)) is True
 
 
 def test_choices_of_another_build_or_a_broken_file_are_passed_over(tmp_path):
@@ -33,10 +44,11 @@ def test_choices_of_another_build_or_a_broken_file_are_passed_over(tmp_path):
     record = {"made_for": ["another card", "0.0", "gemm-0.so", "gemm_tile-0.so", "core-0.so"],
               "k_split_choices": [[[1536, 8960], 6]]}
     path.write_text(json.dumps(record))
-    assert policy.read_choices(str(path)) == 0 and not policy.k_split_choices
+    assert policy.read_choices(str(path)) == 0 and policy.recall("k_split_choices", (1536, 8960)) is None
     record["made_for"] = ops._choices_made_for()
     path.write_text(json.dumps(record))
-    assert policy.read_choices(str(path)) == 1 and policy.k_split_choices == {(1536, 8960): 6}
+    assert policy.read_choices(str(path)) == 1 and policy.recall("k_split_choices", (1536, 8960)) == 6
+    assert policy.k_split_choices == {(1536, 8960): 6}
     # a folder that cannot be written: nothing is kept, nothing is raised
     policy.write_choices(str(tmp_path / "missing" / "choices.json"))
 
