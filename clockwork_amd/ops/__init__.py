@@ -12,6 +12,7 @@ from __future__ import annotations
 import contextlib
 import ctypes
 import gc
+import hashlib
 import json
 import os
 import tempfile
@@ -528,15 +529,24 @@ class ProductPolicy:
 
 def choices_file() -> str:
     """Where a tuning start-up keeps what it measured for this package's own kernels: a file in
-    the temporary folder, one per user, or where CLOCKWORK_AMD_CHOICES_FILE points."""
-    return os.environ.get("CLOCKWORK_AMD_CHOICES_FILE") or os.path.join(
-        tempfile.gettempdir(), f"clockwork_amd_choices_{os.getuid()}.json")
+    the temporary folder, one per user and per card and kernel build (so that what one kind of
+    card measured is never handed to, or overwritten by, another), or where
+    CLOCKWORK_AMD_CHOICES_FILE points."""
+    named = os.environ.get("CLOCKWORK_AMD_CHOICES_FILE")
+    if named:
+        return named
+    mark = hashlib.sha256(json.dumps(_choices_made_for()).encode()).hexdigest()[:10]
+    return os.path.join(tempfile.gettempdir(), f"clockwork_amd_choices_{os.getuid()}_{mark}.json")
 
 
 def _choices_made_for() -> list:
-    """What measured choices hold for: the card and the builds of the kernels that were timed."""
-    card = torch.cuda.get_device_name() if torch.cuda.is_available() else "none"
-    return [card, torch.__version__] + [build.library_path(n).name for n in ("gemm", "gemm_tile", "core")]
+    """What measured choices hold for: the card (its architecture, compute units and memory: the
+    marketing name is empty under a profiler) and the builds of the kernels that were timed."""
+    card = ["none"]
+    if torch.cuda.is_available():
+        props = torch.cuda.get_device_properties(torch.cuda.current_device())
+        card = [str(getattr(props, "gcnArchName", props.name)), int(props.multi_processor_count), int(props.total_memory)]
+    return card + [torch.__version__] + [build.library_path(n).name for n in ("gemm", "gemm_tile", "core")]
 
 
 # what a call without an engine behind it runs by: the library for large products, nothing timed

@@ -41,7 +41,7 @@ def test_choices_of_another_build_or_a_broken_file_are_passed_over(tmp_path):
     assert policy.read_choices(str(path)) == 0                      # no file
     path.write_text("{ not json")
     assert policy.read_choices(str(path)) == 0
-    record = {"made_for": ["another card", "0.0", "gemm-0.so", "gemm_tile-0.so", "core-0.so"],
+    record = {"made_for": ["another card", 1, 2, "0.0", "gemm-0.so", "gemm_tile-0.so", "core-0.so"],
               "k_split_choices": [[[1536, 8960], 6]]}
     path.write_text(json.dumps(record))
     assert policy.read_choices(str(path)) == 0 and policy.recall("k_split_choices", (1536, 8960)) is None
@@ -58,3 +58,23 @@ def test_choices_file_follows_the_environment(monkeypatch, tmp_path):
     assert ops.choices_file() == str(tmp_path / "c.json")
     monkeypatch.delenv("CLOCKWORK_AMD_CHOICES_FILE")
     assert "clockwork_amd_choices_" in ops.choices_file()
+
+
+def test_the_card_is_known_by_more_than_its_name(monkeypatch):
+    """Under a profiler the card's marketing name comes back empty: what identifies it to the
+    choices file is its architecture, its compute units and its memory, and another card has
+    another file."""
+    import types
+
+    import torch
+
+    def card(arch, units):
+        return types.SimpleNamespace(name="", gcnArchName=arch, multi_processor_count=units, total_memory=1 << 38)
+
+    monkeypatch.setattr(torch.cuda, "is_available", lambda: True)
+    monkeypatch.setattr(torch.cuda, "current_device", lambda: 0)
+    monkeypatch.setattr(torch.cuda, "get_device_properties", lambda d: card("gfx950:sramecc+:xnack-", 256))
+    made_for, path = ops._choices_made_for(), ops.choices_file()
+    assert made_for[:3] == ["gfx950:sramecc+:xnack-", 256, 1 << 38]
+    monkeypatch.setattr(torch.cuda, "get_device_properties", lambda d: card("gfx950:sramecc+:xnack-", 128))
+    assert ops._choices_made_for() != made_for and ops.choices_file() != path
