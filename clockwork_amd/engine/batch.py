@@ -9,7 +9,7 @@ in a single copy; the kernels read device views of that buffer.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Optional, Sequence
+from typing import Sequence
 
 import numpy as np
 import torch

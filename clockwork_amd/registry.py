@@ -113,6 +113,10 @@ def register_arrangement(name: str, factory: Callable[..., Any]) -> None:
     _ARRANGEMENTS[name] = factory
 
 
+def unregister_arrangement(name: str) -> None:
+    _ARRANGEMENTS.pop(name, None)
+
+
 def build_arrangement(name: str, **parts) -> Any:
     factory = _ARRANGEMENTS.get(name)
     if factory is None:

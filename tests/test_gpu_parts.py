@@ -13,7 +13,8 @@ import torch
 
 from clockwork_amd.config.spec import LayerSpec, ModelSpec, PagedRowsSpec, ParamSpec, RunEntry, StateSpec, WeightTarget
 from clockwork_amd.parts.specs import AttentionSpec, RMSNormSpec, RopeNeoxSpec, SwiGLUSpec
-from clockwork_amd.registry import Architecture, build_part, register_architecture, register_part
+from clockwork_amd.registry import (Architecture, build_part, register_architecture, register_part,
+                                    unregister_architecture, unregister_arrangement, unregister_part)
 from tests import replay
 from tests.plain import qwen2_plain as plain
 
@@ -276,7 +277,11 @@ def toy_dir(tmp_path_factory):
     )
     config = {"architectures": ["ToyForCausalLM"], "vocab": 300, "hidden": 64, "window": 6, "eps": 1e-5,
               "kinds": ["full", "window", "again", "ema", "borrow", "routed"]}
-    return write_random_model(tmp_path_factory.mktemp("toy") / "toy", config, seed=3)
+    yield write_random_model(tmp_path_factory.mktemp("toy") / "toy", config, seed=3)
+    # what this file brought into the registries leaves with it
+    unregister_architecture(["ToyForCausalLM"])
+    for spec_type in (EmaMixerSpec, RoutedFFNSpec, SinePositionSpec):
+        unregister_part(spec_type)
 
 
 def _toy_plain_logits(model_dir, tokens, close_calls=None):
@@ -560,7 +565,11 @@ def toy2_dir(tmp_path_factory):
     )
     config = {"architectures": ["Toy2ForCausalLM"], "vocab": 211, "hidden": 64, "multiplier": 3.0, "cap": 0.4,
               "decay": 0.8, "eps": 1e-5}
-    return write_random_model(tmp_path_factory.mktemp("toy2") / "toy2", config, seed=8)
+    yield write_random_model(tmp_path_factory.mktemp("toy2") / "toy2", config, seed=8)
+    unregister_architecture(["Toy2ForCausalLM"])
+    unregister_arrangement("one_norm")
+    for spec_type in (ScaledEmbeddingSpec, CappedHeadSpec, DecayMixerSpec):
+        unregister_part(spec_type)
 
 
 def _toy2_plain_logits(model_dir, tokens):
@@ -798,7 +807,11 @@ def toy3_dir(tmp_path_factory):
     )
     config = {"architectures": ["Toy3ForCausalLM"], "vocab": 190, "hidden": 48, "latent": 24, "offset": 11, "begin": 0.5,
               "eps": 1e-5}
-    return write_random_model(tmp_path_factory.mktemp("toy3") / "toy3", config, seed=21)
+    yield write_random_model(tmp_path_factory.mktemp("toy3") / "toy3", config, seed=21)
+    unregister_architecture(["Toy3ForCausalLM"])
+    unregister_arrangement("renamed")
+    for spec_type in (OffsetEmbeddingSpec, LatentMixerSpec, WarmDecayMixerSpec):
+        unregister_part(spec_type)
 
 
 def _toy3_plain_logits(model_dir, tokens, offset=None):
