@@ -1473,3 +1473,42 @@ def test_attention_part_alone_as_the_benchmark_times_it(monkeypatch):
     assert set(record["grid"]) == {"batch2_ctx128", "batch4_ctx512"}
     for point in record["grid"].values():
         assert 0 < point["ms"] < 1 and point["key_splits"] >= 1 and point["GB_per_s"] > 0
+
+
+def test_candidates_are_timed_inside_graphs_over_copies_of_the_weights():
+    """What a tuning start-up ranks its own kernels' variants by: each candidate runs inside a
+    captured graph, round after round on another copy of the weights (together more than the
+    caches hold). Twice the work must take clearly longer, the same work about the same, and the
+    count of parts over K it chooses for a shape is one the kernel takes."""
+    from clockwork_amd import ops
+
+    N, K = 1536, 8960
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    w = (torch.randn(N, K, device=DEV, generator=gen) / K ** 0.5).to(torch.bfloat16)
+    x = torch.randn(8, K, device=DEV, generator=gen).to(torch.bfloat16)
+    copies = ops._cold_copies(w)
+    assert 2 <= len(copies) <= 16 and copies[0] is w
+    assert sum(c.numel() * 2 for c in copies) > 256 << 20
+    assert all(torch.equal(c, w) for c in copies[1:3])
+
+    def once(i):
+        ops.linear(x, copies[i % len(copies)])
+
+    def twice(i):
+        ops.linear(x, copies[(2 * i) % len(copies)])
+        ops.linear(x, copies[(2 * i + 1) % len(copies)])
+
+    times = ops._replayed_us({"once": once, "again": once, "twice": twice}, rounds=len(copies), flush=False)
+    assert 2 < times["once"] < 60, times
+    assert abs(times["again"] - times["once"]) < 0.2 * times["once"], times
+    assert times["twice"] > 1.5 * times["once"], times
+    # with the caches washed between the rounds instead (no memory for copies): the same ranking
+    washed = ops._replayed_us({"once": lambda i: ops.linear(x, w), "twice": lambda i: (ops.linear(x, w), ops.linear(x, w))},
+                              rounds=4, flush=True)
+    assert washed["twice"] > 1.4 * washed["once"] > 0, washed
+    chosen = ops._measure_k_splits(x, w, ops._load("gemm").cw_gemm_bf16_skinny_ksplits(8, N, K))
+    policy = ops.ProductPolicy()
+    policy.k_split_choices[(N, K)] = chosen
+    got = ops.linear(x, w, partial_ok=True, policy=policy)
+    assert got.parts.shape[0] == chosen
+    torch.testing.assert_close(got.sum(), x.float() @ w.float().t(), rtol=2e-2, atol=2e-2)
